@@ -1,0 +1,176 @@
+"""Builds the native libraries in-tree and loads them with ctypes.
+
+Two kinds of library live under ``mini_llm_amd/_lib``:
+
+* ``runtime``: the host-only C++ runtime (cache manager, scheduler), built with g++;
+* one library per kernel source under ``csrc/kernels`` built with hipcc for gfx950.
+  A kernel library is built the first time one of its ops is called, so a model only
+  compiles what it needs.
+
+A library is rebuilt when the hash of its sources differs from the one recorded
+beside it, so a stale binary is never loaded.
+"""
+from __future__ import annotations
+
+import ctypes
+import hashlib
+import os
+import shutil
+import subprocess
+import sys
+import tempfile
+import threading
+import time
+from typing import Dict, List, Optional
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+CSRC = os.path.join(_HERE, "csrc")
+LIB_DIR = os.path.join(_HERE, "_lib")
+
+GPU_ARCH = "gfx950"
+HIPCC_FLAGS = [
+    "-O3", "-std=c++17", "-fPIC", "-shared", f"--offload-arch={GPU_ARCH}",
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-Wno-unused-command-line-argument", "-Wno-unknown-warning-option",
+]
+CXX_FLAGS = ["-O2", "-std=c++17", "-fPIC", "-shared", "-Wall"]
+
+# library name -> (compiler kind, sources relative to csrc, headers that also enter the hash)
+LIBRARIES: Dict[str, dict] = {
+    "runtime": {
+        "kind": "cxx",
+        "sources": ["runtime/cache_manager.cc", "runtime/scheduler.cc", "runtime/c_api.cc"],
+        "headers": ["runtime/cache_manager.h", "runtime/scheduler.h"],
+    },
+    "elementwise": {"kind": "hip", "sources": ["kernels/elementwise.hip"], "headers": ["kernels/common.h"]},
+    "gemm_f32": {"kind": "hip", "sources": ["kernels/gemm_f32.hip"], "headers": ["kernels/common.h"]},
+    "gemm_bf16": {"kind": "hip", "sources": ["kernels/gemm_bf16.hip"], "headers": ["kernels/common.h"]},
+    "attention": {"kind": "hip", "sources": ["kernels/attention.hip"], "headers": ["kernels/common.h"]},
+    "sampling": {"kind": "hip", "sources": ["kernels/sampling.hip"], "headers": ["kernels/common.h"]},
+}
+
+_loaded: Dict[str, ctypes.CDLL] = {}
+_lock = threading.Lock()
+
+
+class BuildError(RuntimeError):
+    pass
+
+
+def _say(msg: str) -> None:
+    print(f"[mini_llm_amd build] {msg}", file=sys.stderr, flush=True)
+
+
+def _paths(name: str):
+    spec = LIBRARIES[name]
+    srcs = [os.path.join(CSRC, s) for s in spec["sources"]]
+    hdrs = [os.path.join(CSRC, h) for h in spec.get("headers", [])]
+    return spec, srcs, hdrs
+
+
+def _source_hash(name: str) -> str:
+    spec, srcs, hdrs = _paths(name)
+    h = hashlib.sha256()
+    flags = HIPCC_FLAGS if spec["kind"] == "hip" else CXX_FLAGS
+    h.update(" ".join(flags).encode())
+    for p in srcs + hdrs:
+        with open(p, "rb") as f:
+            h.update(p[len(CSRC):].encode())
+            h.update(f.read())
+    return h.hexdigest()
+
+
+def lib_path(name: str) -> str:
+    return os.path.join(LIB_DIR, f"libmllm_{name}.so")
+
+
+def is_current(name: str) -> bool:
+    so, stamp = lib_path(name), lib_path(name) + ".hash"
+    if not (os.path.isfile(so) and os.path.isfile(stamp)):
+        return False
+    with open(stamp) as f:
+        return f.read().strip() == _source_hash(name)
+
+
+def _find(tool: str, extra: List[str]) -> str:
+    p = shutil.which(tool)
+    if p:
+        return p
+    for d in extra:
+        c = os.path.join(d, tool)
+        if os.path.isfile(c):
+            return c
+    raise BuildError(f"'{tool}' not found on PATH or in {extra}")
+
+
+def build_library(name: str, verbose: bool = True) -> str:
+    """Compiles one library unconditionally and returns its path."""
+    spec, srcs, _ = _paths(name)
+    os.makedirs(LIB_DIR, exist_ok=True)
+    so = lib_path(name)
+    if spec["kind"] == "hip":
+        cc = _find("hipcc", ["/opt/rocm/bin"])
+        cmd = [cc] + HIPCC_FLAGS
+    else:
+        cc = _find("g++", ["/usr/bin"])
+        cmd = [cc] + CXX_FLAGS
+    # Compile to a private name, then rename: a concurrent process never sees a half-written file.
+    fd, tmp = tempfile.mkstemp(prefix=f".{name}.", suffix=".so", dir=LIB_DIR)
+    os.close(fd)
+    cmd = cmd + [f"-I{os.path.join(CSRC, 'kernels')}", f"-I{os.path.join(CSRC, 'runtime')}"] + srcs + ["-o", tmp]
+    env = dict(os.environ)
+    env.setdefault("TMPDIR", tempfile.gettempdir())
+    if not env.get("HOME") or not os.access(env["HOME"], os.W_OK):
+        env["HOME"] = tempfile.gettempdir()
+    if verbose:
+        _say(f"compiling {name} ({', '.join(spec['sources'])}) ...")
+    t0 = time.time()
+    proc = subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, env=env, text=True)
+    out_lines: List[str] = []
+
+    def _drain():
+        for line in proc.stdout:
+            out_lines.append(line)
+
+    th = threading.Thread(target=_drain, daemon=True)
+    th.start()
+    while proc.poll() is None:
+        th.join(timeout=15)
+        if proc.poll() is None and verbose:
+            _say(f"  ... still compiling {name} ({time.time() - t0:.0f} s)")
+    th.join()
+    if proc.returncode != 0:
+        try:
+            os.unlink(tmp)
+        except OSError:
+            pass
+        raise BuildError(f"building {name} failed:\n{' '.join(cmd)}\n{''.join(out_lines)}")
+    os.replace(tmp, so)
+    os.chmod(so, 0o755)
+    with open(so + ".hash", "w") as f:
+        f.write(_source_hash(name))
+    if verbose:
+        _say(f"built {name} in {time.time() - t0:.1f} s")
+    return so
+
+
+def build_all(verbose: bool = True, jobs: int = 4) -> None:
+    """Compiles every library, whatever is there already."""
+    from concurrent.futures import ThreadPoolExecutor
+    with ThreadPoolExecutor(max_workers=jobs) as ex:
+        list(ex.map(lambda n: build_library(n, verbose), LIBRARIES))
+    with _lock:
+        _loaded.clear()
+
+
+def load_library(name: str) -> ctypes.CDLL:
+    """Loads a library, building it first if it is missing or out of date."""
+    with _lock:
+        lib = _loaded.get(name)
+        if lib is not None:
+            return lib
+        if not is_current(name):
+            build_library(name)
+        lib = ctypes.CDLL(lib_path(name))
+        _loaded[name] = lib
+        return lib

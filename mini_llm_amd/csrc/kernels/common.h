@@ -1,0 +1,133 @@
+// Shared device helpers for the gfx950 kernels: bf16 conversion, wave/block
+// reductions for 64-wide wavefronts, activation functions and the GEMM epilogue.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#define MLLM_WAVE 64
+
+// dtype codes of the C ABI
+#define MLLM_F32 0
+#define MLLM_BF16 1
+
+// GEMM epilogues
+#define EPI_STORE 0         // out[m,n] = acc + bias            (activation dtype)
+#define EPI_GELU_TANH 1     // out[m,n] = gelu_tanh(acc + bias) (activation dtype)
+#define EPI_GELU_ERF 2      // out[m,n] = gelu_erf(acc + bias)  (activation dtype)
+#define EPI_ADD_RESIDUAL 3  // res[m,n] += acc + bias           (fp32, in place)
+#define EPI_STORE_F32 4     // out[m,n] = acc + bias            (fp32)
+
+struct bf16_t {
+    uint16_t bits;
+};
+
+__device__ __forceinline__ float bf16_to_float(bf16_t v) {
+    return __uint_as_float(static_cast<uint32_t>(v.bits) << 16);
+}
+
+// Round to nearest, ties to even; NaN stays NaN.
+__device__ __forceinline__ bf16_t float_to_bf16(float f) {
+    uint32_t u = __float_as_uint(f);
+    bf16_t r;
+    if ((u & 0x7fffffffu) > 0x7f800000u) {
+        r.bits = static_cast<uint16_t>((u >> 16) | 0x0040u);
+    } else {
+        u += 0x7fffu + ((u >> 16) & 1u);
+        r.bits = static_cast<uint16_t>(u >> 16);
+    }
+    return r;
+}
+
+__device__ __forceinline__ float to_float(float v) { return v; }
+__device__ __forceinline__ float to_float(bf16_t v) { return bf16_to_float(v); }
+
+template <typename T> __device__ __forceinline__ T from_float(float v);
+template <> __device__ __forceinline__ float from_float<float>(float v) { return v; }
+template <> __device__ __forceinline__ bf16_t from_float<bf16_t>(float v) { return float_to_bf16(v); }
+
+// Loads 8 consecutive elements as floats; the address must be 16-byte aligned.
+__device__ __forceinline__ void load8(const float* p, float (&v)[8]) {
+    float4 a = *reinterpret_cast<const float4*>(p);
+    float4 b = *reinterpret_cast<const float4*>(p + 4);
+    v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w;
+    v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
+}
+__device__ __forceinline__ void load8(const bf16_t* p, float (&v)[8]) {
+    uint4 a = *reinterpret_cast<const uint4*>(p);
+    v[0] = __uint_as_float(a.x << 16); v[1] = __uint_as_float(a.x & 0xffff0000u);
+    v[2] = __uint_as_float(a.y << 16); v[3] = __uint_as_float(a.y & 0xffff0000u);
+    v[4] = __uint_as_float(a.z << 16); v[5] = __uint_as_float(a.z & 0xffff0000u);
+    v[6] = __uint_as_float(a.w << 16); v[7] = __uint_as_float(a.w & 0xffff0000u);
+}
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+    for (int off = MLLM_WAVE / 2; off > 0; off >>= 1) v += __shfl_xor(v, off, MLLM_WAVE);
+    return v;
+}
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+    for (int off = MLLM_WAVE / 2; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, MLLM_WAVE));
+    return v;
+}
+
+// Orders LDS traffic between the lanes of ONE wavefront (which run in lockstep):
+// what lanes wrote before it is visible to all lanes after it.
+__device__ __forceinline__ void wave_lds_sync() {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
+// Block-wide sum for blocks of up to 1024 threads; `scratch` holds >= 16 floats of LDS.
+// Every thread gets the result. Safe to call repeatedly with the same scratch.
+__device__ __forceinline__ float block_sum(float v, float* scratch) {
+    v = wave_sum(v);
+    const int wave = threadIdx.x / MLLM_WAVE, lane = threadIdx.x % MLLM_WAVE;
+    const int n_waves = (blockDim.x + MLLM_WAVE - 1) / MLLM_WAVE;
+    __syncthreads();
+    if (lane == 0) scratch[wave] = v;
+    __syncthreads();
+    float t = 0.f;
+    for (int w = 0; w < n_waves; ++w) t += scratch[w];
+    return t;
+}
+__device__ __forceinline__ float block_max(float v, float* scratch) {
+    v = wave_max(v);
+    const int wave = threadIdx.x / MLLM_WAVE, lane = threadIdx.x % MLLM_WAVE;
+    const int n_waves = (blockDim.x + MLLM_WAVE - 1) / MLLM_WAVE;
+    __syncthreads();
+    if (lane == 0) scratch[wave] = v;
+    __syncthreads();
+    float t = scratch[0];
+    for (int w = 1; w < n_waves; ++w) t = fmaxf(t, scratch[w]);
+    return t;
+}
+
+// GELU, tanh form: /root/reference/src/kernels/gelu.cu:7-9.
+__device__ __forceinline__ float gelu_tanh(float v) {
+    return 0.5f * v * (1.f + tanhf(0.7978845608f * (v + 0.044715f * v * v * v)));
+}
+// GELU, exact form 0.5 v (1 + erf(v / sqrt 2)); the reference has only the tanh form.
+__device__ __forceinline__ float gelu_erf(float v) {
+    return 0.5f * v * (1.f + erff(v * 0.70710678118654752440f));
+}
+
+template <typename OutT>
+__device__ __forceinline__ void epilogue(int mode, float acc, float bias, void* out, size_t idx) {
+    float v = acc + bias;
+    switch (mode) {
+        case EPI_STORE: reinterpret_cast<OutT*>(out)[idx] = from_float<OutT>(v); break;
+        case EPI_GELU_TANH: reinterpret_cast<OutT*>(out)[idx] = from_float<OutT>(gelu_tanh(v)); break;
+        case EPI_GELU_ERF: reinterpret_cast<OutT*>(out)[idx] = from_float<OutT>(gelu_erf(v)); break;
+        case EPI_ADD_RESIDUAL: reinterpret_cast<float*>(out)[idx] += v; break;
+        default: reinterpret_cast<float*>(out)[idx] = v; break;
+    }
+}
+
+#define MLLM_LAUNCH_CHECK()                                   \
+    do {                                                      \
+        hipError_t e_ = hipGetLastError();                    \
+        if (e_ != hipSuccess) return static_cast<int>(e_);    \
+    } while (0)

@@ -1,0 +1,115 @@
+// Embedding, LayerNorm and key/value page writes for gfx950.
+#include "common.h"
+
+// ---------------------------------------------------------------------------
+// Token + position embedding: x[t,:] = wte[ids[t],:] + wpe[pos[t],:]   (fp32 out)
+// /root/reference/src/kernels/embedding.cu:23-43. wpe may be null (no learned positions).
+// ---------------------------------------------------------------------------
+template <typename T>
+__global__ void embed_kernel(const int* __restrict__ ids, const int* __restrict__ pos,
+                             const T* __restrict__ wte, const T* __restrict__ wpe,
+                             float* __restrict__ x, int D) {
+    const int t = blockIdx.x;
+    const T* te = wte + static_cast<size_t>(ids[t]) * D;
+    float* xr = x + static_cast<size_t>(t) * D;
+    if (wpe != nullptr) {
+        const T* pe = wpe + static_cast<size_t>(pos[t]) * D;
+        for (int d = threadIdx.x; d < D; d += blockDim.x) xr[d] = to_float(te[d]) + to_float(pe[d]);
+    } else {
+        for (int d = threadIdx.x; d < D; d += blockDim.x) xr[d] = to_float(te[d]);
+    }
+}
+
+// ---------------------------------------------------------------------------
+// LayerNorm over the last dimension, statistics in fp32, two passes:
+// mean, then biased variance of (x - mean); y = (x - mean) * rsqrt(var + eps) * g + b.
+// /root/reference/src/kernels/layernorm.cu:32-49. `rows` (optional) selects input rows.
+// ---------------------------------------------------------------------------
+template <typename OutT>
+__global__ void layernorm_kernel(const float* __restrict__ x, const int* __restrict__ rows,
+                                 const float* __restrict__ gamma, const float* __restrict__ beta,
+                                 OutT* __restrict__ y, int D, float eps) {
+    __shared__ float scratch[16];
+    const int r = blockIdx.x;
+    const int src = rows ? rows[r] : r;
+    const float* xr = x + static_cast<size_t>(src) * D;
+    OutT* yr = y + static_cast<size_t>(r) * D;
+    float s = 0.f;
+    for (int d = threadIdx.x; d < D; d += blockDim.x) s += xr[d];
+    const float mean = block_sum(s, scratch) / static_cast<float>(D);
+    float q = 0.f;
+    for (int d = threadIdx.x; d < D; d += blockDim.x) {
+        float c = xr[d] - mean;
+        q += c * c;
+    }
+    const float var = block_sum(q, scratch) / static_cast<float>(D);
+    const float inv = 1.0f / sqrtf(var + eps);
+    for (int d = threadIdx.x; d < D; d += blockDim.x) {
+        float v = (xr[d] - mean) * inv * gamma[d];
+        if (beta) v += beta[d];
+        yr[d] = from_float<OutT>(v);
+    }
+}
+
+// ---------------------------------------------------------------------------
+// Key/value write: copies the key and value columns of each token's row into the
+// row `slots[t]` of the page pools (slot = page * page_size + offset; < 0: skip).
+// /root/reference/src/kernels/prefill/append_kv.cu:28-46.
+// ---------------------------------------------------------------------------
+template <typename T>
+__global__ void kv_append_kernel(const T* __restrict__ src, int src_stride, int k_col, int v_col,
+                                 T* __restrict__ k_pages, T* __restrict__ v_pages, int kv_dim,
+                                 const int* __restrict__ slots) {
+    const int t = blockIdx.x;
+    const int slot = slots[t];
+    if (slot < 0) return;
+    const T* ks = src + static_cast<size_t>(t) * src_stride + k_col;
+    const T* vs = src + static_cast<size_t>(t) * src_stride + v_col;
+    T* kd = k_pages + static_cast<size_t>(slot) * kv_dim;
+    T* vd = v_pages + static_cast<size_t>(slot) * kv_dim;
+    for (int d = threadIdx.x; d < kv_dim; d += blockDim.x) {
+        kd[d] = ks[d];
+        vd[d] = vs[d];
+    }
+}
+
+extern "C" {
+
+int mllm_embed(const int* ids, const int* pos, const void* wte, const void* wpe, float* x, int T, int D,
+               int dtype, hipStream_t stream) {
+    if (T <= 0) return 0;
+    if (dtype == MLLM_F32)
+        embed_kernel<float><<<T, 256, 0, stream>>>(ids, pos, (const float*)wte, (const float*)wpe, x, D);
+    else
+        embed_kernel<bf16_t><<<T, 256, 0, stream>>>(ids, pos, (const bf16_t*)wte, (const bf16_t*)wpe, x, D);
+    MLLM_LAUNCH_CHECK();
+    return 0;
+}
+
+int mllm_layernorm(const float* x, const int* rows, const float* gamma, const float* beta, void* y, int n,
+                   int D, float eps, int out_dtype, hipStream_t stream) {
+    if (n <= 0) return 0;
+    const int threads = D >= 1024 ? 512 : 256;
+    if (out_dtype == MLLM_F32)
+        layernorm_kernel<float><<<n, threads, 0, stream>>>(x, rows, gamma, beta, (float*)y, D, eps);
+    else
+        layernorm_kernel<bf16_t><<<n, threads, 0, stream>>>(x, rows, gamma, beta, (bf16_t*)y, D, eps);
+    MLLM_LAUNCH_CHECK();
+    return 0;
+}
+
+int mllm_kv_append(const void* src, int src_stride, int k_col, int v_col, void* k_pages, void* v_pages,
+                   int kv_dim, const int* slots, int T, int dtype, hipStream_t stream) {
+    if (T <= 0) return 0;
+    const int threads = kv_dim >= 512 ? 256 : 64;
+    if (dtype == MLLM_F32)
+        kv_append_kernel<float><<<T, threads, 0, stream>>>((const float*)src, src_stride, k_col, v_col,
+                                                            (float*)k_pages, (float*)v_pages, kv_dim, slots);
+    else
+        kv_append_kernel<bf16_t><<<T, threads, 0, stream>>>((const bf16_t*)src, src_stride, k_col, v_col,
+                                                             (bf16_t*)k_pages, (bf16_t*)v_pages, kv_dim, slots);
+    MLLM_LAUNCH_CHECK();
+    return 0;
+}
+
+}  // extern "C"

@@ -1,0 +1,95 @@
+// True fp32 matrix product for the 32-bit path: C[M,N] = A[M,K] * W[N,K]^T (+ bias, epilogue).
+// Plain FMA in fp32, every output accumulated over k in ascending order, so a row's
+// result does not depend on which other rows share the launch. No reduced-precision
+// matrix mode is involved. Any M, N, K.
+//
+// Same contract as the reference's bounds-safe kernel
+// (/root/reference/src/kernels/gemm.cu:238-392: alpha*acc + beta*old + bias, optional GELU),
+// with the weight held as [N,K] (k contiguous) instead of [K,N].
+#include "common.h"
+
+#define F32_BM 64
+#define F32_BN 64
+#define F32_BK 16
+
+__global__ void __launch_bounds__(256)
+gemm_f32_kernel(const float* __restrict__ A, int lda, const float* __restrict__ W, int ldw,
+                const float* __restrict__ bias, void* __restrict__ C, int ldc, int M, int N, int K, int mode) {
+    __shared__ float As[F32_BK][F32_BM + 4];
+    __shared__ float Ws[F32_BK][F32_BN + 4];
+    const int tid = threadIdx.x;
+    const int tx = tid % 16, ty = tid / 16;
+    const int m0 = blockIdx.y * F32_BM, n0 = blockIdx.x * F32_BN;
+    // loader mapping: 64 rows x 4 k-quads
+    const int lrow = tid / 4, lk = (tid % 4) * 4;
+    const bool vec_a = (lda % 4 == 0) && ((reinterpret_cast<uintptr_t>(A) & 15) == 0);
+    const bool vec_w = (ldw % 4 == 0) && ((reinterpret_cast<uintptr_t>(W) & 15) == 0);
+
+    float acc[4][4] = {};
+    for (int k0 = 0; k0 < K; k0 += F32_BK) {
+        float av[4] = {0.f, 0.f, 0.f, 0.f}, wv[4] = {0.f, 0.f, 0.f, 0.f};
+        const int kk = k0 + lk;
+        const int am = m0 + lrow, wn = n0 + lrow;
+        if (am < M) {
+            const float* p = A + static_cast<size_t>(am) * lda + kk;
+            if (vec_a && kk + 3 < K) {
+                float4 v = *reinterpret_cast<const float4*>(p);
+                av[0] = v.x; av[1] = v.y; av[2] = v.z; av[3] = v.w;
+            } else {
+                for (int i = 0; i < 4; ++i) if (kk + i < K) av[i] = p[i];
+            }
+        }
+        if (wn < N) {
+            const float* p = W + static_cast<size_t>(wn) * ldw + kk;
+            if (vec_w && kk + 3 < K) {
+                float4 v = *reinterpret_cast<const float4*>(p);
+                wv[0] = v.x; wv[1] = v.y; wv[2] = v.z; wv[3] = v.w;
+            } else {
+                for (int i = 0; i < 4; ++i) if (kk + i < K) wv[i] = p[i];
+            }
+        }
+        __syncthreads();   // the previous tile's readers are done
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            As[lk + i][lrow] = av[i];
+            Ws[lk + i][lrow] = wv[i];
+        }
+        __syncthreads();
+#pragma unroll
+        for (int k = 0; k < F32_BK; ++k) {
+            float a[4], b[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) a[i] = As[k][ty * 4 + i];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) b[j] = Ws[k][tx * 4 + j];
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) acc[i][j] = fmaf(a[i], b[j], acc[i][j]);
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int m = m0 + ty * 4 + i;
+        if (m >= M) continue;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int n = n0 + tx * 4 + j;
+            if (n >= N) continue;
+            epilogue<float>(mode, acc[i][j], bias ? bias[n] : 0.f, C, static_cast<size_t>(m) * ldc + n);
+        }
+    }
+}
+
+extern "C" {
+
+int mllm_gemm_f32(const float* A, int lda, const float* W, int ldw, const float* bias, void* C, int ldc,
+                  int M, int N, int K, int mode, hipStream_t stream) {
+    if (M <= 0 || N <= 0) return 0;
+    dim3 grid((N + F32_BN - 1) / F32_BN, (M + F32_BM - 1) / F32_BM);
+    gemm_f32_kernel<<<grid, 256, 0, stream>>>(A, lda, W, ldw, bias, C, ldc, M, N, K, mode);
+    MLLM_LAUNCH_CHECK();
+    return 0;
+}
+
+}  // extern "C"

@@ -1,0 +1,252 @@
+"""The engine's device operations: thin, checked wrappers over the HIP kernels.
+
+Every op takes torch tensors that live on the GPU, checks on the host that shapes,
+strides and dtypes match what the kernel and its grid assume, and launches on the
+current HIP stream (so the calls can be captured in a HIP graph). There is no CPU
+path: a tensor that is not on the GPU, or a kernel library that cannot be built and
+loaded, raises.
+
+Parts look ops up as ``ops.<name>`` at call time.
+"""
+from __future__ import annotations
+
+import ctypes
+from typing import Optional
+
+import torch
+
+from ..build import load_library
+
+EPILOGUES = {"store": 0, "gelu_tanh": 1, "gelu_erf": 2, "add_residual": 3, "store_f32": 4}
+_DT = {torch.float32: 0, torch.bfloat16: 1}
+
+
+class KernelError(RuntimeError):
+    pass
+
+
+def _dt(t: torch.Tensor) -> int:
+    if t.dtype not in _DT:
+        raise KernelError(f"unsupported dtype {t.dtype} (float32 or bfloat16)")
+    return _DT[t.dtype]
+
+
+def _gpu(*tensors: Optional[torch.Tensor]) -> None:
+    for t in tensors:
+        if t is not None and not t.is_cuda:
+            raise KernelError(
+                "tensor is not on the GPU: the engine has no CPU path "
+                f"(device={t.device}, shape={tuple(t.shape)})")
+
+
+def _stream() -> ctypes.c_void_p:
+    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _p(t: Optional[torch.Tensor]) -> ctypes.c_void_p:
+    return ctypes.c_void_p(0 if t is None else t.data_ptr())
+
+
+def _check(rc: int, what: str) -> None:
+    if rc == 0:
+        return
+    if rc < 0:
+        raise KernelError(f"{what}: the kernel refuses these sizes (code {rc})")
+    raise KernelError(f"{what}: HIP error {rc} at launch")
+
+
+def _rows2d(t: torch.Tensor, name: str) -> None:
+    if t.dim() != 2 or t.stride(1) != 1:
+        raise KernelError(f"{name} must be 2-D with a contiguous last dimension, got shape "
+                          f"{tuple(t.shape)} strides {t.stride()}")
+
+
+def _i32(t: torch.Tensor, name: str, n: Optional[int] = None) -> None:
+    if t.dtype != torch.int32 or not t.is_contiguous():
+        raise KernelError(f"{name} must be a contiguous int32 tensor")
+    if n is not None and t.numel() < n:
+        raise KernelError(f"{name} has {t.numel()} entries, {n} needed")
+
+
+# ---------------------------------------------------------------------------------
+
+def embed(ids: torch.Tensor, positions: Optional[torch.Tensor], wte: torch.Tensor,
+          wpe: Optional[torch.Tensor], out: torch.Tensor) -> torch.Tensor:
+    """out[t,:] = wte[ids[t],:] + wpe[positions[t],:] in fp32. ids/positions must be in range
+    (the caller checks them on the host)."""
+    _gpu(ids, positions, wte, wpe, out)
+    T = ids.numel()
+    _rows2d(wte, "wte")
+    D = wte.shape[1]
+    _i32(ids, "ids")
+    if not wte.is_contiguous():
+        raise KernelError("wte must be contiguous")
+    if wpe is not None:
+        if positions is None:
+            raise KernelError("positions are needed with a position table")
+        _i32(positions, "positions", T)
+        if wpe.dtype != wte.dtype or wpe.dim() != 2 or wpe.shape[1] != D or not wpe.is_contiguous():
+            raise KernelError("wpe must be contiguous [P, D] in wte's dtype")
+    if out.dtype != torch.float32 or out.shape != (T, D) or not out.is_contiguous():
+        raise KernelError(f"out must be contiguous fp32 [{T}, {D}]")
+    lib = load_library("elementwise")
+    _check(lib.mllm_embed(_p(ids), _p(positions if wpe is not None else None), _p(wte), _p(wpe), _p(out),
+                          T, D, _dt(wte), _stream()), "embed")
+    return out
+
+
+def layernorm(x: torch.Tensor, gamma: torch.Tensor, beta: Optional[torch.Tensor], eps: float,
+              out: torch.Tensor, rows: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """out[i,:] = LayerNorm(x[rows[i] if rows else i,:]); statistics in fp32."""
+    _gpu(x, gamma, beta, out, rows)
+    if x.dtype != torch.float32 or x.dim() != 2 or not x.is_contiguous():
+        raise KernelError("layernorm input must be contiguous fp32 [rows, D]")
+    D = x.shape[1]
+    n = rows.numel() if rows is not None else x.shape[0]
+    if rows is not None:
+        _i32(rows, "rows")
+    if gamma.dtype != torch.float32 or gamma.numel() != D or not gamma.is_contiguous():
+        raise KernelError(f"gamma must be fp32 [{D}]")
+    if beta is not None and (beta.dtype != torch.float32 or beta.numel() != D or not beta.is_contiguous()):
+        raise KernelError(f"beta must be fp32 [{D}]")
+    if out.shape != (n, D) or not out.is_contiguous():
+        raise KernelError(f"out must be contiguous [{n}, {D}]")
+    lib = load_library("elementwise")
+    _check(lib.mllm_layernorm(_p(x), _p(rows), _p(gamma), _p(beta), _p(out), n, D, ctypes.c_float(eps),
+                              _dt(out), _stream()), "layernorm")
+    return out
+
+
+def linear(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], out: torch.Tensor,
+           epilogue: str = "store") -> torch.Tensor:
+    """out = epilogue(a @ w.T + bias). a: [M,K], w: [N,K] (same dtype), bias: fp32 [N].
+
+    epilogue: "store" | "gelu_tanh" | "gelu_erf" (out in a's dtype), "add_residual"
+    (out fp32, accumulated in place), "store_f32" (out fp32).
+    """
+    _gpu(a, w, bias, out)
+    _rows2d(a, "a")
+    _rows2d(w, "w")
+    _rows2d(out, "out")
+    M, K = a.shape
+    N = w.shape[0]
+    if w.shape[1] != K or w.dtype != a.dtype:
+        raise KernelError(f"linear: a is {tuple(a.shape)} {a.dtype}, w is {tuple(w.shape)} {w.dtype}")
+    if epilogue not in EPILOGUES:
+        raise KernelError(f"unknown epilogue '{epilogue}'")
+    want = torch.float32 if epilogue in ("add_residual", "store_f32") else a.dtype
+    if out.shape != (M, N) or out.dtype != want:
+        raise KernelError(f"linear({epilogue}): out must be [{M}, {N}] {want}, got {tuple(out.shape)} {out.dtype}")
+    if bias is not None and (bias.dtype != torch.float32 or bias.numel() != N or not bias.is_contiguous()):
+        raise KernelError(f"bias must be contiguous fp32 [{N}]")
+    mode = EPILOGUES[epilogue]
+    if a.dtype == torch.float32:
+        lib = load_library("gemm_f32")
+        rc = lib.mllm_gemm_f32(_p(a), a.stride(0), _p(w), w.stride(0), _p(bias), _p(out), out.stride(0),
+                               M, N, K, mode, _stream())
+    elif a.dtype == torch.bfloat16:
+        lib = load_library("gemm_bf16")
+        rc = lib.mllm_gemm_bf16(_p(a), a.stride(0), _p(w), w.stride(0), _p(bias), _p(out), out.stride(0),
+                                M, N, K, mode, _stream())
+        if rc == -1:
+            raise KernelError(
+                f"linear(bf16): K={K} and the row strides ({a.stride(0)}, {w.stride(0)}) must be multiples "
+                "of 8 elements and the operands 16-byte aligned")
+    else:
+        raise KernelError(f"linear: unsupported dtype {a.dtype}")
+    _check(rc, "linear")
+    return out
+
+
+def kv_append(src: torch.Tensor, k_col: int, v_col: int, kv_dim: int, k_pages: torch.Tensor,
+              v_pages: torch.Tensor, slots: torch.Tensor) -> None:
+    """Copies columns [k_col, k_col+kv_dim) and [v_col, v_col+kv_dim) of each row of ``src``
+    into row ``slots[t]`` of the key and value pages (slot < 0: skipped)."""
+    _gpu(src, k_pages, v_pages, slots)
+    _rows2d(src, "src")
+    T = src.shape[0]
+    _i32(slots, "slots", T)
+    for name, pg in (("k_pages", k_pages), ("v_pages", v_pages)):
+        if pg.dim() != 2 or pg.shape[1] != kv_dim or not pg.is_contiguous() or pg.dtype != src.dtype:
+            raise KernelError(f"{name} must be contiguous [rows, {kv_dim}] {src.dtype}")
+    if max(k_col, v_col) + kv_dim > src.shape[1] or min(k_col, v_col) < 0:
+        raise KernelError("key/value columns lie outside the source rows")
+    lib = load_library("elementwise")
+    _check(lib.mllm_kv_append(_p(src), src.stride(0), k_col, v_col, _p(k_pages), _p(v_pages), kv_dim,
+                              _p(slots), T, _dt(src), _stream()), "kv_append")
+
+
+def paged_attention(q: torch.Tensor, q_col: int, n_heads: int, n_kv_heads: int, head_dim: int,
+                    k_pages: torch.Tensor, v_pages: torch.Tensor, page_size: int,
+                    block_tables: torch.Tensor, token_seq: torch.Tensor, positions: torch.Tensor,
+                    scale: float, window: int, out: torch.Tensor, *, cu_q: Optional[torch.Tensor] = None,
+                    ctx_len: Optional[torch.Tensor] = None, max_q_len: int = 0, max_ctx_len: int = 0) -> torch.Tensor:
+    """Causal attention of the step's queries over the pages.
+
+    q: [T, >= q_col + n_heads*head_dim] (queries of token t start at column q_col);
+    block_tables: int32 [B, max_blocks]; token_seq[t]: row of block_tables; positions[t]:
+    position of token t in its sequence. A query at position p sees keys
+    [max(0, p-window+1) if window else 0, p]. out: [T, n_heads*head_dim].
+    """
+    _gpu(q, k_pages, v_pages, block_tables, token_seq, positions, out)
+    _rows2d(q, "q")
+    _rows2d(out, "out")
+    T = q.shape[0]
+    kv_dim = n_kv_heads * head_dim
+    if q_col < 0 or q_col + n_heads * head_dim > q.shape[1]:
+        raise KernelError("query columns lie outside q's rows")
+    if out.shape[0] != T or out.shape[1] != n_heads * head_dim or out.dtype != q.dtype:
+        raise KernelError(f"out must be [{T}, {n_heads * head_dim}] {q.dtype}")
+    for name, pg in (("k_pages", k_pages), ("v_pages", v_pages)):
+        if pg.dim() != 2 or pg.shape[1] != kv_dim or not pg.is_contiguous() or pg.dtype != q.dtype:
+            raise KernelError(f"{name} must be contiguous [rows, {kv_dim}] {q.dtype}")
+    if k_pages.shape[0] % page_size != 0:
+        raise KernelError("the page pool is not a whole number of pages")
+    if block_tables.dim() != 2 or block_tables.dtype != torch.int32 or not block_tables.is_contiguous():
+        raise KernelError("block_tables must be contiguous int32 [B, max_blocks]")
+    _i32(token_seq, "token_seq", T)
+    _i32(positions, "positions", T)
+    if head_dim % 8 != 0 or head_dim > 256:
+        raise KernelError(f"head_dim={head_dim} is not supported (multiples of 8 up to 256)")
+    if n_heads % n_kv_heads != 0:
+        raise KernelError(f"n_heads={n_heads} is not a multiple of n_kv_heads={n_kv_heads}")
+    esz = q.element_size()
+    if (q.stride(0) * esz) % 16 or (q_col * esz) % 16 or (head_dim * esz) % 16 or q.data_ptr() % 16:
+        raise KernelError("query rows and heads must be 16-byte aligned")
+    lib = load_library("attention")
+    _check(lib.mllm_paged_attention_generic(
+        _p(q), q.stride(0), q_col, _p(k_pages), _p(v_pages), kv_dim, _p(block_tables), block_tables.shape[1],
+        _p(token_seq), _p(positions), T, n_heads, n_kv_heads, head_dim, page_size, ctypes.c_float(scale),
+        int(window or 0), _p(out), out.stride(0), _dt(q), _stream()), "paged_attention")
+    return out
+
+
+def argmax(logits: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+    """out[i] = index of the largest logits[i,:], the lowest index on ties."""
+    _gpu(logits, out)
+    _rows2d(logits, "logits")
+    if logits.dtype != torch.float32:
+        raise KernelError("logits must be fp32")
+    n, V = logits.shape
+    _i32(out, "out", n)
+    lib = load_library("sampling")
+    _check(lib.mllm_argmax(_p(logits), logits.stride(0), n, V, _p(out), _stream()), "argmax")
+    return out
+
+
+def sample(logits: torch.Tensor, temperature: torch.Tensor, u: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+    """Row i: temperature[i] <= 0 takes the argmax; otherwise draws from
+    softmax(logits[i]/temperature[i]) by inverse CDF at u[i] in [0,1)."""
+    _gpu(logits, temperature, u, out)
+    _rows2d(logits, "logits")
+    if logits.dtype != torch.float32:
+        raise KernelError("logits must be fp32")
+    n, V = logits.shape
+    for name, t in (("temperature", temperature), ("u", u)):
+        if t.dtype != torch.float32 or t.numel() < n or not t.is_contiguous():
+            raise KernelError(f"{name} must be contiguous fp32 [{n}]")
+    _i32(out, "out", n)
+    lib = load_library("sampling")
+    _check(lib.mllm_sample(_p(logits), logits.stride(0), n, V, _p(temperature), _p(u), _p(out), _stream()),
+           "sample")
+    return out

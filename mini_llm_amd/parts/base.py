@@ -1,0 +1,121 @@
+"""Interfaces of the parts a model is put together from, and their registries.
+
+A part knows its own sizes and constants (given as parameters), the tensors it owns
+and what it needs from the cache. It does not know which model it is in.
+
+Interfaces (``ctx`` is the step's ``StepContext``; ``x`` is the fp32 residual
+stream ``[T, hidden]``; ``h`` a normalised activation ``[T, hidden]`` in the compute
+dtype):
+
+* ``Norm.forward(x, rows=None) -> h``
+* ``Mixer.forward(h, ctx, cache_view, x, write=True)``: adds the mixer's output into ``x``
+  in place; ``cache_spec()`` says what cache it needs (or None).
+* ``FeedForward.forward(h, ctx, x)``: adds its output into ``x`` in place.
+* ``PositionEncoding.at_embedding(x, ctx)`` / ``.table``: acts where tokens are
+  embedded; ``.in_mixer(q, k, ctx)``: acts on queries/keys inside a mixer.
+* ``Block.forward(x, ctx, cache_view, write)``: runs one layer on the stream.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import Callable, Dict, List, Optional, Tuple
+
+import torch
+
+
+@dataclass
+class ParamSpec:
+    """One tensor a part expects from the checkpoint.
+
+    role: "matrix" (kept in the compute dtype), "vector" (kept in fp32),
+          "table" (integers, kept as int32).
+    layout: "as_stored" or "transpose" (stored [in, out], used as [out, in]).
+    init: (mean, std) of the random-weights mode.
+    """
+    name: str
+    shape: Tuple[int, ...]           # as stored in the checkpoint
+    role: str
+    assign: Callable[[torch.Tensor], None]
+    init: Tuple[float, float] = (0.0, 0.02)
+    layout: str = "as_stored"
+
+
+class Part:
+    def __init__(self, dtype: torch.dtype, device):
+        self.dtype = dtype
+        self.device = torch.device(device)
+
+    def param_specs(self, prefix: str) -> List[ParamSpec]:
+        return []
+
+
+class Norm(Part):
+    def forward(self, x: torch.Tensor, rows: Optional[torch.Tensor] = None) -> torch.Tensor:
+        raise NotImplementedError
+
+
+class Mixer(Part):
+    def cache_spec(self):
+        """KVCacheSpec, StateCacheSpec or None."""
+        return None
+
+    def forward(self, h, ctx, cache_view, x, write: bool = True) -> None:
+        raise NotImplementedError
+
+
+class FeedForward(Part):
+    def forward(self, h, ctx, x) -> None:
+        raise NotImplementedError
+
+
+class PositionEncoding(Part):
+    table: Optional[torch.Tensor] = None     # learned absolute table, if the encoding is one
+
+    def at_embedding(self, x, ctx) -> None:
+        pass
+
+    def in_mixer(self, q, k, ctx):
+        return q, k
+
+
+class Block(Part):
+    def forward(self, x, ctx, cache_view, write: bool = True) -> None:
+        raise NotImplementedError
+
+    def cache_spec(self):
+        return None
+
+
+# ---------------------------------------------------------------------------------
+# registries: kind name -> class. A part class is built as cls(dtype=, device=, **params)
+# (blocks: cls(mixer=, feed_forward=, norms=, dtype=, device=)).
+# ---------------------------------------------------------------------------------
+MIXERS: Dict[str, type] = {}
+FEED_FORWARDS: Dict[str, type] = {}
+NORMS: Dict[str, type] = {}
+POSITIONS: Dict[str, type] = {}
+BLOCKS: Dict[str, type] = {}
+
+
+def _register(table: Dict[str, type], what: str):
+    def deco(kind: str, replace: bool = False):
+        def wrap(cls):
+            if kind in table and not replace:
+                raise ValueError(f"{what} '{kind}' is already registered")
+            table[kind] = cls
+            return cls
+        return wrap
+    return deco
+
+
+register_mixer = _register(MIXERS, "mixer")
+register_feed_forward = _register(FEED_FORWARDS, "feed-forward")
+register_norm = _register(NORMS, "norm")
+register_position = _register(POSITIONS, "position encoding")
+register_block = _register(BLOCKS, "block")
+
+
+def build_part(table: Dict[str, type], spec, dtype, device, what: str):
+    if spec.kind not in table:
+        raise KeyError(f"unknown {what} '{spec.kind}'; registered: {sorted(table)}")
+    return table[spec.kind](dtype=dtype, device=device, **spec.params)
