@@ -1,0 +1,170 @@
+"""Builds replay traces (the four schedule families) and runs them, in-process through the
+engine's ModelRunner or through bin/trace_run, collecting logits per request position."""
+from __future__ import annotations
+
+import json
+import os
+import random
+import subprocess
+import sys
+from typing import Dict, List, Sequence
+
+import numpy as np
+import torch
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def random_requests(vocab: int, lengths: Sequence[int], seed: int) -> Dict[str, List[int]]:
+    g = torch.Generator().manual_seed(seed)
+    return {f"r{i}": torch.randint(0, vocab, (n,), generator=g).tolist() for i, n in enumerate(lengths)}
+
+
+def trace_whole(reqs):
+    """Each request alone and whole: one step, logits at every position."""
+    steps = []
+    for rid, toks in reqs.items():
+        steps.append({"step": len(steps), "entries": [{"id": rid, "tokens": toks, "want": list(range(len(toks)))}],
+                      "end": [rid]})
+    return steps
+
+
+def trace_decode_tail(reqs, tail=32):
+    """Most of a request in one step, then its last `tail` tokens one by one."""
+    steps = []
+    for rid, toks in reqs.items():
+        head = max(1, len(toks) - tail)
+        steps.append({"step": len(steps), "entries": [{"id": rid, "tokens": toks[:head],
+                                                       "want": list(range(head))}], "end": []})
+        for i in range(head, len(toks)):
+            steps.append({"step": len(steps), "entries": [{"id": rid, "tokens": [toks[i]], "want": [0]}],
+                          "end": [rid] if i == len(toks) - 1 else []})
+        if head == len(toks):
+            steps[-1]["end"] = [rid]
+    return steps
+
+
+def trace_chunks(reqs, seed=0, sizes=(2, 3, 5, 7, 16, 17, 2, 31, 4, 64)):
+    """Portions of changing size, down to two tokens."""
+    rng = random.Random(seed)
+    steps = []
+    for rid, toks in reqs.items():
+        i, k = 0, rng.randrange(len(sizes))
+        while i < len(toks):
+            n = min(sizes[k % len(sizes)], len(toks) - i)
+            k += 1
+            steps.append({"step": len(steps), "entries": [{"id": rid, "tokens": toks[i:i + n],
+                                                           "want": list(range(n))}],
+                          "end": [rid] if i + n == len(toks) else []})
+            i += n
+    return steps
+
+
+def trace_mixed(reqs, seed=0, max_live=4, tail=12, sizes=(2, 3, 5, 9, 16, 2, 24)):
+    """Up to `max_live` live requests; portions of some beside decoded tokens of others; a
+    request may sit a step out. Returns (steps, peak of live tokens rounded up to 64 each)."""
+    rng = random.Random(seed)
+    waiting = list(reqs.items())
+    live: Dict[str, int] = {}        # id -> tokens fed so far
+    steps, peak = [], 0
+    while waiting or live:
+        while waiting and len(live) < max_live:
+            rid, _ = waiting.pop(0)
+            live[rid] = 0
+        entries, end = [], []
+        for rid in list(live):
+            toks, fed = reqs[rid], live[rid]
+            if len(live) > 1 and rng.random() < 0.2:
+                continue                                  # left out of this step
+            remaining = len(toks) - fed
+            n = 1 if remaining <= tail else min(rng.choice(sizes), remaining - tail)
+            entries.append({"id": rid, "tokens": toks[fed:fed + n], "want": list(range(n))})
+            live[rid] = fed + n
+        peak = max(peak, sum(-(-max(v, 1) // 64) * 64 for v in live.values()))
+        for rid in list(live):
+            if live[rid] == len(reqs[rid]):
+                end.append(rid)
+                del live[rid]
+        if entries:
+            steps.append({"step": len(steps), "entries": entries, "end": end})
+    return steps, peak
+
+
+def peak_tokens(steps) -> int:
+    live: Dict[str, int] = {}
+    peak = 0
+    for s in steps:
+        for e in s["entries"]:
+            live[e["id"]] = live.get(e["id"], 0) + len(e["tokens"])
+        peak = max(peak, sum(-(-v // 64) * 64 for v in live.values()))
+        for rid in s["end"]:
+            live.pop(rid, None)
+    return peak
+
+
+def collect(steps, outputs: Dict[int, np.ndarray], vocab: int) -> Dict[str, Dict[int, np.ndarray]]:
+    """Maps each step's logits rows back to (request, position)."""
+    fed: Dict[str, int] = {}
+    got: Dict[str, Dict[int, np.ndarray]] = {}
+    for s in steps:
+        rows = outputs.get(s["step"])
+        r = 0
+        for e in s["entries"]:
+            base = fed.get(e["id"], 0)
+            for w in e["want"]:
+                got.setdefault(e["id"], {})[base + w] = rows[r]
+                r += 1
+            fed[e["id"]] = base + len(e["tokens"])
+        assert rows is None or r == rows.shape[0]
+        for rid in s["end"]:
+            fed.pop(rid, None)
+    return got
+
+
+def run_in_process(runner, steps) -> Dict[int, np.ndarray]:
+    from mini_llm_amd.engine.step import StepEntry
+    ids: Dict[str, int] = {}
+    out = {}
+    nxt = 0
+    for s in steps:
+        entries = []
+        for e in s["entries"]:
+            if e["id"] not in ids:
+                ids[e["id"]] = nxt
+                nxt += 1
+            entries.append(StepEntry(ids[e["id"]], e["tokens"], e["want"]))
+        logits = runner.step(entries)
+        if logits is not None:
+            out[s["step"]] = logits.float().cpu().numpy()
+        for rid in s["end"]:
+            runner.end_request(ids.pop(rid))
+    return out
+
+
+def run_trace_run(model_dir, dtype, steps, out_dir, max_tokens, extra=(), env=None, timeout=600):
+    """Drives bin/trace_run the way a user does: one line in, wait for 'done <step>', next line."""
+    cmd = [sys.executable, os.path.join(ROOT, "bin", "trace_run"), "--model", model_dir, "--dtype", dtype,
+           "--out", out_dir, "--max-tokens", str(max_tokens), *extra]
+    p = subprocess.Popen(cmd, stdin=subprocess.PIPE, stdout=subprocess.PIPE, text=True, env=env)
+    try:
+        for s in steps:
+            p.stdin.write(json.dumps(s) + "\n")
+            p.stdin.flush()
+            line = p.stdout.readline().strip()
+            assert line == f"done {s['step']}", f"trace_run answered {line!r} to step {s['step']}"
+        p.stdin.close()
+        assert p.wait(timeout=timeout) == 0
+    finally:
+        if p.poll() is None:
+            p.kill()
+    out = {}
+    vocab = None
+    for s in steps:
+        f = os.path.join(out_dir, f"{s['step']}.f32")
+        n = sum(len(e["want"]) for e in s["entries"])
+        if n:
+            a = np.fromfile(f, dtype="<f4")
+            out[s["step"]] = a.reshape(n, -1)
+        else:
+            assert not os.path.exists(f)
+    return out

@@ -1,0 +1,276 @@
+"""Each HIP kernel alone against its plain reference (tests/plain_ops.py), at sizes other
+than the engine's tiny models: widths and vocabularies that are no power of two,
+ragged row counts, several head sizes and group counts."""
+import math
+
+import pytest
+import torch
+
+import plain_ops
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda:0"
+DTYPES = [torch.float32, torch.bfloat16]
+
+
+@pytest.fixture(scope="module")
+def ops():
+    from mini_llm_amd.kernels import ops as o
+    return o
+
+
+def _tol(dtype, scale=1.0):
+    return (2e-5 if dtype == torch.float32 else 1.6e-2) * scale
+
+
+def _rand(shape, dtype, gen, std=1.0):
+    return (torch.randn(shape, generator=gen, dtype=torch.float32) * std).to(dtype)
+
+
+def test_loaded_libraries_are_in_tree(ops):
+    from mini_llm_amd import build
+    lib = build.load_library("elementwise")
+    assert build.lib_path("elementwise").startswith(build.LIB_DIR) and lib is not None
+
+
+def test_ops_refuse_cpu_tensors(ops):
+    x = torch.zeros(2, 8)
+    with pytest.raises(ops.KernelError, match="not on the GPU"):
+        ops.layernorm(x, torch.ones(8), None, 1e-5, torch.empty(2, 8))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_embed_reference_vector(ops, dtype):
+    # /root/reference/tests/kernels/embedding/gen.py:13-27
+    V, P, D = 64, 32, 768
+    wte = (torch.arange(V)[:, None] * 0.01 + torch.arange(D)[None, :] * 0.0001).to(dtype)
+    wpe = (torch.arange(P)[:, None] * 0.001 + torch.arange(D)[None, :] * 0.00001).to(dtype)
+    ids = torch.tensor([3, 5, 7, 5, 11, 13, 17], dtype=torch.int32)
+    pos = torch.arange(7, dtype=torch.int32)
+    out = torch.empty(7, D, dtype=torch.float32, device=DEV)
+    ops.embed(ids.to(DEV), pos.to(DEV), wte.to(DEV), wpe.to(DEV), out)
+    ref = wte[ids.long()].float() + wpe[pos.long()].float()
+    assert (out.cpu() - ref).abs().max() <= 1e-6
+    # without a position table
+    ops.embed(ids.to(DEV), None, wte.to(DEV), None, out)
+    assert torch.equal(out.cpu(), wte[ids.long()].float())
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("rows,D,eps", [(17, 768, 1e-5), (5, 100, 1e-6), (3, 1600, 1e-5), (1, 16, 1e-3)])
+def test_layernorm(ops, dtype, rows, D, eps):
+    g = torch.Generator().manual_seed(0)
+    x = _rand((rows, D), torch.float32, g) + 0.5
+    gamma = 1 + 0.1 * _rand((D,), torch.float32, g)
+    beta = 0.1 * _rand((D,), torch.float32, g)
+    out = torch.empty(rows, D, dtype=dtype, device=DEV)
+    ops.layernorm(x.to(DEV), gamma.to(DEV), beta.to(DEV), eps, out)
+    ref = plain_ops.layernorm(x, gamma, beta, eps, torch.empty(rows, D, dtype=torch.float64))
+    assert (out.cpu().double() - ref).abs().max() <= _tol(dtype, 4)
+    # selected rows, no bias
+    sel = torch.tensor([rows - 1, 0], dtype=torch.int32)
+    out2 = torch.empty(2, D, dtype=dtype, device=DEV)
+    ops.layernorm(x.to(DEV), gamma.to(DEV), None, eps, out2, rows=sel.to(DEV))
+    ref2 = plain_ops.layernorm(x, gamma, None, eps, torch.empty(2, D, dtype=torch.float64), rows=sel)
+    assert (out2.cpu().double() - ref2).abs().max() <= _tol(dtype, 4)
+
+
+def test_layernorm_constant_row_gives_beta(ops):
+    D = 96
+    x = torch.full((2, D), 3.25)
+    beta = torch.linspace(-1, 1, D)
+    out = torch.empty(2, D, dtype=torch.float32, device=DEV)
+    ops.layernorm(x.to(DEV), torch.ones(D, device=DEV), beta.to(DEV), 1e-6, out)
+    assert (out.cpu() - beta).abs().max() <= 1e-6
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("M,N,K", [(67, 79, 40), (5, 2304, 768), (1, 1000, 96), (130, 320, 96),
+                                   (9, 73, 320), (200, 50257, 64), (33, 96, 3072), (257, 257, 264)])
+@pytest.mark.parametrize("epi", ["store", "gelu_tanh", "gelu_erf", "add_residual", "store_f32"])
+def test_linear(ops, dtype, M, N, K, epi):
+    if N == 50257 and epi not in ("store_f32", "store"):
+        pytest.skip("the wide case is the logits head")
+    g = torch.Generator().manual_seed(M * 1000 + N + K)
+    a = _rand((M, K), dtype, g)
+    w = _rand((N, K), dtype, g, std=1.0 / math.sqrt(K))
+    bias = 0.5 * _rand((N,), torch.float32, g)
+    f32_out = epi in ("add_residual", "store_f32")
+    out0 = _rand((M, N), torch.float32 if f32_out else dtype, g)
+    out = out0.clone().to(DEV)
+    ops.linear(a.to(DEV), w.to(DEV), bias.to(DEV), out, epi)
+    ref = plain_ops.linear(a, w, bias, out0.double().clone(), epi)
+    err = (out.cpu().double() - ref).abs().max().item()
+    tol = 3e-5 if dtype == torch.float32 else (2e-5 + 2e-5 * math.sqrt(K) if f32_out else 4e-2)
+    assert err <= tol, (err, tol)
+    # no bias, strided input rows
+    a2 = _rand((M, K + 8), dtype, g).to(DEV)[:, :K]
+    out = out0.clone().to(DEV)
+    ops.linear(a2, w.to(DEV), None, out, epi)
+    ref = plain_ops.linear(a2.cpu(), w, None, out0.double().clone(), epi)
+    assert (out.cpu().double() - ref).abs().max().item() <= tol
+
+
+def test_linear_fp32_is_true_fp32(ops):
+    """Values that bf16 or tf32 inputs would destroy: 1 + 2^-20 differs from 1 only in true fp32."""
+    K = 64
+    a = torch.ones(4, K)
+    a[:, 0] = 1 + 2.0 ** -20
+    w = torch.zeros(3, K)
+    w[0, 0], w[0, 1] = 1.0, -1.0
+    out = torch.empty(4, 3, device=DEV)
+    ops.linear(a.to(DEV), w.to(DEV), None, out, "store")
+    assert out[0, 0].item() == 2.0 ** -20
+
+
+def test_linear_bf16_refuses_odd_k(ops):
+    a = torch.zeros(4, 36, dtype=torch.bfloat16, device=DEV)
+    w = torch.zeros(8, 36, dtype=torch.bfloat16, device=DEV)
+    with pytest.raises(ops.KernelError, match="multiples of 8"):
+        ops.linear(a, w, None, torch.empty(4, 8, dtype=torch.bfloat16, device=DEV))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_kv_append_reference_vector(ops, dtype):
+    # /root/reference/tests/kernels/append_kv/gen.py:12-24: blocks [3,3,7,7,7,9], offsets [0,1,0,1,2,4]
+    D, BS, NB = 768, 16, 12
+    blocks = torch.tensor([3, 3, 7, 7, 7, 9])
+    offs = torch.tensor([0, 1, 0, 1, 2, 4])
+    qkv = torch.zeros(6, 3 * D)
+    for t in range(6):
+        for part, base in enumerate((10000, 20000, 30000)):
+            qkv[t, part * D:(part + 1) * D] = (base + t * 100 + torch.arange(D)) / 64.0
+    qkv = qkv.to(dtype)
+    kp = torch.full((NB * BS, D), -1.0, dtype=dtype, device=DEV)
+    vp = torch.full((NB * BS, D), -1.0, dtype=dtype, device=DEV)
+    slots = (blocks * BS + offs).to(torch.int32)
+    slots_skip = torch.cat([slots, torch.tensor([-1], dtype=torch.int32)])
+    src = torch.cat([qkv, torch.ones(1, 3 * D, dtype=dtype)])
+    ops.kv_append(src.to(DEV), D, 2 * D, D, kp, vp, slots_skip.to(DEV))
+    assert torch.equal(kp.cpu()[slots.long()], qkv[:, D:2 * D])
+    assert torch.equal(vp.cpu()[slots.long()], qkv[:, 2 * D:])
+    untouched = torch.ones(NB * BS, dtype=torch.bool)
+    untouched[slots.long()] = False
+    assert (kp.cpu()[untouched] == -1).all() and (vp.cpu()[untouched] == -1).all()
+
+
+def _attention_case(ops, dtype, H, Hkv, dh, page, seqs, window, gen, boost=None):
+    """seqs: list of (start, q_len). Builds pages in scrambled order, garbage elsewhere."""
+    B = len(seqs)
+    ctx = [s + n for s, n in seqs]
+    nblk = [-(-c // page) for c in ctx]
+    n_pages = sum(nblk) + 3
+    perm = torch.randperm(n_pages, generator=gen).tolist()
+    kv_dim = Hkv * dh
+    kp = torch.full((n_pages * page, kv_dim), float("nan"), dtype=dtype)
+    vp = torch.full((n_pages * page, kv_dim), float("nan"), dtype=dtype)
+    tables = torch.zeros(B, max(nblk), dtype=torch.int32)
+    T = sum(n for _, n in seqs)
+    q = _rand((T, H * dh + 16), dtype, gen)
+    token_seq, positions = [], []
+    used = 0
+    for b, (s, n) in enumerate(seqs):
+        for j in range(nblk[b]):
+            tables[b, j] = perm[used]
+            used += 1
+        k = _rand((ctx[b], kv_dim), dtype, gen)
+        v = _rand((ctx[b], kv_dim), dtype, gen)
+        if boost is not None and ctx[b] > boost[0]:
+            # one far key stands out: its score dominates for the last query
+            far = boost[0]
+            k[far] = k[far] * 0 + (q[len(token_seq) + n - 1, 8:8 + H * dh].float().view(H, dh)[::H // Hkv]
+                                   .reshape(-1) * boost[1]).to(dtype)
+        js = torch.arange(ctx[b])
+        rows = tables[b].long()[js // page] * page + js % page
+        kp[rows] = k
+        vp[rows] = v
+        token_seq += [b] * n
+        positions += list(range(s, s + n))
+    token_seq = torch.tensor(token_seq, dtype=torch.int32)
+    positions = torch.tensor(positions, dtype=torch.int32)
+    scale = dh ** -0.5
+    out = torch.zeros(T, H * dh, dtype=dtype, device=DEV)
+    ops.paged_attention(q.to(DEV), 8, H, Hkv, dh, kp.to(DEV), vp.to(DEV), page, tables.to(DEV),
+                        token_seq.to(DEV), positions.to(DEV), scale, window, out,
+                        max_q_len=max(n for _, n in seqs), max_ctx_len=max(ctx))
+    ref = torch.zeros(T, H * dh, dtype=torch.float64)
+    plain_ops.paged_attention(q, 8, H, Hkv, dh, kp, vp, page, tables, token_seq, positions, scale, window, ref)
+    return out.cpu().double(), ref
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("H,Hkv,dh,page", [(12, 12, 64, 16), (4, 4, 16, 4), (3, 3, 32, 8), (6, 2, 48, 16),
+                                           (5, 1, 128, 32), (2, 2, 256, 64)])
+def test_paged_attention_mixed_batch(ops, dtype, H, Hkv, dh, page):
+    g = torch.Generator().manual_seed(H * 100 + dh)
+    seqs = [(0, 37), (130, 1), (64, 2), (5, 70), (0, 1), (199, 1)]
+    out, ref = _attention_case(ops, dtype, H, Hkv, dh, page, seqs, 0, g)
+    assert torch.isfinite(out).all()
+    assert (out - ref).abs().max() <= _tol(dtype, 2)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_paged_attention_far_key_stands_out(ops, dtype):
+    """One key hundreds of positions back carries almost all the weight of the last query."""
+    g = torch.Generator().manual_seed(7)
+    out, ref = _attention_case(ops, dtype, 4, 2, 64, 16, [(600, 3), (0, 300)], 0, g, boost=(3, 4.0))
+    assert (out - ref).abs().max() <= _tol(dtype, 2)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("window", [1, 7, 64, 65])
+def test_paged_attention_window_edge(ops, dtype, window):
+    g = torch.Generator().manual_seed(window)
+    out, ref = _attention_case(ops, dtype, 4, 2, 32, 8, [(0, 80), (130, 1), (63, 3)], window, g)
+    assert (out - ref).abs().max() <= _tol(dtype, 2)
+
+
+def test_argmax_ties_take_lowest_index(ops):
+    V = 50257
+    g = torch.Generator().manual_seed(3)
+    logits = _rand((5, V), torch.float32, g)
+    logits[0, 40000] = logits[0, 123] = 9.0
+    logits[1, V - 1] = 10.0
+    logits[2, 0] = 10.0
+    logits[3, :] = 0.5
+    out = torch.empty(5, dtype=torch.int32, device=DEV)
+    ops.argmax(logits.to(DEV), out)
+    ref = plain_ops.argmax(logits, torch.empty(5, dtype=torch.int32))
+    assert out.cpu().tolist() == ref.tolist()
+    assert out.cpu().tolist()[:4] == [123, V - 1, 0, 0]
+
+
+@pytest.mark.parametrize("V", [4, 1000, 50257])
+def test_sample_inverse_cdf(ops, V):
+    g = torch.Generator().manual_seed(V)
+    n = 64
+    logits = _rand((n, V), torch.float32, g, std=2.0)
+    temps = torch.rand(n, generator=g) * 1.5 + 0.2
+    temps[::7] = 0.0
+    u = torch.rand(n, generator=g)
+    out = torch.empty(n, dtype=torch.int32, device=DEV)
+    ops.sample(logits.to(DEV), temps.to(DEV), u.to(DEV), out)
+    got = out.cpu().tolist()
+    for i in range(n):
+        row = logits[i].double()
+        if temps[i] <= 0:
+            assert got[i] == int(row.argmax())
+            continue
+        p = torch.softmax(row / temps[i].double(), 0)
+        c = torch.cumsum(p, 0)
+        lo = float(c[got[i] - 1]) if got[i] > 0 else 0.0
+        hi = float(c[got[i]])
+        assert lo - 1e-5 <= float(u[i]) <= hi + 1e-5, (i, got[i], lo, float(u[i]), hi)
+
+
+def test_sample_frequencies_follow_softmax(ops):
+    logits = torch.tensor([[0.0, 1.0, 2.0, -1.0]]).repeat(4096, 1)
+    g = torch.Generator().manual_seed(11)
+    u = torch.rand(4096, generator=g)
+    temps = torch.full((4096,), 0.8)
+    out = torch.empty(4096, dtype=torch.int32, device=DEV)
+    ops.sample(logits.to(DEV), temps.to(DEV), u.to(DEV), out)
+    freq = torch.bincount(out.cpu().long(), minlength=4).double() / 4096
+    p = torch.softmax(logits[0].double() / 0.8, 0)
+    assert (freq - p).abs().max() < 4 * math.sqrt(0.25 / 4096)
