@@ -1,0 +1,163 @@
+"""Headline benchmark: decode tokens/s (batch 8 by default) and prefill tokens/s at 2,048
+tokens for GPT-2 small sizes with random weights on one MI355X, with roofline fractions.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch B] [--dtype bfloat16]
+
+A "step" is one decode step of the whole engine (scheduler, step function, kernels,
+sampling). Prints ONE JSON line.
+"""
+import argparse
+import json
+import os
+import sys
+import tempfile
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK = 8.0e12                                   # bytes/s
+MFMA_PEAK = {"bfloat16": 2.5e15, "float32": 157.3e12}
+
+
+def small_config(n_layer):
+    # BASELINE.json configs[2]: GPT-2 small sizes
+    return dict(architectures=["GPT2LMHeadModel"], model_type="gpt2", n_layer=n_layer, n_embd=768, n_head=12,
+                n_inner=3072, vocab_size=50257, n_positions=1024, layer_norm_epsilon=1e-5,
+                activation_function="gelu_new", eos_token_id=50256, bos_token_id=50256)
+
+
+def matmul_params(cfg):
+    D, F = cfg["n_embd"], cfg["n_inner"]
+    return cfg["n_layer"] * (3 * D * D + D * D + 2 * D * F)
+
+
+def weight_bytes(cfg, esz):
+    D, F, L, V = cfg["n_embd"], cfg["n_inner"], cfg["n_layer"], cfg["vocab_size"]
+    vec = L * (3 * D + D + F + D + 4 * D) + 2 * D
+    return (matmul_params(cfg) + V * D) * esz + vec * 4
+
+
+def kv_bytes_per_token(cfg, esz):
+    return cfg["n_layer"] * 2 * cfg["n_embd"] * esz
+
+
+def decode_run(model_dir, dtype, batch, prompt_len, steps, warmup, cfg):
+    import torch
+    from mini_llm_amd import Engine, EngineOptions, SamplingParams
+    pages = batch * (cfg["n_positions"] // 16) + 16
+    engine = Engine.from_pretrained(model_dir, dtype=dtype, device="cuda:0",
+                                    options=EngineOptions(kv_block_size=16, total_kv_blocks=pages,
+                                                          max_batch_num=max(batch, 1),
+                                                          max_tokens_per_step=max(2048, batch),
+                                                          prefill_chunk=1024))
+    g = torch.Generator().manual_seed(2)
+    prompts = [torch.randint(0, cfg["vocab_size"], (prompt_len,), generator=g).tolist() for _ in range(batch)]
+    total_new = warmup + steps + 1 + batch      # requests that were prefilled first decode longer
+    assert prompt_len + total_new <= cfg["n_positions"], "the run would pass the last position"
+    params = SamplingParams(max_new_tokens=total_new, ignore_eos=True)
+    for p in prompts:
+        engine.add_request(p, params)
+    # untimed: prefill until every request is decoding
+    while engine.scheduler.queue_length("decode") < batch:
+        engine.step()
+    for _ in range(warmup):
+        engine.step()
+    torch.cuda.synchronize()
+    ctx0 = prompt_len + 1 + warmup
+    t0 = time.perf_counter()
+    n_tok = 0
+    for _ in range(steps):
+        n_tok += len(engine.step())
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    assert n_tok == batch * steps, (n_tok, batch, steps)
+    mean_ctx = ctx0 + (steps - 1) / 2.0
+    del engine
+    torch.cuda.empty_cache()
+    return n_tok / dt, dt / steps, mean_ctx
+
+
+def prefill_run(model_dir, dtype, cfg, n_req=2, n_tok=1024, reps=5):
+    import torch
+    from mini_llm_amd.engine.step import ModelRunner, StepEntry
+    from mini_llm_amd.models import load_model
+    model = load_model(model_dir, dtype, "cuda:0")
+    runner = ModelRunner(model, 16, n_req * n_tok // 16 + 8, n_req)
+    g = torch.Generator().manual_seed(3)
+    toks = [torch.randint(0, cfg["vocab_size"], (n_tok,), generator=g).tolist() for _ in range(n_req)]
+    times = []
+    for rep in range(reps + 2):
+        entries = [StepEntry(i, toks[i], [n_tok - 1]) for i in range(n_req)]
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        logits = runner.step(entries)
+        torch.cuda.synchronize()
+        times.append(time.perf_counter() - t0)
+        for i in range(n_req):
+            runner.end_request(i)
+    dt = min(times[2:])
+    T = n_req * n_tok
+    D, V, L = cfg["n_embd"], cfg["vocab_size"], cfg["n_layer"]
+    flops = 2.0 * T * matmul_params(cfg) + L * n_req * 4.0 * D * (n_tok * (n_tok + 1) / 2) + 2.0 * D * V * n_req
+    del runner, model
+    torch.cuda.empty_cache()
+    return T / dt, dt, flops
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=256)
+    ap.add_argument("--warmup", type=int, default=32)
+    ap.add_argument("--batch", type=int, default=8)
+    ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
+    ap.add_argument("--layers", type=int, default=12, help="fewer layers than GPT-2 small's 12 are named in config")
+    ap.add_argument("--prompt-len", type=int, default=512)
+    ap.add_argument("--no-points", action="store_true", help="skip the batch-1/64 and prefill measurements")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
+        return 2
+    import torch
+    from mini_llm_amd import write_random_model
+
+    cfg = small_config(args.layers)
+    esz = 2 if args.dtype == "bfloat16" else 4
+    steps = min(args.steps, cfg["n_positions"] - args.prompt_len - args.warmup - 2 - 64)
+    with tempfile.TemporaryDirectory() as d:
+        write_random_model(dict(cfg), d, seed=2)
+        tps, step_s, mean_ctx = decode_run(d, args.dtype, args.batch, args.prompt_len, steps, args.warmup, cfg)
+        bytes_step = weight_bytes(cfg, esz) + args.batch * mean_ctx * kv_bytes_per_token(cfg, esz)
+        achieved = bytes_step / step_s
+        rec = {
+            "metric": "decode tok/s at batch 8 (GPT-2 small sizes, 512-token prompts, context to 1024)",
+            "value": round(tps, 1), "unit": "tok/s", "n_gpus": 1, "steps": steps, "warmup": args.warmup,
+            "ms_per_step": round(step_s * 1e3, 4), "higher_is_better": True, "scaling": "weak",
+            "vs_baseline": None, "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
+            "data": "synthetic (random weights seed 2, uniform random token ids)",
+            "config": {"model": "gpt2-small-sizes", "n_layer": cfg["n_layer"], "n_layer_full": 12,
+                       "n_embd": cfg["n_embd"], "n_head": cfg["n_head"], "head_dim": 64,
+                       "n_inner": cfg["n_inner"], "vocab_size": cfg["vocab_size"],
+                       "n_positions": cfg["n_positions"], "global_batch": args.batch,
+                       "prompt_len": args.prompt_len, "seq_len": cfg["n_positions"],
+                       "mean_context": round(mean_ctx, 1), "kv_block_size": 16, "parallelism": "single-gpu"},
+            "roofline": {"bound": "hbm", "achieved": round(achieved / 1e9, 2), "peak": HBM_PEAK / 1e9,
+                         "unit": "GB/s", "frac": round(achieved / HBM_PEAK, 5)},
+        }
+        if not args.no_points:
+            ptps, pdt, flops = prefill_run(d, args.dtype, cfg)
+            rec["prefill"] = {"value": round(ptps, 1), "tokens": 2048, "ms": round(pdt * 1e3, 4),
+                              "frac": round(flops / pdt / MFMA_PEAK[args.dtype], 5)}
+            points = {}
+            for b in (1, 64):
+                s = min(steps, 128)
+                v, _, _ = decode_run(d, args.dtype, b, args.prompt_len, s, min(args.warmup, 16), cfg)
+                points[f"decode_b{b}"] = round(v, 1)
+            rec["points"] = points
+    print(json.dumps(rec))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())
