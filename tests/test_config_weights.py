@@ -1,0 +1,172 @@
+"""Configuration, registry, safetensors I/O, loader errors and the random-weights mode."""
+import json
+import os
+
+import pytest
+import torch
+
+import mini_llm_amd.models  # noqa: F401  (registers the architecture)
+from conftest import TINY_A, TINY_B
+from mini_llm_amd.config.base import ConfigError, LayerCall
+from mini_llm_amd.config.gpt2 import GPT2Config
+from mini_llm_amd.config.registry import (architecture_of, get_architecture, load_config,
+                                          registered_architectures)
+from mini_llm_amd.models import load_model
+from mini_llm_amd.weights.loader import WeightsError, load_weights
+from mini_llm_amd.weights.random_init import write_random_model
+from mini_llm_amd.weights.safetensors_io import SafetensorsError, SafetensorsFile, save_file
+
+
+def test_config_reads_its_own_keys():
+    a, b = GPT2Config.from_dict(TINY_A), GPT2Config.from_dict(TINY_B)
+    assert (a.n_layer, a.n_embd, a.n_head, a.head_dim, a.inner_dim, a.vocab_size, a.n_positions) == \
+           (2, 64, 4, 16, 256, 512, 128)
+    assert (b.n_layer, b.n_embd, b.n_head, b.head_dim, b.inner_dim, b.vocab_size, b.n_positions) == \
+           (3, 96, 3, 32, 320, 1000, 256)
+    assert a.layer_norm_epsilon == 1e-5 and b.layer_norm_epsilon == 1e-6
+    assert a.eos_token_id == 511 and b.max_positions == 256
+    sa, sb = a.layer_specs(), b.layer_specs()
+    assert len(sa) == 2 and len(sb) == 3
+    assert sa[0].feed_forward.params["activation"] == "gelu_tanh"
+    assert sb[0].feed_forward.params["activation"] == "gelu_erf"
+    assert sb[2].mixer.params["scale"] == pytest.approx(32 ** -0.5) and sb[2].weight_prefix == "h.2."
+    assert a.layer_order() == [LayerCall(0, 0, True), LayerCall(1, 1, True)]
+    assert GPT2Config.from_dict(a.to_dict()) == a
+
+
+@pytest.mark.parametrize("change,match", [
+    ({"n_embd": None}, "n_embd"), ({"vocab_size": "x"}, "vocab_size"), ({"n_head": 5}, "divisible"),
+    ({"activation_function": "relu"}, "activation_function"), ({"layer_norm_epsilon": 0}, "positive"),
+    ({"scale_attn_by_inverse_layer_idx": True}, "not supported"), ({"reorder_and_upcast_attn": True}, "not supported"),
+    ({"tie_word_embeddings": False}, "untied"), ({"n_layer": 0}, "positive"), ({"n_inner": 1.5}, "n_inner"),
+])
+def test_config_refuses(change, match):
+    d = dict(TINY_A, **change)
+    d = {k: v for k, v in d.items() if not (k in change and change[k] is None and k != "n_inner")}
+    with pytest.raises(ConfigError, match=match):
+        GPT2Config.from_dict(d)
+
+
+def test_registry(tmp_path):
+    assert "GPT2LMHeadModel" in registered_architectures()
+    assert architecture_of({"model_type": "gpt2"}).name == "GPT2LMHeadModel"
+    with pytest.raises(ConfigError, match="unknown architecture 'LlamaForCausalLM'.*GPT2LMHeadModel"):
+        get_architecture("LlamaForCausalLM")
+    with pytest.raises(ConfigError, match="names no architecture"):
+        architecture_of({"n_embd": 4})
+    with pytest.raises(ConfigError, match="no such file"):
+        load_config(str(tmp_path))
+    (tmp_path / "config.json").write_text("{not json")
+    with pytest.raises(ConfigError, match="not valid JSON"):
+        load_config(str(tmp_path))
+
+
+def test_safetensors_roundtrip_and_interop(tmp_path):
+    from safetensors.torch import load_file, save_file as st_save
+    g = torch.Generator().manual_seed(0)
+    tensors = {"a.weight": torch.randn(3, 5, generator=g).bfloat16(), "b": torch.randn(7, generator=g),
+               "c.table": torch.arange(6, dtype=torch.int32).reshape(2, 3), "d": torch.tensor(2.5)}
+    p = str(tmp_path / "x.safetensors")
+    save_file(tensors, p, metadata={"format": "pt"})
+    theirs = load_file(p)                                   # the library reads what we wrote
+    with SafetensorsFile(p) as f:
+        assert sorted(f.names()) == sorted(tensors)
+        for k, v in tensors.items():
+            assert f.info(k) == (v.dtype, tuple(v.shape))
+            assert torch.equal(f.tensor(k), v) and torch.equal(theirs[k], v)
+    q = str(tmp_path / "y.safetensors")
+    st_save({k: v for k, v in tensors.items()}, q)          # we read what the library wrote
+    with SafetensorsFile(q) as f:
+        for k, v in tensors.items():
+            assert torch.equal(f.tensor(k), v)
+
+
+def test_safetensors_refuses_broken_files(tmp_path):
+    p = tmp_path / "short.safetensors"
+    p.write_bytes(b"\x01\x02")
+    with pytest.raises(SafetensorsError, match="too short"):
+        SafetensorsFile(str(p))
+    save_file({"a": torch.zeros(4, 4)}, str(p))
+    raw = p.read_bytes()
+    p.write_bytes(raw[:-8])                                  # data cut off
+    with pytest.raises(SafetensorsError, match="offsets"):
+        SafetensorsFile(str(p))
+    p.write_bytes((10 ** 9).to_bytes(8, "little") + b"{}")
+    with pytest.raises(SafetensorsError, match="header length"):
+        SafetensorsFile(str(p))
+
+
+def _tensors(model_dir):
+    with SafetensorsFile(os.path.join(model_dir, "model.safetensors")) as f:
+        return {n: f.tensor(n) for n in f.names()}
+
+
+def test_random_model_folder(tmp_path):
+    d = write_random_model(dict(TINY_B), str(tmp_path / "m"), seed=1)
+    cfg = json.load(open(os.path.join(d, "config.json")))
+    assert cfg["architectures"] == ["GPT2LMHeadModel"] and cfg["n_inner"] == 320
+    t = _tensors(d)
+    assert len(t) == 2 + 3 * 12 + 2
+    assert t["wte.weight"].shape == (1000, 96) and t["wte.weight"].dtype == torch.bfloat16
+    assert t["h.1.attn.c_attn.weight"].shape == (96, 288)          # Conv1D: [in, out]
+    assert t["h.2.mlp.c_fc.weight"].shape == (96, 320) and t["h.2.mlp.c_proj.weight"].shape == (320, 96)
+    assert t["h.0.ln_1.weight"].dtype == torch.float32 and t["h.0.attn.c_attn.bias"].dtype == torch.float32
+    # the distributions BASELINE names: N(0, .02); residual projections N(0, .02/sqrt(2L)); gains N(1, .1)
+    assert t["wte.weight"].float().std().item() == pytest.approx(0.02, rel=0.05)
+    assert t["h.0.mlp.c_proj.weight"].float().std().item() == pytest.approx(0.02 / 6 ** 0.5, rel=0.05)
+    assert t["h.0.attn.c_proj.weight"].float().std().item() == pytest.approx(0.02 / 6 ** 0.5, rel=0.08)
+    assert t["ln_f.weight"].mean().item() == pytest.approx(1.0, abs=0.05)
+    assert t["ln_f.weight"].std().item() == pytest.approx(0.1, rel=0.3)
+    # same seed, same bytes; another seed, other values
+    d2 = write_random_model(dict(TINY_B), str(tmp_path / "m2"), seed=1)
+    d3 = write_random_model(dict(TINY_B), str(tmp_path / "m3"), seed=2)
+    assert open(os.path.join(d, "model.safetensors"), "rb").read() == open(os.path.join(d2, "model.safetensors"), "rb").read()
+    assert not torch.equal(_tensors(d3)["wpe.weight"], t["wpe.weight"])
+
+
+def test_loader_places_and_converts(tmp_path):
+    d = write_random_model(dict(TINY_A), str(tmp_path / "m"), seed=0, weights_dtype="float32")
+    t = _tensors(d)
+    for dtype in (torch.float32, torch.bfloat16):
+        m = load_model(d, dtype, "cpu")
+        att = m.layers[1].mixer
+        assert att.qkv.weight.dtype == dtype and att.qkv.weight.shape == (192, 64)       # held [out, in]
+        assert torch.equal(att.qkv.weight, t["h.1.attn.c_attn.weight"].t().to(dtype))
+        assert att.qkv.bias.dtype == torch.float32 and torch.equal(att.qkv.bias, t["h.1.attn.c_attn.bias"])
+        assert m.layers[0].norm2.gamma.dtype == torch.float32           # stored in 32-bit, stays so
+        assert torch.equal(m.final_norm.beta, t["ln_f.bias"])
+        assert m.embedding.weight.dtype == dtype and m.position.table.shape == (128, 64)
+        assert m.head.embedding is m.embedding                           # tied head
+
+
+def test_loader_accepts_prefix_and_mask_buffers(tmp_path):
+    d = write_random_model(dict(TINY_A), str(tmp_path / "m"), seed=0)
+    t = {"transformer." + k: v for k, v in _tensors(d).items()}
+    t["transformer.h.0.attn.bias"] = torch.ones(1, 1, 8, 8)
+    t["transformer.h.1.attn.masked_bias"] = torch.tensor(-1e4)
+    t["lm_head.weight"] = t["transformer.wte.weight"].clone()
+    save_file(t, os.path.join(d, "model.safetensors"))
+    load_model(d, "float32", "cpu")
+
+
+def test_loader_lists_every_mismatch(tmp_path):
+    d = write_random_model(dict(TINY_A), str(tmp_path / "m"), seed=0)
+    t = _tensors(d)
+    del t["h.1.ln_2.bias"], t["wpe.weight"]
+    t["h.0.mlp.c_fc.weight"] = torch.zeros(256, 64, dtype=torch.bfloat16)     # transposed by mistake
+    t["h.0.attn.c_attn.bias"] = torch.zeros(64)
+    t["h.7.extra.weight"] = torch.zeros(2)
+    save_file(t, os.path.join(d, "model.safetensors"))
+    with pytest.raises(WeightsError) as ei:
+        load_model(d, "float32", "cpu")
+    e = ei.value
+    assert e.missing == ["h.1.ln_2.bias", "wpe.weight"]
+    assert e.unexpected == ["h.7.extra.weight"]
+    assert sorted(n for n, _, _ in e.wrong_shape) == ["h.0.attn.c_attn.bias", "h.0.mlp.c_fc.weight"]
+    msg = str(e)
+    for piece in ("missing tensors (2)", "h.1.ln_2.bias", "unexpected tensors (1)", "h.7.extra.weight",
+                  "wrong shapes (2)", "expected [64, 256], found [256, 64]"):
+        assert piece in msg
+    os.remove(os.path.join(d, "model.safetensors"))
+    with pytest.raises(WeightsError, match="neither model.safetensors"):
+        load_model(d, "float32", "cpu")

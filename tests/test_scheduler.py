@@ -1,0 +1,217 @@
+"""The scheduler's decisions, driven without a model (the reference tests its scheduler with a
+mock backend that emits 1000, 1001, ... : /root/reference/include/runtime/mock_backend.h:10-48,
+/root/reference/tests/cpp/test_scheduler.cpp:160-221), and the engine under page pressure on
+the CPU reference ops."""
+import pytest
+import torch
+
+import plain_ops
+from conftest import TINY
+from mini_llm_amd.cache.manager import CacheManager, GroupSpec
+from mini_llm_amd.engine.scheduler import Scheduler
+
+
+def drive(s, eos_after=None, max_iters=10000):
+    """Runs the loop with a fake model; returns per-request token counts and the plans."""
+    produced, plans = {}, []
+    for _ in range(max_iters):
+        plan = s.schedule()
+        if not plan:
+            break
+        plans.append(plan)
+        s.commit()
+        for e in plan:
+            if e.want_last:
+                n = produced.get(e.request_id, 0) + 1
+                produced[e.request_id] = n
+                s.on_token(e.request_id, eos_after is not None and n >= eos_after.get(e.request_id, 10 ** 9))
+    return produced, plans
+
+
+def make(n_pages=64, page=4, seqs=4, budget=32, chunk=16, max_pos=128, slots=None):
+    cm = CacheManager([GroupSpec(page, n_pages)], slots or seqs)
+    return cm, Scheduler(cm, seqs, budget, chunk, max_pos)
+
+
+def test_single_request_lifecycle():
+    cm, s = make()
+    s.add_request(7, 5, 4)
+    assert s.state(7) == "waiting_prefill"
+    plan = s.schedule()
+    assert [(e.request_id, e.start, e.n_tokens, e.want_last) for e in plan] == [(7, 0, 5, True)]
+    assert s.state(7) == "prefill"
+    s.commit()
+    assert not s.on_token(7, False) and s.state(7) == "decode_ready"
+    starts = []
+    for i in range(3):
+        (e,) = s.schedule()
+        starts.append((e.start, e.n_tokens, e.want_last))
+        s.commit()
+        done = s.on_token(7, False)
+        assert done == (i == 2)
+    assert starts == [(5, 1, True), (6, 1, True), (7, 1, True)]       # the prefill's token is output #1
+    assert s.state(7) == "finished" and s.generated(7) == 4 and not s.has_work()
+    assert cm.free_pages() == 64 and cm.n_requests() == 0 and cm.check() == ""
+    assert s.schedule() == []
+
+
+def test_refused_requests():
+    cm, s = make(max_pos=16)
+    with pytest.raises(ValueError):
+        s.add_request(1, 0, 4)
+    with pytest.raises(ValueError):
+        s.add_request(1, 17, 4)
+    with pytest.raises(ValueError):
+        s.add_request(1, 4, 0)
+    s.add_request(1, 16, 4)
+    with pytest.raises(KeyError):
+        s.add_request(1, 3, 4)
+    produced, _ = drive(s)
+    assert produced == {1: 1}              # the prompt fills every position: one token, then the length cap
+
+
+def test_prompts_are_cut_under_the_budget_and_decodes_come_first():
+    cm, s = make(budget=12, chunk=8)
+    s.add_request(1, 20, 3)
+    s.add_request(2, 6, 3)
+    p1 = s.schedule()
+    assert [(e.request_id, e.start, e.n_tokens, e.want_last) for e in p1] == [(1, 0, 8, False), (2, 0, 4, False)]
+    s.commit()
+    p2 = s.schedule()
+    assert [(e.request_id, e.start, e.n_tokens, e.want_last) for e in p2] == [(1, 8, 8, False), (2, 4, 2, True)]
+    s.commit(); s.on_token(2, False)
+    p3 = s.schedule()          # request 2 decodes first, then request 1's last portion
+    assert [(e.request_id, e.start, e.n_tokens, e.want_last) for e in p3] == [(2, 6, 1, True), (1, 16, 4, True)]
+    s.commit(); s.on_token(2, False); s.on_token(1, False)
+    produced, _ = drive(s)
+    assert s.generated(1) == 3 and s.generated(2) == 3 and cm.free_pages() == 64
+
+
+def test_max_num_seqs_limits_a_step_and_nobody_starves():
+    cm, s = make(seqs=2, slots=8)
+    for i in range(5):
+        s.add_request(i, 3, 4)
+    produced, plans = drive(s)
+    assert all(len(p) <= 2 for p in plans)
+    assert produced == {i: 4 for i in range(5)}
+    c = s.counters()
+    assert c["finished"] == 5 and c["prefill_tokens"] == 15 and c["decode_tokens"] == 15
+
+
+def test_admission_waits_for_pages_first_come_first_served():
+    cm, s = make(n_pages=6, page=4)             # 24 tokens of cache
+    s.add_request(1, 16, 3)                     # 4 pages, 5 with its outputs
+    s.add_request(2, 12, 2)                     # 3 pages: does not fit beside request 1
+    s.add_request(3, 2, 2)                      # would fit, but may not overtake request 2
+    plan = s.schedule()
+    assert [e.request_id for e in plan] == [1]
+    assert s.state(2) == "deferred_prefill" and s.state(3) == "waiting_prefill"
+    assert (2, "deferred") in s.pop_events()
+    produced, _ = drive(s)
+    assert produced == {1: 3, 2: 2, 3: 2} and s.counters()["preemptions"] == 0
+    assert cm.free_pages() == 6 and cm.check() == ""
+
+
+def test_out_of_pages_defers_decodes_then_preempts_the_latest():
+    cm, s = make(n_pages=4, page=4, budget=16, chunk=16)
+    s.add_request(1, 7, 8)                      # 2 pages; needs a 3rd at length 9, a 4th at 13
+    s.add_request(2, 7, 8)                      # 2 pages
+    events = []
+    produced = {}
+    for _ in range(200):
+        plan = s.schedule()
+        events += s.pop_events()
+        if not plan:
+            break
+        s.commit()
+        for e in plan:
+            if e.want_last:
+                produced[e.request_id] = produced.get(e.request_id, 0) + 1
+                s.on_token(e.request_id, False)
+        assert cm.check() == ""
+    # both need a third page at the same step: the later one is preempted, recomputed after the first ends
+    assert (2, "preempted") in events
+    assert produced == {1: 8, 2: 8}
+    c = s.counters()
+    assert c["preemptions"] >= 1 and c["deferred_decodes"] >= 1 and c["failures"] == 0
+    assert cm.free_pages() == 4 and cm.n_requests() == 0
+
+
+def test_a_request_larger_than_the_pool_fails_alone():
+    cm, s = make(n_pages=2, page=4)
+    s.add_request(1, 9, 2)                      # 3 pages, the pool has 2
+    s.add_request(2, 3, 2)
+    produced, _ = drive(s)
+    assert s.state(1) == "failed" and produced == {2: 2}
+    assert (1, "failed") in s.pop_events()
+    # one that fits at first and outgrows the pool fails when it is alone
+    s.add_request(3, 7, 8)
+    produced, _ = drive(s)
+    assert s.state(3) == "failed" and produced[3] == 2 and cm.free_pages() == 2
+
+
+def test_eos_and_abort_free_everything():
+    cm, s = make()
+    s.add_request(1, 5, 50)
+    s.add_request(2, 5, 50)
+    s.add_request(3, 40, 50)
+    plan = s.schedule(); s.commit()
+    for e in plan:
+        if e.want_last:
+            s.on_token(e.request_id, e.request_id == 1)
+    assert s.state(1) == "finished" and s.state(3) == "prefill"
+    s.abort(3)
+    assert s.state(3) == "failed"
+    produced, _ = drive(s, eos_after={2: 3})
+    assert s.generated(2) == 4 and cm.free_pages() == 64 and cm.n_requests() == 0 and not s.has_work()
+
+
+# ---- the engine above it, on the CPU reference ops -------------------------------------------
+
+@pytest.fixture()
+def cpu_ops(monkeypatch):
+    plain_ops.install(monkeypatch)
+
+
+def _engine(model_dir, **opt):
+    from mini_llm_amd import Engine, EngineOptions, load_model
+    return Engine(load_model(model_dir, "float32", "cpu"), EngineOptions(**opt))
+
+
+def test_generation_is_the_same_alone_and_under_page_pressure(cpu_ops, tiny_model_dirs):
+    from mini_llm_amd import SamplingParams
+    g = torch.Generator().manual_seed(4)
+    prompts = [torch.randint(0, 1000, (n,), generator=g).tolist() for n in (1, 9, 40, 100)]
+    params = [SamplingParams(temperature=0.8, seed=i, max_new_tokens=24, ignore_eos=True) for i in range(4)]
+    alone = []
+    for p, sp in zip(prompts, params):
+        e = _engine(tiny_model_dirs["b"], kv_block_size=8, total_kv_blocks=64, max_batch_num=4)
+        alone.append(e.generate([p], sp)[0])
+    assert all(len(o) == 24 for o in alone) and len({tuple(o) for o in alone}) == 4
+    roomy = _engine(tiny_model_dirs["b"], kv_block_size=8, total_kv_blocks=64, max_batch_num=4,
+                    max_tokens_per_step=32, prefill_chunk=16)
+    assert roomy.generate(prompts, params) == alone
+    # 26 pages: the four requests need 4+5+8+16 = 33 at the end, so some are deferred or recomputed
+    tight = _engine(tiny_model_dirs["b"], kv_block_size=8, total_kv_blocks=26, max_batch_num=4,
+                    max_tokens_per_step=32, prefill_chunk=16)
+    assert tight.generate(prompts, params) == alone
+    st = tight.stats()
+    assert st["deferred_prefills"] + st["deferred_decodes"] + st["preemptions"] > 0
+    assert st["free_pages"] == 26 and tight.runner.manager.check() == ""
+
+
+def test_greedy_generation_matches_plain_and_stops_at_eos(cpu_ops, tiny_model_dirs):
+    import plain_gpt2
+    from mini_llm_amd import SamplingParams
+    cfg, w = plain_gpt2.read_model(tiny_model_dirs["a"])
+    g = torch.Generator().manual_seed(1)
+    prompts = [torch.randint(0, 511, (n,), generator=g).tolist() for n in (5, 17, 33)]
+    e = _engine(tiny_model_dirs["a"], kv_block_size=4, total_kv_blocks=40, max_batch_num=4)
+    outs = e.generate(prompts, SamplingParams(max_new_tokens=16, ignore_eos=True))
+    for p, o in zip(prompts, outs):
+        assert o == plain_gpt2.greedy_generate(cfg, w, p, 16)
+    # declare the first generated token to be EOS: generation ends there
+    e2 = _engine(tiny_model_dirs["a"], kv_block_size=4, total_kv_blocks=40, max_batch_num=4)
+    e2.eos_token_id = outs[0][0]
+    assert e2.generate([prompts[0]], SamplingParams(max_new_tokens=16)) == [[outs[0][0]]]
+    assert e2.generate([prompts[0]], SamplingParams(max_new_tokens=3, ignore_eos=True)) == [outs[0][:3]]
