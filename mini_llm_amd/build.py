@@ -46,6 +46,7 @@ LIBRARIES: Dict[str, dict] = {
     "gemm_f32": {"kind": "hip", "sources": ["kernels/gemm_f32.hip"], "headers": ["kernels/common.h"]},
     "gemm_bf16": {"kind": "hip", "sources": ["kernels/gemm_bf16.hip"], "headers": ["kernels/common.h"]},
     "attention": {"kind": "hip", "sources": ["kernels/attention.hip"], "headers": ["kernels/common.h"]},
+    "attention_decode": {"kind": "hip", "sources": ["kernels/attention_decode.hip"], "headers": ["kernels/common.h"]},
     "sampling": {"kind": "hip", "sources": ["kernels/sampling.hip"], "headers": ["kernels/common.h"]},
 }
 

@@ -1,0 +1,243 @@
+// Decode attention over the paged cache for gfx950: one query token per (token, head),
+// its keys split over `nsplit` workgroups so that small batches still fill the chip.
+//
+// Inside a workgroup, LPK lanes share one key: each lane loads 16 bytes of the key row
+// and of the value row (so a wavefront covers 64/LPK whole rows per load instruction),
+// the LPK partial dot products are summed with DPP shuffles, and every lane keeps the
+// running maximum, sum and its slice of the output for the keys of its lane group
+// (recurrence of /root/reference/src/kernels/prefill/flashattention.cu:129-178, in base 2).
+// Groups, wavefronts and splits are merged with the same (m, l, o) rule; the last
+// workgroup to finish a (token, head) pair merges the splits, found through an atomic
+// counter (no workgroup ever waits for another).
+//
+// It stands where the reference has its three-pass decode kernel
+// (/root/reference/src/kernels/decode/paged_attention.cu:58-120); no 1e-6 is added to
+// the denominator.
+#include "common.h"
+
+#define DEC_WAVES 4
+#define DEC_UNROLL 4
+
+template <typename T> struct Vec16;
+template <> struct Vec16<bf16_t> {
+    static constexpr int N = 8;
+    __device__ static void load(const bf16_t* p, float (&v)[8]) { load8(p, v); }
+};
+template <> struct Vec16<float> {
+    static constexpr int N = 4;
+    __device__ static void load(const float* p, float (&v)[4]) {
+        float4 a = *reinterpret_cast<const float4*>(p);
+        v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w;
+    }
+};
+
+template <int N>
+__device__ __forceinline__ void merge_state(float& m, float& l, float (&o)[N], float m2, float l2,
+                                            const float (&o2)[N]) {
+    const float mn = fmaxf(m, m2);
+    if (mn == -INFINITY) return;          // both empty
+    const float a = exp2f(m - mn), b = exp2f(m2 - mn);
+    l = l * a + l2 * b;
+#pragma unroll
+    for (int e = 0; e < N; ++e) o[e] = o[e] * a + o2[e] * b;
+    m = mn;
+}
+
+template <typename T, int LPK>
+__global__ void __launch_bounds__(DEC_WAVES * MLLM_WAVE)
+decode_attention_kernel(const T* __restrict__ q, int q_stride, int q_col,
+                        const T* __restrict__ k_pages, const T* __restrict__ v_pages, int kv_dim,
+                        const int* __restrict__ block_tables, int max_blocks,
+                        const int* __restrict__ token_seq, const int* __restrict__ positions,
+                        int n_heads, int n_kv_heads, int page_size, float scale_log2e, int window,
+                        int nsplit, T* __restrict__ out, int out_stride,
+                        float* __restrict__ ws_o, float* __restrict__ ws_ml, int* __restrict__ counters) {
+    constexpr int EPL = Vec16<T>::N;        // elements per lane
+    constexpr int DH = LPK * EPL;           // head size
+    constexpr int KPW = MLLM_WAVE / LPK;    // keys per wavefront and load instruction
+    __shared__ float sm_m[DEC_WAVES], sm_l[DEC_WAVES];
+    __shared__ float sm_o[DEC_WAVES][DH];
+    __shared__ int sm_last;
+
+    const int pair = blockIdx.x, split = blockIdx.y;
+    const int t = pair / n_heads, h = pair % n_heads;
+    const int hk = h / (n_heads / n_kv_heads);
+    const int wave = threadIdx.x / MLLM_WAVE, lane = threadIdx.x % MLLM_WAVE;
+    const int c = lane % LPK, g = lane / LPK;
+    const int b = token_seq[t], p = positions[t];
+    const int lo = (window > 0 && p - window + 1 > 0) ? p - window + 1 : 0;
+    const int n_keys = p - lo + 1;
+    const int per = (n_keys + nsplit - 1) / nsplit;
+    const int kb = lo + split * per;
+    const int ke = min(p + 1, kb + per);
+    const int* table = block_tables + static_cast<size_t>(b) * max_blocks;
+
+    float qf[EPL];
+    Vec16<T>::load(q + static_cast<size_t>(t) * q_stride + q_col + h * DH + c * EPL, qf);
+#pragma unroll
+    for (int e = 0; e < EPL; ++e) qf[e] *= scale_log2e;
+
+    float m = -INFINITY, l = 0.f, o[EPL];
+#pragma unroll
+    for (int e = 0; e < EPL; ++e) o[e] = 0.f;
+    const size_t col = static_cast<size_t>(hk) * DH + c * EPL;
+
+    for (int j0 = kb + wave * KPW; j0 < ke; j0 += DEC_WAVES * KPW * DEC_UNROLL) {
+        float kf[DEC_UNROLL][EPL], vf[DEC_UNROLL][EPL];
+        bool valid[DEC_UNROLL];
+#pragma unroll
+        for (int u = 0; u < DEC_UNROLL; ++u) {
+            const int j = j0 + u * DEC_WAVES * KPW + g;
+            valid[u] = j < ke;
+            if (valid[u]) {
+                const size_t row = static_cast<size_t>(table[j / page_size]) * page_size + j % page_size;
+                Vec16<T>::load(k_pages + row * kv_dim + col, kf[u]);
+                Vec16<T>::load(v_pages + row * kv_dim + col, vf[u]);
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < DEC_UNROLL; ++u) {
+            float dot = 0.f;
+            if (valid[u]) {
+#pragma unroll
+                for (int e = 0; e < EPL; ++e) dot = fmaf(qf[e], kf[u][e], dot);
+            }
+#pragma unroll
+            for (int off = 1; off < LPK; off <<= 1) dot += __shfl_xor(dot, off, MLLM_WAVE);
+            if (valid[u]) {
+                const float mn = fmaxf(m, dot);
+                const float a = exp2f(m - mn), pj = exp2f(dot - mn);
+                l = l * a + pj;
+#pragma unroll
+                for (int e = 0; e < EPL; ++e) o[e] = o[e] * a + pj * vf[u][e];
+                m = mn;
+            }
+        }
+    }
+    // lane groups of one wavefront
+#pragma unroll
+    for (int off = LPK; off < MLLM_WAVE; off <<= 1) {
+        const float m2 = __shfl_xor(m, off, MLLM_WAVE), l2 = __shfl_xor(l, off, MLLM_WAVE);
+        float o2[EPL];
+#pragma unroll
+        for (int e = 0; e < EPL; ++e) o2[e] = __shfl_xor(o[e], off, MLLM_WAVE);
+        merge_state<EPL>(m, l, o, m2, l2, o2);
+    }
+    // wavefronts of the workgroup
+    if (g == 0) {
+        if (c == 0) { sm_m[wave] = m; sm_l[wave] = l; }
+#pragma unroll
+        for (int e = 0; e < EPL; ++e) sm_o[wave][c * EPL + e] = o[e];
+    }
+    __syncthreads();
+    if (wave == 0 && g == 0) {
+        for (int w = 1; w < DEC_WAVES; ++w) {
+            float o2[EPL];
+#pragma unroll
+            for (int e = 0; e < EPL; ++e) o2[e] = sm_o[w][c * EPL + e];
+            merge_state<EPL>(m, l, o, sm_m[w], sm_l[w], o2);
+        }
+    }
+    T* op = out + static_cast<size_t>(t) * out_stride + h * DH + c * EPL;
+    if (nsplit == 1) {
+        if (wave == 0 && g == 0) {
+            const float inv = 1.0f / l;
+#pragma unroll
+            for (int e = 0; e < EPL; ++e) op[e] = from_float<T>(o[e] * inv);
+        }
+        return;
+    }
+    // partial result of this split
+    const size_t slot = static_cast<size_t>(pair) * nsplit + split;
+    if (wave == 0 && g == 0) {
+#pragma unroll
+        for (int e = 0; e < EPL; ++e) ws_o[slot * DH + c * EPL + e] = o[e];
+        if (c == 0) { ws_ml[slot * 2] = m; ws_ml[slot * 2 + 1] = l; }
+    }
+    __threadfence();
+    __syncthreads();
+    if (threadIdx.x == 0) sm_last = (atomicAdd(&counters[pair], 1) == nsplit - 1) ? 1 : 0;
+    __syncthreads();
+    if (!sm_last) return;
+    __threadfence();
+    if (wave == 0 && g == 0) {
+        float M = -INFINITY, L = 0.f, O[EPL];
+#pragma unroll
+        for (int e = 0; e < EPL; ++e) O[e] = 0.f;
+        for (int s = 0; s < nsplit; ++s) {
+            const size_t sl = static_cast<size_t>(pair) * nsplit + s;
+            const float m2 = __hip_atomic_load(&ws_ml[sl * 2], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            const float l2 = __hip_atomic_load(&ws_ml[sl * 2 + 1], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            float o2[EPL];
+#pragma unroll
+            for (int e = 0; e < EPL; ++e)
+                o2[e] = __hip_atomic_load(&ws_o[sl * DH + c * EPL + e], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            merge_state<EPL>(M, L, O, m2, l2, o2);
+        }
+        const float inv = 1.0f / L;
+#pragma unroll
+        for (int e = 0; e < EPL; ++e) op[e] = from_float<T>(O[e] * inv);
+    }
+    if (threadIdx.x == 0) counters[pair] = 0;     // ready for the next launch
+}
+
+template <typename T>
+static int launch_decode(int lpk, dim3 grid, hipStream_t stream, const T* q, int q_stride, int q_col,
+                         const T* k_pages, const T* v_pages, int kv_dim, const int* block_tables,
+                         int max_blocks, const int* token_seq, const int* positions, int n_heads,
+                         int n_kv_heads, int page_size, float scale_log2e, int window, int nsplit, T* out,
+                         int out_stride, float* ws_o, float* ws_ml, int* counters) {
+#define DEC_CASE(L)                                                                                    \
+    case L:                                                                                            \
+        decode_attention_kernel<T, L><<<grid, DEC_WAVES * MLLM_WAVE, 0, stream>>>(                     \
+            q, q_stride, q_col, k_pages, v_pages, kv_dim, block_tables, max_blocks, token_seq,         \
+            positions, n_heads, n_kv_heads, page_size, scale_log2e, window, nsplit, out, out_stride,   \
+            ws_o, ws_ml, counters);                                                                    \
+        return 0;
+    switch (lpk) {
+        DEC_CASE(2) DEC_CASE(4) DEC_CASE(8) DEC_CASE(16) DEC_CASE(32) DEC_CASE(64)
+        default: return -1;
+    }
+#undef DEC_CASE
+}
+
+extern "C" {
+
+// Number of floats of workspace (partial outputs and their max/sum) for n_q tokens.
+long mllm_decode_attention_ws_floats(int n_q, int n_heads, int head_dim, int nsplit) {
+    return static_cast<long>(n_q) * n_heads * nsplit * (head_dim + 2);
+}
+
+// Returns 0, a HIP error code, or -1 for sizes the kernel refuses: head_dim * element size / 16
+// must be a power of two in [2, 64]. `counters` holds n_q*n_heads ints that are zero before the
+// first launch (the kernel leaves them zero).
+int mllm_decode_attention(const void* q, int q_stride, int q_col, const void* k_pages, const void* v_pages,
+                          int kv_dim, const int* block_tables, int max_blocks, const int* token_seq,
+                          const int* positions, int n_q, int n_heads, int n_kv_heads, int head_dim,
+                          int page_size, float scale, int window, int nsplit, void* out, int out_stride,
+                          float* ws, int* counters, int dtype, hipStream_t stream) {
+    if (n_q <= 0) return 0;
+    const int esz = dtype == MLLM_F32 ? 4 : 2;
+    const int lpk = head_dim * esz / 16;
+    if (head_dim * esz % 16 != 0 || n_heads % n_kv_heads != 0 || nsplit < 1 || nsplit > 65535) return -1;
+    dim3 grid(n_q * n_heads, nsplit);
+    float* ws_o = ws;
+    float* ws_ml = ws + static_cast<size_t>(n_q) * n_heads * nsplit * head_dim;
+    const float sl2 = scale * 1.44269504088896340736f;
+    int rc;
+    if (dtype == MLLM_F32)
+        rc = launch_decode<float>(lpk, grid, stream, (const float*)q, q_stride, q_col, (const float*)k_pages,
+                                  (const float*)v_pages, kv_dim, block_tables, max_blocks, token_seq, positions,
+                                  n_heads, n_kv_heads, page_size, sl2, window, nsplit, (float*)out, out_stride,
+                                  ws_o, ws_ml, counters);
+    else
+        rc = launch_decode<bf16_t>(lpk, grid, stream, (const bf16_t*)q, q_stride, q_col, (const bf16_t*)k_pages,
+                                   (const bf16_t*)v_pages, kv_dim, block_tables, max_blocks, token_seq, positions,
+                                   n_heads, n_kv_heads, page_size, sl2, window, nsplit, (bf16_t*)out, out_stride,
+                                   ws_o, ws_ml, counters);
+    if (rc != 0) return rc;
+    MLLM_LAUNCH_CHECK();
+    return 0;
+}
+
+}  // extern "C"

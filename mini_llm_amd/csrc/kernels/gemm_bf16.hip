@@ -110,6 +110,124 @@ gemm_bf16_mfma(const bf16_t* __restrict__ A, int lda, const bf16_t* __restrict__
     }
 }
 
+
+// ---------------------------------------------------------------------------------------------
+// Few rows (decode): M <= 64. The product is bound by streaming W once, so the grid is
+// one workgroup per 16 output columns and the wavefronts of a workgroup split K
+// (wavefront w takes the 32-wide k steps w, w+NW, ...), each lane loading 16 contiguous
+// bytes of a weight row straight from global memory into the B operand of
+// v_mfma_f32_16x16x32_bf16. The activations (a few KB, shared by all workgroups) are read
+// from L2, or, with LN_FUSED, normalised from the fp32 stream into LDS first: LayerNorm
+// (/root/reference/src/kernels/layernorm.cu:32-49) fused into the product that follows it.
+// Partial sums of the wavefronts are added in LDS in a fixed order.
+// ---------------------------------------------------------------------------------------------
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+template <int MT, bool LN_FUSED>
+__global__ void __launch_bounds__(1024)
+gemm_bf16_skinny(const void* __restrict__ Ain, int lda, const bf16_t* __restrict__ W, int ldw,
+                 const float* __restrict__ bias, void* __restrict__ C, int ldc, int M, int N, int K, int mode,
+                 const float* __restrict__ gamma, const float* __restrict__ beta, float eps) {
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
+    const int tid = threadIdx.x, wave = tid / 64, lane = tid % 64;
+    const int nw = blockDim.x / 64;
+    const int n0 = blockIdx.x * 16;
+    const int row16 = lane % 16, kq = lane / 16;
+    float* red = reinterpret_cast<float*>(smem_raw);                       // [nw][MT][256]
+    bf16_t* a_s = reinterpret_cast<bf16_t*>(smem_raw + static_cast<size_t>(nw) * MT * 256 * sizeof(float));
+    const int a_stride = K + 8;
+
+    if (LN_FUSED) {
+        // one wavefront per row: mean, then variance of the centred values, all in fp32
+        const float* x = static_cast<const float*>(Ain);
+        for (int m = wave; m < 16 * MT; m += nw) {
+            bf16_t* dst = a_s + static_cast<size_t>(m) * a_stride;
+            if (m < M) {
+                const float* xr = x + static_cast<size_t>(m) * lda;
+                float s = 0.f;
+                for (int k = lane; k < K; k += 64) s += xr[k];
+                const float mean = wave_sum(s) / static_cast<float>(K);
+                float q = 0.f;
+                for (int k = lane; k < K; k += 64) { const float c = xr[k] - mean; q += c * c; }
+                const float inv = 1.0f / sqrtf(wave_sum(q) / static_cast<float>(K) + eps);
+                for (int k = lane; k < K; k += 64) {
+                    float v = (xr[k] - mean) * inv * gamma[k];
+                    if (beta) v += beta[k];
+                    dst[k] = float_to_bf16(v);
+                }
+            } else {
+                for (int k = lane; k < K; k += 64) dst[k].bits = 0;
+            }
+        }
+        __syncthreads();
+    }
+
+    f32x4 acc[MT];
+#pragma unroll
+    for (int i = 0; i < MT; ++i) acc[i] = f32x4{0.f, 0.f, 0.f, 0.f};
+    const int n = n0 + row16;
+    const bf16_t* wrow = W + static_cast<size_t>(n < N ? n : 0) * ldw;
+    const bf16_t* A = static_cast<const bf16_t*>(Ain);
+    const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
+
+#pragma unroll 4
+    for (int k0 = wave * 32; k0 < K; k0 += nw * 32) {
+        const int k = k0 + 8 * kq;
+        const bool kin = k < K;
+        bf16x8 b = (kin && n < N) ? *reinterpret_cast<const bf16x8*>(wrow + k) : zero;
+#pragma unroll
+        for (int i = 0; i < MT; ++i) {
+            const int m = i * 16 + row16;
+            bf16x8 a;
+            if (LN_FUSED) a = kin ? *reinterpret_cast<const bf16x8*>(a_s + static_cast<size_t>(m) * a_stride + k) : zero;
+            else a = (kin && m < M) ? *reinterpret_cast<const bf16x8*>(A + static_cast<size_t>(m) * lda + k) : zero;
+            acc[i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, acc[i], 0, 0, 0);
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < MT; ++i)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) red[(static_cast<size_t>(wave) * MT + i) * 256 + r * 64 + lane] = acc[i][r];
+    __syncthreads();
+    // accumulator layout of the 16x16 tile: register r of lane l holds row 4*(l/16) + r, column l%16
+    for (int idx = tid; idx < MT * 256; idx += blockDim.x) {
+        const int i = idx / 256, r = (idx % 256) / 64, l = idx % 64;
+        float v = 0.f;
+        for (int w = 0; w < nw; ++w) v += red[(static_cast<size_t>(w) * MT + i) * 256 + r * 64 + l];
+        const int m = i * 16 + 4 * (l / 16) + r, nn = n0 + l % 16;
+        if (m < M && nn < N) epilogue<bf16_t>(mode, v, bias ? bias[nn] : 0.f, C, static_cast<size_t>(m) * ldc + nn);
+    }
+}
+
+static int skinny_waves(int N, int K) {
+    const int blocks = (N + 15) / 16, steps = (K + 31) / 32;
+    int nw = 16;
+    while (nw > 1 && (nw * 3 > steps || blocks * nw > 4096)) nw >>= 1;
+    return nw;
+}
+
+template <bool LN_FUSED>
+static int launch_skinny(const void* A, int lda, const bf16_t* W, int ldw, const float* bias, void* C, int ldc,
+                         int M, int N, int K, int mode, const float* gamma, const float* beta, float eps,
+                         hipStream_t stream) {
+    const int mt = (M + 15) / 16, nw = skinny_waves(N, K);
+    const dim3 grid((N + 15) / 16), block(nw * 64);
+    size_t smem = static_cast<size_t>(nw) * mt * 256 * sizeof(float);
+    if (LN_FUSED) smem += static_cast<size_t>(16) * mt * (K + 8) * sizeof(bf16_t);
+    if (smem > 64 * 1024) return -2;
+#define SKINNY_CASE(MTV)                                                                                  \
+    case MTV:                                                                                             \
+        gemm_bf16_skinny<MTV, LN_FUSED><<<grid, block, smem, stream>>>(A, lda, W, ldw, bias, C, ldc, M, N, K, \
+                                                                       mode, gamma, beta, eps);           \
+        break;
+    switch (mt) {
+        SKINNY_CASE(1) SKINNY_CASE(2) SKINNY_CASE(3) SKINNY_CASE(4)
+        default: return -2;
+    }
+#undef SKINNY_CASE
+    return 0;
+}
+
 extern "C" {
 
 // Returns 0, a HIP error code, or -1 when K or the row strides are not multiples of 8
@@ -122,7 +240,10 @@ int mllm_gemm_bf16(const void* A, int lda, const void* W, int ldw, const float* 
     const bf16_t* a = static_cast<const bf16_t*>(A);
     const bf16_t* w = static_cast<const bf16_t*>(W);
     auto blocks = [&](int bm, int bn) { return static_cast<long>((M + bm - 1) / bm) * ((N + bn - 1) / bn); };
-    if (M <= 32) {
+    if (M <= 64 && launch_skinny<false>(A, lda, w, ldw, bias, C, ldc, M, N, K, mode, nullptr, nullptr, 0.f,
+                                        stream) == 0) {
+        // few rows: weight-streaming kernel
+    } else if (M <= 32) {
         dim3 grid((N + 127) / 128, (M + 31) / 32);
         gemm_bf16_mfma<1, 4, 1, 1><<<grid, 256, 0, stream>>>(a, lda, w, ldw, bias, C, ldc, M, N, K, mode);
     } else if (blocks(128, 128) >= 512) {
@@ -132,6 +253,22 @@ int mllm_gemm_bf16(const void* A, int lda, const void* W, int ldw, const float* 
         dim3 grid((N + 63) / 64, (M + 63) / 64);
         gemm_bf16_mfma<2, 2, 1, 1><<<grid, 256, 0, stream>>>(a, lda, w, ldw, bias, C, ldc, M, N, K, mode);
     }
+    MLLM_LAUNCH_CHECK();
+    return 0;
+}
+
+// LayerNorm of the fp32 rows x[M,K] fused into the product with W[N,K]: C = epilogue(LN(x) W^T + bias).
+// Returns 0, a HIP error code, -1 for misaligned operands, or -2 when M or K is too large for the
+// fused kernel (the caller then runs the norm and the product separately).
+int mllm_ln_gemm_bf16(const float* x, int ldx, const float* gamma, const float* beta, float eps, const void* W,
+                      int ldw, const float* bias, void* C, int ldc, int M, int N, int K, int mode,
+                      hipStream_t stream) {
+    if (M <= 0 || N <= 0) return 0;
+    if (K % 8 != 0 || ldw % 8 != 0 || (reinterpret_cast<uintptr_t>(W) & 15)) return -1;
+    if (M > 16) return -2;
+    int rc = launch_skinny<true>(x, ldx, static_cast<const bf16_t*>(W), ldw, bias, C, ldc, M, N, K, mode, gamma,
+                                 beta, eps, stream);
+    if (rc != 0) return rc;
     MLLM_LAUNCH_CHECK();
     return 0;
 }

@@ -158,6 +158,44 @@ def linear(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], out: 
     return out
 
 
+def ln_linear(x: torch.Tensor, gamma: torch.Tensor, beta: Optional[torch.Tensor], eps: float,
+              w: torch.Tensor, bias: Optional[torch.Tensor], out: torch.Tensor, epilogue: str = "store") -> torch.Tensor:
+    """out = epilogue(LayerNorm(x) @ w.T + bias) with x the fp32 stream [M,K] and w [N,K].
+
+    For bfloat16 weights and at most 16 rows the norm is fused into the product (one kernel);
+    otherwise the norm and the product run one after the other. Same numerics either way:
+    statistics in fp32, the normalised rows rounded to w's dtype before the product.
+    """
+    _gpu(x, gamma, beta, w, bias, out)
+    M, K = x.shape
+    N = w.shape[0]
+    if w.dtype == torch.bfloat16 and M <= 16 and x.dtype == torch.float32 and x.is_contiguous():
+        _rows2d(w, "w")
+        _rows2d(out, "out")
+        if w.shape[1] != K or gamma.numel() != K or gamma.dtype != torch.float32:
+            raise KernelError(f"ln_linear: x is {tuple(x.shape)}, w is {tuple(w.shape)}, gamma {tuple(gamma.shape)}")
+        if beta is not None and (beta.numel() != K or beta.dtype != torch.float32):
+            raise KernelError("ln_linear: beta must be fp32 [K]")
+        if epilogue not in EPILOGUES:
+            raise KernelError(f"unknown epilogue '{epilogue}'")
+        want = torch.float32 if epilogue in ("add_residual", "store_f32") else w.dtype
+        if out.shape != (M, N) or out.dtype != want:
+            raise KernelError(f"ln_linear({epilogue}): out must be [{M}, {N}] {want}")
+        if bias is not None and (bias.dtype != torch.float32 or bias.numel() != N or not bias.is_contiguous()):
+            raise KernelError(f"bias must be contiguous fp32 [{N}]")
+        lib = load_library("gemm_bf16")
+        rc = lib.mllm_ln_gemm_bf16(_p(x), x.stride(0), _p(gamma), _p(beta), ctypes.c_float(eps), _p(w),
+                                   w.stride(0), _p(bias), _p(out), out.stride(0), M, N, K, EPILOGUES[epilogue],
+                                   _stream())
+        if rc == 0:
+            return out
+        if rc != -2:
+            _check(rc, "ln_linear")
+    h = torch.empty((M, K), dtype=w.dtype, device=x.device)
+    layernorm(x, gamma, beta, eps, h)
+    return linear(h, w, bias, out, epilogue)
+
+
 def kv_append(src: torch.Tensor, k_col: int, v_col: int, kv_dim: int, k_pages: torch.Tensor,
               v_pages: torch.Tensor, slots: torch.Tensor) -> None:
     """Copies columns [k_col, k_col+kv_dim) and [v_col, v_col+kv_dim) of each row of ``src``
@@ -213,12 +251,42 @@ def paged_attention(q: torch.Tensor, q_col: int, n_heads: int, n_kv_heads: int, 
     esz = q.element_size()
     if (q.stride(0) * esz) % 16 or (q_col * esz) % 16 or (head_dim * esz) % 16 or q.data_ptr() % 16:
         raise KernelError("query rows and heads must be 16-byte aligned")
+    lpk = head_dim * esz // 16
+    if max_q_len == 1 and lpk >= 2 and (lpk & (lpk - 1)) == 0:
+        # every query is a single decoded token: split its keys over workgroups
+        pairs = T * n_heads
+        nsplit = max(1, min(16, 1024 // pairs, -(-max(max_ctx_len, 1) // 64)))
+        ws, counters = _decode_workspace(q.device, pairs, nsplit, head_dim)
+        lib = load_library("attention_decode")
+        _check(lib.mllm_decode_attention(
+            _p(q), q.stride(0), q_col, _p(k_pages), _p(v_pages), kv_dim, _p(block_tables), block_tables.shape[1],
+            _p(token_seq), _p(positions), T, n_heads, n_kv_heads, head_dim, page_size, ctypes.c_float(scale),
+            int(window or 0), nsplit, _p(out), out.stride(0), _p(ws), _p(counters), _dt(q), _stream()),
+            "decode_attention")
+        return out
     lib = load_library("attention")
     _check(lib.mllm_paged_attention_generic(
         _p(q), q.stride(0), q_col, _p(k_pages), _p(v_pages), kv_dim, _p(block_tables), block_tables.shape[1],
         _p(token_seq), _p(positions), T, n_heads, n_kv_heads, head_dim, page_size, ctypes.c_float(scale),
         int(window or 0), _p(out), out.stride(0), _dt(q), _stream()), "paged_attention")
     return out
+
+
+_DECODE_WS = {}
+
+
+def _decode_workspace(device, pairs: int, nsplit: int, head_dim: int):
+    """Scratch of the split decode attention: partial outputs and a zeroed counter per
+    (token, head). It is kept per device and only ever grows; launches on one stream use it
+    one after the other."""
+    need_f = pairs * nsplit * (head_dim + 2)
+    ws, counters = _DECODE_WS.get(device, (None, None))
+    if ws is None or ws.numel() < need_f:
+        ws = torch.empty(max(need_f, 1 << 16), dtype=torch.float32, device=device)
+    if counters is None or counters.numel() < pairs:
+        counters = torch.zeros(max(pairs, 4096), dtype=torch.int32, device=device)
+    _DECODE_WS[device] = (ws, counters)
+    return ws, counters
 
 
 def argmax(logits: torch.Tensor, out: torch.Tensor) -> torch.Tensor:

@@ -7,7 +7,7 @@ import torch
 
 from ..cache.manager import KVCacheSpec, KVCacheView
 from ..kernels import ops
-from .base import Mixer, ParamSpec, PositionEncoding, register_mixer
+from .base import Mixer, NormedInput, ParamSpec, PositionEncoding, register_mixer
 from .linear import Linear
 
 
@@ -22,6 +22,8 @@ class CausalSelfAttention(Mixer):
     Column layout of qkv: queries [0, H*dh), keys [H*dh, H*dh + Hkv*dh), values after
     them; head h at h*dh (/root/reference/src/kernels/prefill/append_kv.cu:31-33).
     """
+
+    accepts_normed_input = True
 
     def __init__(self, hidden_size: int, n_heads: int, n_kv_heads: int, head_dim: int, scale: float,
                  window: Optional[int], bias: bool, weight_layout: str, names: Dict[str, str],
@@ -50,7 +52,10 @@ class CausalSelfAttention(Mixer):
     def forward(self, h, ctx, cache_view: KVCacheView, x, write: bool = True) -> None:
         T = h.shape[0]
         qkv = torch.empty((T, self.q_dim + 2 * self.kv_dim), dtype=self.dtype, device=h.device)
-        self.qkv(h, qkv, "store")
+        if isinstance(h, NormedInput):
+            h.linear(self.qkv, qkv, "store")
+        else:
+            self.qkv(h, qkv, "store")
         if self.position is not None:
             self.position.in_mixer(qkv, self, ctx)
         g = cache_view.group

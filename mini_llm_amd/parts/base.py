@@ -53,8 +53,36 @@ class Norm(Part):
     def forward(self, x: torch.Tensor, rows: Optional[torch.Tensor] = None) -> torch.Tensor:
         raise NotImplementedError
 
+    def linear(self, x: torch.Tensor, lin, out: torch.Tensor, epilogue: str = "store") -> torch.Tensor:
+        """out = epilogue(lin(norm(x))). A norm with a fused kernel overrides this."""
+        return lin(self.forward(x), out, epilogue)
+
+
+class NormedInput:
+    """The input of a sub-layer as (stream, norm), not yet normalised. A part that sets
+    ``accepts_normed_input`` receives this instead of a tensor and can let its first linear
+    map absorb the norm (``linear``); ``tensor()`` gives the normalised activation."""
+
+    def __init__(self, norm: "Norm", x: torch.Tensor):
+        self.norm, self.x = norm, x
+        self._h = None
+        self.shape = x.shape
+        self.device = x.device
+
+    def tensor(self) -> torch.Tensor:
+        if self._h is None:
+            self._h = self.norm.forward(self.x)
+        return self._h
+
+    def linear(self, lin, out: torch.Tensor, epilogue: str = "store") -> torch.Tensor:
+        if self._h is not None:
+            return lin(self._h, out, epilogue)
+        return self.norm.linear(self.x, lin, out, epilogue)
+
 
 class Mixer(Part):
+    accepts_normed_input = False     # True: forward() takes a NormedInput instead of a tensor
+
     def cache_spec(self):
         """KVCacheSpec, StateCacheSpec or None."""
         return None
@@ -64,6 +92,8 @@ class Mixer(Part):
 
 
 class FeedForward(Part):
+    accepts_normed_input = False
+
     def forward(self, h, ctx, x) -> None:
         raise NotImplementedError
 

@@ -3,7 +3,7 @@ from __future__ import annotations
 
 from typing import List, Sequence
 
-from .base import Block, FeedForward, Mixer, Norm, ParamSpec, register_block
+from .base import Block, FeedForward, Mixer, Norm, NormedInput, ParamSpec, register_block
 
 
 @register_block("pre_norm")
@@ -30,7 +30,7 @@ class PreNormBlock(Block):
         return self.mixer.cache_spec()
 
     def forward(self, x, ctx, cache_view, write: bool = True) -> None:
-        h = self.norm1.forward(x)
+        h = NormedInput(self.norm1, x) if self.mixer.accepts_normed_input else self.norm1.forward(x)
         self.mixer.forward(h, ctx, cache_view, x, write)
-        h = self.norm2.forward(x)
+        h = NormedInput(self.norm2, x) if self.feed_forward.accepts_normed_input else self.norm2.forward(x)
         self.feed_forward.forward(h, ctx, x)

@@ -5,7 +5,7 @@ from typing import Dict, List
 
 import torch
 
-from .base import FeedForward, ParamSpec, register_feed_forward
+from .base import FeedForward, NormedInput, ParamSpec, register_feed_forward
 from .linear import Linear
 
 _ACT_EPILOGUE = {"gelu_tanh": "gelu_tanh", "gelu_erf": "gelu_erf"}
@@ -17,6 +17,8 @@ class DenseMLP(FeedForward):
     product and the residual add into the second
     (/root/reference/src/model/gpt2_model.cu:345-363). Activations: tanh-GELU
     (/root/reference/src/kernels/gelu.cu:7-9) and exact erf-GELU."""
+
+    accepts_normed_input = True
 
     def __init__(self, hidden_size: int, inner_size: int, activation: str, bias: bool, weight_layout: str,
                  names: Dict[str, str], dtype, device, init_std: float = 0.02, out_init_std: float = 0.02):
@@ -33,5 +35,8 @@ class DenseMLP(FeedForward):
 
     def forward(self, h, ctx, x) -> None:
         inner = torch.empty((h.shape[0], self.inner_size), dtype=self.dtype, device=h.device)
-        self.up(h, inner, _ACT_EPILOGUE[self.activation])
+        if isinstance(h, NormedInput):
+            h.linear(self.up, inner, _ACT_EPILOGUE[self.activation])
+        else:
+            self.up(h, inner, _ACT_EPILOGUE[self.activation])
         self.down(inner, x, "add_residual")

@@ -58,6 +58,11 @@ def linear(a, w, bias, out, epilogue="store"):
     return out
 
 
+def ln_linear(x, gamma, beta, eps, w, bias, out, epilogue="store"):
+    h = layernorm(x, gamma, beta, eps, torch.empty(x.shape, dtype=w.dtype))
+    return linear(h, w, bias, out, epilogue)
+
+
 def kv_append(src, k_col, v_col, kv_dim, k_pages, v_pages, slots):
     T = src.shape[0]
     s = slots[:T].long()
@@ -110,7 +115,7 @@ def sample(logits, temperature, u, out):
     return out
 
 
-_NAMES = ("embed", "layernorm", "linear", "kv_append", "paged_attention", "argmax", "sample")
+_NAMES = ("embed", "layernorm", "linear", "ln_linear", "kv_append", "paged_attention", "argmax", "sample")
 
 
 def install(monkeypatch):

@@ -112,6 +112,50 @@ def test_linear(ops, dtype, M, N, K, epi):
     assert (out.cpu().double() - ref).abs().max().item() <= tol
 
 
+@pytest.mark.parametrize("M", [1, 8, 16, 17, 48, 64])
+@pytest.mark.parametrize("N,K", [(2304, 768), (768, 3072), (1000, 96), (50257, 768), (72, 1600)])
+def test_linear_bf16_few_rows(ops, M, N, K):
+    """The weight-streaming kernel of decode steps (M <= 64), every wavefront count and m-tile count."""
+    g = torch.Generator().manual_seed(M + N + K)
+    a = _rand((M, K), torch.bfloat16, g)
+    w = _rand((N, K), torch.bfloat16, g, std=1.0 / math.sqrt(K))
+    bias = 0.5 * _rand((N,), torch.float32, g)
+    for epi in ("store_f32", "add_residual", "gelu_tanh"):
+        f32_out = epi != "gelu_tanh"
+        out0 = _rand((M, N), torch.float32 if f32_out else torch.bfloat16, g)
+        out = out0.clone().to(DEV)
+        ops.linear(a.to(DEV), w.to(DEV), bias.to(DEV), out, epi)
+        ref = plain_ops.linear(a, w, bias, out0.double().clone(), epi)
+        err = (out.cpu().double() - ref).abs().max().item()
+        assert err <= (2e-5 + 2e-5 * math.sqrt(K) if f32_out else 4e-2), (epi, err)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("M,N,K", [(1, 2304, 768), (8, 3072, 768), (16, 320, 96), (5, 200, 1600), (17, 96, 64),
+                                   (3, 64, 4096)])
+@pytest.mark.parametrize("epi", ["store", "gelu_tanh", "gelu_erf", "store_f32"])
+def test_ln_linear(ops, dtype, M, N, K, epi):
+    """LayerNorm fused into the product (bf16, few rows) and its unfused form give the plain result."""
+    g = torch.Generator().manual_seed(M * 7 + N + K)
+    x = _rand((M, K), torch.float32, g, std=2.0) + 0.3
+    gamma = 1 + 0.1 * _rand((K,), torch.float32, g)
+    beta = 0.1 * _rand((K,), torch.float32, g)
+    w = _rand((N, K), dtype, g, std=1.0 / math.sqrt(K))
+    bias = 0.5 * _rand((N,), torch.float32, g)
+    odt = torch.float32 if epi == "store_f32" else dtype
+    out = torch.zeros(M, N, dtype=odt, device=DEV)
+    ops.ln_linear(x.to(DEV), gamma.to(DEV), beta.to(DEV), 1e-5, w.to(DEV), bias.to(DEV), out, epi)
+    h = plain_ops.layernorm(x, gamma, beta, 1e-5, torch.empty(M, K, dtype=dtype))     # rounded as the kernel rounds
+    ref = plain_ops.linear(h, w, bias, torch.zeros(M, N, dtype=torch.float64), epi)
+    tol = 3e-5 if dtype == torch.float32 else (2e-2 if epi == "store_f32" else 4e-2)
+    assert (out.cpu().double() - ref).abs().max().item() <= tol
+    out2 = torch.zeros(M, N, dtype=odt, device=DEV)
+    ops.ln_linear(x.to(DEV), gamma.to(DEV), None, 1e-5, w.to(DEV), None, out2, epi)
+    h = plain_ops.layernorm(x, gamma, None, 1e-5, torch.empty(M, K, dtype=dtype))
+    ref = plain_ops.linear(h, w, None, torch.zeros(M, N, dtype=torch.float64), epi)
+    assert (out2.cpu().double() - ref).abs().max().item() <= tol
+
+
 def test_linear_fp32_is_true_fp32(ops):
     """Values that bf16 or tf32 inputs would destroy: 1 + 2^-20 differs from 1 only in true fp32."""
     K = 64
@@ -207,6 +251,24 @@ def test_paged_attention_mixed_batch(ops, dtype, H, Hkv, dh, page):
     seqs = [(0, 37), (130, 1), (64, 2), (5, 70), (0, 1), (199, 1)]
     out, ref = _attention_case(ops, dtype, H, Hkv, dh, page, seqs, 0, g)
     assert torch.isfinite(out).all()
+    assert (out - ref).abs().max() <= _tol(dtype, 2)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("H,Hkv,dh,page", [(12, 12, 64, 16), (4, 4, 16, 4), (3, 3, 32, 8), (6, 2, 128, 16),
+                                           (2, 1, 256, 64), (5, 5, 48, 16)])
+@pytest.mark.parametrize("window", [0, 33])
+def test_paged_attention_decode_only(ops, dtype, H, Hkv, dh, page, window):
+    """Every query a single token: the split-key decode kernel (power-of-two head sizes; others
+    fall back), contexts from 1 token to a thousand so that splits are empty, partial and full."""
+    g = torch.Generator().manual_seed(H * 10 + dh + window)
+    for seqs in ([(0, 1)], [(1023, 1), (0, 1), (63, 1), (64, 1), (500, 1), (17, 1), (129, 1), (255, 1)],
+                 [(s, 1) for s in range(3, 300, 7)]):
+        out, ref = _attention_case(ops, dtype, H, Hkv, dh, page, seqs, window, g)
+        assert torch.isfinite(out).all()
+        assert (out - ref).abs().max() <= _tol(dtype, 2)
+    # run twice in a row: the split counters must be back at zero
+    out, ref = _attention_case(ops, dtype, H, Hkv, dh, page, [(700, 1), (2, 1)], window, g)
     assert (out - ref).abs().max() <= _tol(dtype, 2)
 
 
