@@ -41,6 +41,8 @@ def _rt():
         "mllm_cache_length": (i, [vp, i64]),
         "mllm_cache_state_slot": (i, [vp, i64]),
         "mllm_cache_block_table": (i, [vp, i64, i, ctypes.c_void_p, i]),
+        "mllm_cache_fill_step_common": (i, [vp] * 3 + [i] + [vp] * 6),
+        "mllm_cache_fill_step_group": (i, [vp, vp, vp, i, i, i, vp, vp]),
         "mllm_cache_free_pages": (i, [vp, i]),
         "mllm_cache_total_pages": (i, [vp, i]),
         "mllm_cache_free_state_slots": (i, [vp]),
@@ -164,6 +166,26 @@ class CacheManager:
         if n < 0:
             raise KeyError(f"request {rid} is not registered")
         return out[:min(n, out.shape[0])]
+
+    def fill_step_common(self, ids: np.ndarray, n_tokens: np.ndarray, positions, token_seq, cu_q, starts,
+                         ctx_len, state_slots) -> None:
+        """Fills the step's group-independent int32 index arrays (numpy views) in one native call."""
+        rc = self._lib.mllm_cache_fill_step_common(
+            self._h, ids.ctypes.data, n_tokens.ctypes.data, len(ids), positions.ctypes.data,
+            token_seq.ctypes.data, cu_q.ctypes.data, starts.ctypes.data, ctx_len.ctypes.data,
+            state_slots.ctypes.data)
+        if rc != 0:
+            raise KeyError(f"request {int(ids[-rc - 1])} is not registered")
+
+    def fill_step_group(self, ids: np.ndarray, n_tokens: np.ndarray, group: int, max_blocks: int,
+                        tables, slots) -> None:
+        """Fills one group's block tables [n, max_blocks] and per-token page rows."""
+        rc = self._lib.mllm_cache_fill_step_group(
+            self._h, ids.ctypes.data, n_tokens.ctypes.data, len(ids), group, max_blocks,
+            tables.ctypes.data, slots.ctypes.data)
+        if rc != 0:
+            raise KeyError(f"request {int(ids[-rc - 1])}: not registered, no pages reserved for its tokens "
+                           f"(reserve before the step), or more than {max_blocks} blocks")
 
     def free_pages(self, group: int = 0) -> int:
         return self._lib.mllm_cache_free_pages(self._h, group)

@@ -15,7 +15,7 @@
 // the denominator.
 #include "common.h"
 
-#define DEC_WAVES 4
+#define DEC_MAX_WAVES 16
 #define DEC_UNROLL 4
 
 template <typename T> struct Vec16;
@@ -44,7 +44,7 @@ __device__ __forceinline__ void merge_state(float& m, float& l, float (&o)[N], f
 }
 
 template <typename T, int LPK>
-__global__ void __launch_bounds__(DEC_WAVES * MLLM_WAVE)
+__global__ void __launch_bounds__(DEC_MAX_WAVES * MLLM_WAVE)
 decode_attention_kernel(const T* __restrict__ q, int q_stride, int q_col,
                         const T* __restrict__ k_pages, const T* __restrict__ v_pages, int kv_dim,
                         const int* __restrict__ block_tables, int max_blocks,
@@ -55,9 +55,10 @@ decode_attention_kernel(const T* __restrict__ q, int q_stride, int q_col,
     constexpr int EPL = Vec16<T>::N;        // elements per lane
     constexpr int DH = LPK * EPL;           // head size
     constexpr int KPW = MLLM_WAVE / LPK;    // keys per wavefront and load instruction
-    __shared__ float sm_m[DEC_WAVES], sm_l[DEC_WAVES];
-    __shared__ float sm_o[DEC_WAVES][DH];
+    __shared__ float sm_m[DEC_MAX_WAVES], sm_l[DEC_MAX_WAVES];
+    __shared__ float sm_o[DEC_MAX_WAVES][DH];
     __shared__ int sm_last;
+    const int n_waves = blockDim.x / MLLM_WAVE;
 
     const int pair = blockIdx.x, split = blockIdx.y;
     const int t = pair / n_heads, h = pair % n_heads;
@@ -71,6 +72,9 @@ decode_attention_kernel(const T* __restrict__ q, int q_stride, int q_col,
     const int kb = lo + split * per;
     const int ke = min(p + 1, kb + per);
     const int* table = block_tables + static_cast<size_t>(b) * max_blocks;
+    // pages of a power-of-two size are addressed with a shift and a mask
+    const bool pow2 = (page_size & (page_size - 1)) == 0;
+    const int shift = pow2 ? __ffs(page_size) - 1 : 0;
 
     float qf[EPL];
     Vec16<T>::load(q + static_cast<size_t>(t) * q_stride + q_col + h * DH + c * EPL, qf);
@@ -82,15 +86,16 @@ decode_attention_kernel(const T* __restrict__ q, int q_stride, int q_col,
     for (int e = 0; e < EPL; ++e) o[e] = 0.f;
     const size_t col = static_cast<size_t>(hk) * DH + c * EPL;
 
-    for (int j0 = kb + wave * KPW; j0 < ke; j0 += DEC_WAVES * KPW * DEC_UNROLL) {
+    for (int j0 = kb + wave * KPW; j0 < ke; j0 += n_waves * KPW * DEC_UNROLL) {
         float kf[DEC_UNROLL][EPL], vf[DEC_UNROLL][EPL];
         bool valid[DEC_UNROLL];
 #pragma unroll
         for (int u = 0; u < DEC_UNROLL; ++u) {
-            const int j = j0 + u * DEC_WAVES * KPW + g;
+            const int j = j0 + u * n_waves * KPW + g;
             valid[u] = j < ke;
             if (valid[u]) {
-                const size_t row = static_cast<size_t>(table[j / page_size]) * page_size + j % page_size;
+                const size_t row = pow2 ? ((static_cast<size_t>(table[j >> shift]) << shift) + (j & (page_size - 1)))
+                                        : (static_cast<size_t>(table[j / page_size]) * page_size + j % page_size);
                 Vec16<T>::load(k_pages + row * kv_dim + col, kf[u]);
                 Vec16<T>::load(v_pages + row * kv_dim + col, vf[u]);
             }
@@ -114,30 +119,34 @@ decode_attention_kernel(const T* __restrict__ q, int q_stride, int q_col,
             }
         }
     }
-    // lane groups of one wavefront
+    // Merges the states of all lane groups and wavefronts; the result is valid in lane group 0
+    // of wavefront 0.
+    auto block_merge = [&]() {
 #pragma unroll
-    for (int off = LPK; off < MLLM_WAVE; off <<= 1) {
-        const float m2 = __shfl_xor(m, off, MLLM_WAVE), l2 = __shfl_xor(l, off, MLLM_WAVE);
-        float o2[EPL];
-#pragma unroll
-        for (int e = 0; e < EPL; ++e) o2[e] = __shfl_xor(o[e], off, MLLM_WAVE);
-        merge_state<EPL>(m, l, o, m2, l2, o2);
-    }
-    // wavefronts of the workgroup
-    if (g == 0) {
-        if (c == 0) { sm_m[wave] = m; sm_l[wave] = l; }
-#pragma unroll
-        for (int e = 0; e < EPL; ++e) sm_o[wave][c * EPL + e] = o[e];
-    }
-    __syncthreads();
-    if (wave == 0 && g == 0) {
-        for (int w = 1; w < DEC_WAVES; ++w) {
+        for (int off = LPK; off < MLLM_WAVE; off <<= 1) {
+            const float m2 = __shfl_xor(m, off, MLLM_WAVE), l2 = __shfl_xor(l, off, MLLM_WAVE);
             float o2[EPL];
 #pragma unroll
-            for (int e = 0; e < EPL; ++e) o2[e] = sm_o[w][c * EPL + e];
-            merge_state<EPL>(m, l, o, sm_m[w], sm_l[w], o2);
+            for (int e = 0; e < EPL; ++e) o2[e] = __shfl_xor(o[e], off, MLLM_WAVE);
+            merge_state<EPL>(m, l, o, m2, l2, o2);
         }
-    }
+        __syncthreads();                      // earlier readers of the LDS arrays are done
+        if (g == 0) {
+            if (c == 0) { sm_m[wave] = m; sm_l[wave] = l; }
+#pragma unroll
+            for (int e = 0; e < EPL; ++e) sm_o[wave][c * EPL + e] = o[e];
+        }
+        __syncthreads();
+        if (wave == 0 && g == 0) {
+            for (int w = 1; w < n_waves; ++w) {
+                float o2[EPL];
+#pragma unroll
+                for (int e = 0; e < EPL; ++e) o2[e] = sm_o[w][c * EPL + e];
+                merge_state<EPL>(m, l, o, sm_m[w], sm_l[w], o2);
+            }
+        }
+    };
+    block_merge();
     T* op = out + static_cast<size_t>(t) * out_stride + h * DH + c * EPL;
     if (nsplit == 1) {
         if (wave == 0 && g == 0) {
@@ -160,36 +169,42 @@ decode_attention_kernel(const T* __restrict__ q, int q_stride, int q_col,
     __syncthreads();
     if (!sm_last) return;
     __threadfence();
-    if (wave == 0 && g == 0) {
-        float M = -INFINITY, L = 0.f, O[EPL];
+    // Last workgroup of this (token, head): lane group G takes split G (all loads in flight at
+    // once), then the same merge as above.
+    m = -INFINITY; l = 0.f;
 #pragma unroll
-        for (int e = 0; e < EPL; ++e) O[e] = 0.f;
-        for (int s = 0; s < nsplit; ++s) {
-            const size_t sl = static_cast<size_t>(pair) * nsplit + s;
+    for (int e = 0; e < EPL; ++e) o[e] = 0.f;
+    for (int s0 = 0; s0 < nsplit; s0 += n_waves * KPW) {
+        const int sidx = s0 + wave * KPW + g;
+        if (sidx < nsplit) {
+            const size_t sl = static_cast<size_t>(pair) * nsplit + sidx;
             const float m2 = __hip_atomic_load(&ws_ml[sl * 2], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             const float l2 = __hip_atomic_load(&ws_ml[sl * 2 + 1], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             float o2[EPL];
 #pragma unroll
             for (int e = 0; e < EPL; ++e)
                 o2[e] = __hip_atomic_load(&ws_o[sl * DH + c * EPL + e], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            merge_state<EPL>(M, L, O, m2, l2, o2);
+            merge_state<EPL>(m, l, o, m2, l2, o2);
         }
-        const float inv = 1.0f / L;
+    }
+    block_merge();
+    if (wave == 0 && g == 0) {
+        const float inv = 1.0f / l;
 #pragma unroll
-        for (int e = 0; e < EPL; ++e) op[e] = from_float<T>(O[e] * inv);
+        for (int e = 0; e < EPL; ++e) op[e] = from_float<T>(o[e] * inv);
     }
     if (threadIdx.x == 0) counters[pair] = 0;     // ready for the next launch
 }
 
 template <typename T>
-static int launch_decode(int lpk, dim3 grid, hipStream_t stream, const T* q, int q_stride, int q_col,
+static int launch_decode(int lpk, dim3 grid, int waves, hipStream_t stream, const T* q, int q_stride, int q_col,
                          const T* k_pages, const T* v_pages, int kv_dim, const int* block_tables,
                          int max_blocks, const int* token_seq, const int* positions, int n_heads,
                          int n_kv_heads, int page_size, float scale_log2e, int window, int nsplit, T* out,
                          int out_stride, float* ws_o, float* ws_ml, int* counters) {
 #define DEC_CASE(L)                                                                                    \
     case L:                                                                                            \
-        decode_attention_kernel<T, L><<<grid, DEC_WAVES * MLLM_WAVE, 0, stream>>>(                     \
+        decode_attention_kernel<T, L><<<grid, waves * MLLM_WAVE, 0, stream>>>(                     \
             q, q_stride, q_col, k_pages, v_pages, kv_dim, block_tables, max_blocks, token_seq,         \
             positions, n_heads, n_kv_heads, page_size, scale_log2e, window, nsplit, out, out_stride,   \
             ws_o, ws_ml, counters);                                                                    \
@@ -214,24 +229,25 @@ long mllm_decode_attention_ws_floats(int n_q, int n_heads, int head_dim, int nsp
 int mllm_decode_attention(const void* q, int q_stride, int q_col, const void* k_pages, const void* v_pages,
                           int kv_dim, const int* block_tables, int max_blocks, const int* token_seq,
                           const int* positions, int n_q, int n_heads, int n_kv_heads, int head_dim,
-                          int page_size, float scale, int window, int nsplit, void* out, int out_stride,
-                          float* ws, int* counters, int dtype, hipStream_t stream) {
+                          int page_size, float scale, int window, int nsplit, int waves, void* out,
+                          int out_stride, float* ws, int* counters, int dtype, hipStream_t stream) {
     if (n_q <= 0) return 0;
     const int esz = dtype == MLLM_F32 ? 4 : 2;
     const int lpk = head_dim * esz / 16;
-    if (head_dim * esz % 16 != 0 || n_heads % n_kv_heads != 0 || nsplit < 1 || nsplit > 65535) return -1;
+    if (head_dim * esz % 16 != 0 || n_heads % n_kv_heads != 0 || nsplit < 1 || nsplit > 65535 ||
+        waves < 1 || waves > DEC_MAX_WAVES) return -1;
     dim3 grid(n_q * n_heads, nsplit);
     float* ws_o = ws;
     float* ws_ml = ws + static_cast<size_t>(n_q) * n_heads * nsplit * head_dim;
     const float sl2 = scale * 1.44269504088896340736f;
     int rc;
     if (dtype == MLLM_F32)
-        rc = launch_decode<float>(lpk, grid, stream, (const float*)q, q_stride, q_col, (const float*)k_pages,
+        rc = launch_decode<float>(lpk, grid, waves, stream, (const float*)q, q_stride, q_col, (const float*)k_pages,
                                   (const float*)v_pages, kv_dim, block_tables, max_blocks, token_seq, positions,
                                   n_heads, n_kv_heads, page_size, sl2, window, nsplit, (float*)out, out_stride,
                                   ws_o, ws_ml, counters);
     else
-        rc = launch_decode<bf16_t>(lpk, grid, stream, (const bf16_t*)q, q_stride, q_col, (const bf16_t*)k_pages,
+        rc = launch_decode<bf16_t>(lpk, grid, waves, stream, (const bf16_t*)q, q_stride, q_col, (const bf16_t*)k_pages,
                                    (const bf16_t*)v_pages, kv_dim, block_tables, max_blocks, token_seq, positions,
                                    n_heads, n_kv_heads, page_size, sl2, window, nsplit, (bf16_t*)out, out_stride,
                                    ws_o, ws_ml, counters);

@@ -34,20 +34,43 @@ __global__ void layernorm_kernel(const float* __restrict__ x, const int* __restr
     const int src = rows ? rows[r] : r;
     const float* xr = x + static_cast<size_t>(src) * D;
     OutT* yr = y + static_cast<size_t>(r) * D;
+    // Up to LN_REGS elements per thread stay in registers (one pass over memory); rows longer
+    // than blockDim * LN_REGS read the remainder again.
+    constexpr int LN_REGS = 8;
+    float v[LN_REGS];
     float s = 0.f;
-    for (int d = threadIdx.x; d < D; d += blockDim.x) s += xr[d];
+#pragma unroll
+    for (int u = 0; u < LN_REGS; ++u) {
+        const int d = threadIdx.x + u * blockDim.x;
+        v[u] = d < D ? xr[d] : 0.f;
+        s += v[u];
+    }
+    for (int d = threadIdx.x + LN_REGS * blockDim.x; d < D; d += blockDim.x) s += xr[d];
     const float mean = block_sum(s, scratch) / static_cast<float>(D);
     float q = 0.f;
-    for (int d = threadIdx.x; d < D; d += blockDim.x) {
-        float c = xr[d] - mean;
+#pragma unroll
+    for (int u = 0; u < LN_REGS; ++u) {
+        if (threadIdx.x + u * blockDim.x < D) { const float c = v[u] - mean; q += c * c; }
+    }
+    for (int d = threadIdx.x + LN_REGS * blockDim.x; d < D; d += blockDim.x) {
+        const float c = xr[d] - mean;
         q += c * c;
     }
     const float var = block_sum(q, scratch) / static_cast<float>(D);
     const float inv = 1.0f / sqrtf(var + eps);
-    for (int d = threadIdx.x; d < D; d += blockDim.x) {
-        float v = (xr[d] - mean) * inv * gamma[d];
-        if (beta) v += beta[d];
-        yr[d] = from_float<OutT>(v);
+#pragma unroll
+    for (int u = 0; u < LN_REGS; ++u) {
+        const int d = threadIdx.x + u * blockDim.x;
+        if (d < D) {
+            float o = (v[u] - mean) * inv * gamma[d];
+            if (beta) o += beta[d];
+            yr[d] = from_float<OutT>(o);
+        }
+    }
+    for (int d = threadIdx.x + LN_REGS * blockDim.x; d < D; d += blockDim.x) {
+        float o = (xr[d] - mean) * inv * gamma[d];
+        if (beta) o += beta[d];
+        yr[d] = from_float<OutT>(o);
     }
 }
 

@@ -143,17 +143,44 @@ gemm_bf16_skinny(const void* __restrict__ Ain, int lda, const bf16_t* __restrict
         for (int m = wave; m < 16 * MT; m += nw) {
             bf16_t* dst = a_s + static_cast<size_t>(m) * a_stride;
             if (m < M) {
-                const float* xr = x + static_cast<size_t>(m) * lda;
+                // the row lives in registers: one pass over memory (K <= 2048, K % 4 == 0)
+                const float4* xr = reinterpret_cast<const float4*>(x + static_cast<size_t>(m) * lda);
+                const int nq = K / 4;
+                float4 v[8];
                 float s = 0.f;
-                for (int k = lane; k < K; k += 64) s += xr[k];
+#pragma unroll
+                for (int u = 0; u < 8; ++u) {
+                    const int i = lane + 64 * u;
+                    v[u] = i < nq ? xr[i] : make_float4(0.f, 0.f, 0.f, 0.f);
+                    s += (v[u].x + v[u].y) + (v[u].z + v[u].w);
+                }
                 const float mean = wave_sum(s) / static_cast<float>(K);
                 float q = 0.f;
-                for (int k = lane; k < K; k += 64) { const float c = xr[k] - mean; q += c * c; }
+#pragma unroll
+                for (int u = 0; u < 8; ++u) {
+                    if (lane + 64 * u < nq) {
+                        const float a = v[u].x - mean, b = v[u].y - mean, c = v[u].z - mean, d = v[u].w - mean;
+                        q += (a * a + b * b) + (c * c + d * d);
+                    }
+                }
                 const float inv = 1.0f / sqrtf(wave_sum(q) / static_cast<float>(K) + eps);
-                for (int k = lane; k < K; k += 64) {
-                    float v = (xr[k] - mean) * inv * gamma[k];
-                    if (beta) v += beta[k];
-                    dst[k] = float_to_bf16(v);
+                const float4* g4 = reinterpret_cast<const float4*>(gamma);
+                const float4* b4 = reinterpret_cast<const float4*>(beta);
+#pragma unroll
+                for (int u = 0; u < 8; ++u) {
+                    const int i = lane + 64 * u;
+                    if (i < nq) {
+                        const float4 gg = g4[i];
+                        const float4 bb = beta ? b4[i] : make_float4(0.f, 0.f, 0.f, 0.f);
+                        bf16_t r0 = float_to_bf16((v[u].x - mean) * inv * gg.x + bb.x);
+                        bf16_t r1 = float_to_bf16((v[u].y - mean) * inv * gg.y + bb.y);
+                        bf16_t r2 = float_to_bf16((v[u].z - mean) * inv * gg.z + bb.z);
+                        bf16_t r3 = float_to_bf16((v[u].w - mean) * inv * gg.w + bb.w);
+                        uint2 pk;
+                        pk.x = static_cast<uint32_t>(r0.bits) | (static_cast<uint32_t>(r1.bits) << 16);
+                        pk.y = static_cast<uint32_t>(r2.bits) | (static_cast<uint32_t>(r3.bits) << 16);
+                        *reinterpret_cast<uint2*>(dst + 4 * i) = pk;
+                    }
                 }
             } else {
                 for (int k = lane; k < K; k += 64) dst[k].bits = 0;
@@ -213,7 +240,10 @@ static int launch_skinny(const void* A, int lda, const bf16_t* W, int ldw, const
     const int mt = (M + 15) / 16, nw = skinny_waves(N, K);
     const dim3 grid((N + 15) / 16), block(nw * 64);
     size_t smem = static_cast<size_t>(nw) * mt * 256 * sizeof(float);
-    if (LN_FUSED) smem += static_cast<size_t>(16) * mt * (K + 8) * sizeof(bf16_t);
+    if (LN_FUSED) {
+        smem += static_cast<size_t>(16) * mt * (K + 8) * sizeof(bf16_t);
+        if (K > 2048 || (reinterpret_cast<uintptr_t>(A) & 15) || lda % 4 != 0) return -2;
+    }
     if (smem > 64 * 1024) return -2;
 #define SKINNY_CASE(MTV)                                                                                  \
     case MTV:                                                                                             \

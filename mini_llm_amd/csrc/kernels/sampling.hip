@@ -10,15 +10,29 @@ __device__ __forceinline__ bool better(float v, int i, float bv, int bi) {
     return (v > bv) || (v == bv && i < bi);
 }
 
-__global__ void argmax_kernel(const float* __restrict__ logits, int ld, int V, int* __restrict__ out) {
+#define ARGMAX_CHUNK 2048      // elements per workgroup in the first stage (8 per thread)
+
+// Stage 1: the best (value, index) of one chunk of one row. Stage 2 (n_chunks == 1 input
+// chunks of pairs) reduces the chunks' results. Both keep the lowest index on ties.
+__global__ void argmax_stage1(const float* __restrict__ logits, int ld, int V, int n_chunks,
+                              float* __restrict__ part_val, int* __restrict__ part_idx, int* __restrict__ out) {
     __shared__ float sv[SAMPLE_THREADS / MLLM_WAVE];
     __shared__ int si[SAMPLE_THREADS / MLLM_WAVE];
-    const float* row = logits + static_cast<size_t>(blockIdx.x) * ld;
+    const int row_id = blockIdx.y, chunk = blockIdx.x;
+    const float* row = logits + static_cast<size_t>(row_id) * ld;
+    const int base = chunk * ARGMAX_CHUNK;
+    float v[ARGMAX_CHUNK / SAMPLE_THREADS];
+#pragma unroll
+    for (int u = 0; u < ARGMAX_CHUNK / SAMPLE_THREADS; ++u) {
+        const int i = base + u * SAMPLE_THREADS + threadIdx.x;
+        v[u] = i < V ? row[i] : -INFINITY;
+    }
     float bv = -INFINITY;
     int bi = 0x7fffffff;
-    for (int i = threadIdx.x; i < V; i += blockDim.x) {
-        float v = row[i];
-        if (better(v, i, bv, bi)) { bv = v; bi = i; }
+#pragma unroll
+    for (int u = 0; u < ARGMAX_CHUNK / SAMPLE_THREADS; ++u) {
+        const int i = base + u * SAMPLE_THREADS + threadIdx.x;
+        if (i < V && better(v[u], i, bv, bi)) { bv = v[u]; bi = i; }
     }
 #pragma unroll
     for (int off = MLLM_WAVE / 2; off > 0; off >>= 1) {
@@ -32,8 +46,32 @@ __global__ void argmax_kernel(const float* __restrict__ logits, int ld, int V, i
     if (threadIdx.x == 0) {
         for (int w = 1; w < SAMPLE_THREADS / MLLM_WAVE; ++w)
             if (better(sv[w], si[w], bv, bi)) { bv = sv[w]; bi = si[w]; }
-        out[blockIdx.x] = (bi == 0x7fffffff) ? 0 : bi;   // a row of NaNs yields 0
+        if (n_chunks == 1) {
+            out[row_id] = (bi == 0x7fffffff) ? 0 : bi;       // a row of NaNs yields 0
+        } else {
+            part_val[static_cast<size_t>(row_id) * n_chunks + chunk] = bv;
+            part_idx[static_cast<size_t>(row_id) * n_chunks + chunk] = bi;
+        }
     }
+}
+
+__global__ void argmax_stage2(const float* __restrict__ part_val, const int* __restrict__ part_idx,
+                              int n_chunks, int* __restrict__ out) {
+    const int row_id = blockIdx.x, lane = threadIdx.x;      // one wavefront per row
+    float bv = -INFINITY;
+    int bi = 0x7fffffff;
+    for (int c = lane; c < n_chunks; c += MLLM_WAVE) {
+        const float v = part_val[static_cast<size_t>(row_id) * n_chunks + c];
+        const int i = part_idx[static_cast<size_t>(row_id) * n_chunks + c];
+        if (better(v, i, bv, bi)) { bv = v; bi = i; }
+    }
+#pragma unroll
+    for (int off = MLLM_WAVE / 2; off > 0; off >>= 1) {
+        float ov = __shfl_xor(bv, off, MLLM_WAVE);
+        int oi = __shfl_xor(bi, off, MLLM_WAVE);
+        if (better(ov, oi, bv, bi)) { bv = ov; bi = oi; }
+    }
+    if (lane == 0) out[row_id] = (bi == 0x7fffffff) ? 0 : bi;
 }
 
 // ---------------------------------------------------------------------------
@@ -119,10 +157,20 @@ __global__ void sample_kernel(const float* __restrict__ logits, int ld, int V,
 
 extern "C" {
 
-int mllm_argmax(const float* logits, int ld, int n, int V, int* out, hipStream_t stream) {
+// Chunks of the first stage for a row of V values: the scratch holds n * chunks floats and ints.
+int mllm_argmax_chunks(int V) { return (V + ARGMAX_CHUNK - 1) / ARGMAX_CHUNK; }
+
+int mllm_argmax(const float* logits, int ld, int n, int V, int* out, float* part_val, int* part_idx,
+                hipStream_t stream) {
     if (n <= 0) return 0;
-    argmax_kernel<<<n, SAMPLE_THREADS, 0, stream>>>(logits, ld, V, out);
+    if (V <= 0) return -1;
+    const int n_chunks = (V + ARGMAX_CHUNK - 1) / ARGMAX_CHUNK;
+    argmax_stage1<<<dim3(n_chunks, n), SAMPLE_THREADS, 0, stream>>>(logits, ld, V, n_chunks, part_val, part_idx, out);
     MLLM_LAUNCH_CHECK();
+    if (n_chunks > 1) {
+        argmax_stage2<<<n, MLLM_WAVE, 0, stream>>>(part_val, part_idx, n_chunks, out);
+        MLLM_LAUNCH_CHECK();
+    }
     return 0;
 }
 

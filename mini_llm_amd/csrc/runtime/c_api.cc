@@ -39,6 +39,15 @@ int mllm_cache_state_slot(void* c, int64_t id) { return static_cast<CacheManager
 int mllm_cache_block_table(void* c, int64_t id, int g, int* out, int cap) {
     return static_cast<CacheManager*>(c)->block_table(id, g, out, cap);
 }
+int mllm_cache_fill_step_common(void* c, const int64_t* ids, const int* n_tokens, int n, int* positions,
+                                int* token_seq, int* cu_q, int* starts, int* ctx_len, int* state_slots) {
+    return static_cast<CacheManager*>(c)->fill_step_common(ids, n_tokens, n, positions, token_seq, cu_q, starts,
+                                                          ctx_len, state_slots);
+}
+int mllm_cache_fill_step_group(void* c, const int64_t* ids, const int* n_tokens, int n, int g, int max_blocks,
+                               int* tables, int* slots) {
+    return static_cast<CacheManager*>(c)->fill_step_group(ids, n_tokens, n, g, max_blocks, tables, slots);
+}
 int mllm_cache_free_pages(void* c, int g) { return static_cast<CacheManager*>(c)->free_pages(g); }
 int mllm_cache_total_pages(void* c, int g) { return static_cast<CacheManager*>(c)->total_pages(g); }
 int mllm_cache_free_state_slots(void* c) { return static_cast<CacheManager*>(c)->free_state_slots(); }

@@ -161,6 +161,51 @@ int CacheManager::block_table(int64_t id, int g, int* out, int cap) const {
     return n;
 }
 
+int CacheManager::fill_step_common(const int64_t* ids, const int* n_tokens, int n, int* positions,
+                                   int* token_seq, int* cu_q, int* starts, int* ctx_len, int* state_slots) const {
+    int t = 0;
+    cu_q[0] = 0;
+    for (int i = 0; i < n; ++i) {
+        auto it = requests_.find(ids[i]);
+        if (it == requests_.end()) return -(i + 1);
+        const RequestCache& rc = it->second;
+        starts[i] = rc.length;
+        ctx_len[i] = rc.length + n_tokens[i];
+        state_slots[i] = rc.state_slot;
+        for (int k = 0; k < n_tokens[i]; ++k, ++t) {
+            positions[t] = rc.length + k;
+            token_seq[t] = i;
+        }
+        cu_q[i + 1] = t;
+    }
+    return 0;
+}
+
+int CacheManager::fill_step_group(const int64_t* ids, const int* n_tokens, int n, int g, int max_blocks,
+                                  int* tables, int* slots) const {
+    if (g < 0 || g >= n_groups()) return -1;
+    const int ps = groups_[g].page_size;
+    int t = 0;
+    for (int i = 0; i < n; ++i) {
+        auto it = requests_.find(ids[i]);
+        if (it == requests_.end()) return -(i + 1);
+        const RequestCache& rc = it->second;
+        const auto& tab = rc.tables[g];
+        const int nb = static_cast<int>(tab.size());
+        if (nb > max_blocks) return -(i + 1);
+        int* row = tables + static_cast<size_t>(i) * max_blocks;
+        for (int b = 0; b < nb; ++b) row[b] = tab[b];
+        for (int b = nb; b < max_blocks; ++b) row[b] = 0;
+        for (int k = 0; k < n_tokens[i]; ++k, ++t) {
+            const int pos = rc.length + k;
+            const int blk = pos / ps;
+            if (blk >= nb || tab[blk] < 0) return -(i + 1);
+            slots[t] = tab[blk] * ps + pos % ps;
+        }
+    }
+    return 0;
+}
+
 std::string CacheManager::check() const {
     std::ostringstream err;
     for (int g = 0; g < n_groups(); ++g) {

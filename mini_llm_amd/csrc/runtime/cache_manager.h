@@ -90,6 +90,17 @@ public:
     // of logical blocks, or -2 for an unknown id. At most `cap` entries are written.
     int block_table(int64_t id, int g, int* out, int cap) const;
 
+    // Index arrays of a step in which request ids[i] feeds n_tokens[i] tokens from its committed
+    // length on. Tokens are laid out request after request. Returns 0, or -(i+1) if request i is
+    // unknown.
+    int fill_step_common(const int64_t* ids, const int* n_tokens, int n, int* positions, int* token_seq,
+                         int* cu_q, int* starts, int* ctx_len, int* state_slots) const;
+    // For one group: tables[i*max_blocks ..] = block table of request i (entries beyond it 0), and
+    // slots[t] = page*page_size + offset of every token. Returns 0, or -(i+1) if request i is unknown,
+    // holds no page for one of its tokens, or has more than max_blocks blocks.
+    int fill_step_group(const int64_t* ids, const int* n_tokens, int n, int g, int max_blocks, int* tables,
+                        int* slots) const;
+
     // Consistency check: every page is either free or held by exactly one
     // (request, group, block); every slot likewise. Empty string when consistent.
     std::string check() const;

@@ -101,21 +101,28 @@ class Engine:
                 outputs.append(RequestOutput(rid, -1, True))
         if not plan:
             return outputs
-        entries = []
-        for e in plan:
-            r = self.requests[e.request_id]
-            entries.append(StepEntry(e.request_id, r.tokens[e.start:e.start + e.n_tokens],
-                                     [e.n_tokens - 1] if e.want_last else []))
-        logits = self.runner.step(entries, manage_cache=False)
-        self.scheduler.commit()
         sampled = [e for e in plan if e.want_last]
-        if sampled:
-            temps, us = [], []
-            for e in sampled:
+        temps, us = [], []
+        for e in sampled:
+            r = self.requests[e.request_id]
+            temps.append(r.params.temperature)
+            us.append(uniform01(r.params.seed, len(r.tokens) - r.prompt_len) if r.params.temperature > 0 else 0.0)
+        if self.runner.use_graphs and len(sampled) == len(plan) and all(e.n_tokens == 1 for e in plan):
+            # every entry is one decoded token: the whole step replays as a HIP graph
+            tokens = self.runner.decode_step([e.request_id for e in plan],
+                                             [self.requests[e.request_id].tokens[e.start] for e in plan],
+                                             temps, us)
+            self.scheduler.commit()
+        else:
+            entries = []
+            for e in plan:
                 r = self.requests[e.request_id]
-                temps.append(r.params.temperature)
-                us.append(uniform01(r.params.seed, len(r.tokens) - r.prompt_len))
-            tokens = self.sampler.sample(logits, temps, us)
+                entries.append(StepEntry(e.request_id, r.tokens[e.start:e.start + e.n_tokens],
+                                         [e.n_tokens - 1] if e.want_last else []))
+            logits = self.runner.step(entries, manage_cache=False)
+            self.scheduler.commit()
+            tokens = self.sampler.sample(logits, temps, us) if sampled else []
+        if sampled:
             for e, tok in zip(sampled, tokens):
                 r = self.requests[e.request_id]
                 r.tokens.append(tok)

@@ -58,6 +58,49 @@ class StepError(ValueError):
     pass
 
 
+class _Staging:
+    """Pinned host buffers used in turn, each with the device buffer it is copied to: the host
+    may fill one while the copy out of the other is still queued on the stream."""
+
+    def __init__(self, device, n_buffers: int = 2):
+        self.device = torch.device(device)
+        self._bufs: List[list] = [[None, None, None] for _ in range(n_buffers)]   # pinned, device, event
+        self._turn = 0
+
+    def take(self, n_ints: int):
+        """A host numpy view of n_ints int32 and the matching device tensor (not yet copied)."""
+        self._turn = (self._turn + 1) % len(self._bufs)
+        b = self._bufs[self._turn]
+        if b[0] is None or b[0].numel() < n_ints:
+            cap = max(n_ints, 4096) * 2
+            on_gpu = self.device.type == "cuda"
+            b[0] = torch.empty(cap, dtype=torch.int32, pin_memory=on_gpu)
+            b[1] = torch.empty(cap, dtype=torch.int32, device=self.device)
+            b[2] = torch.cuda.Event() if on_gpu else None
+        elif b[2] is not None:
+            b[2].synchronize()            # the copy that last read this buffer is done
+        return b[0].numpy()[:n_ints], b
+
+    @staticmethod
+    def upload(b, n_ints: int, dst: Optional[torch.Tensor] = None) -> torch.Tensor:
+        dev = b[1] if dst is None else dst
+        dev[:n_ints].copy_(b[0][:n_ints], non_blocking=True)
+        if b[2] is not None:
+            b[2].record()
+        return dev
+
+
+def _layout(T: int, B: int, n_logits: int, max_blocks: Sequence[int]):
+    """Offsets of the step's int32 arrays in one packed buffer."""
+    sizes = [T, T, T, B + 1, B, B, B, max(n_logits, 1)]
+    for mb in max_blocks:
+        sizes += [B * mb, T]
+    offs = [0]
+    for n in sizes:
+        offs.append(offs[-1] + n)
+    return offs
+
+
 class ModelRunner:
     """Owns a model and its cache storage, and runs steps."""
 
@@ -68,10 +111,10 @@ class ModelRunner:
                                   model.device)
         self.manager = self.cache.manager
         self.page_size = page_size
-        # Two staging buffers used in turn: the host may fill one while the copy out of
-        # the other is still queued on the stream.
-        self._staging: List[list] = [[None, None, None], [None, None, None]]   # pinned, device, event
-        self._turn = 0
+        self.n_pages = n_pages
+        self._staging = _Staging(self.device)
+        self._graphs: Dict[tuple, "DecodeGraph"] = {}
+        self.use_graphs = self.device.type == "cuda" and getattr(model, "graph_safe", True)
 
     # -- cache bookkeeping for callers without a scheduler ---------------------------
     def ensure_request(self, rid: int) -> None:
@@ -82,98 +125,78 @@ class ModelRunner:
         self.manager.free_request(rid)
 
     # -- the step ----------------------------------------------------------------------
-    def build_context(self, entries: Sequence[StepEntry]) -> StepContext:
-        mgr, B = self.manager, len(entries)
-        if B == 0:
-            raise StepError("a step needs at least one entry")
-        vocab, max_pos = self.model.vocab_size, self.model.max_positions
-        seen = set()
-        q_lens = np.empty(B, dtype=np.int64)
-        starts = np.empty(B, dtype=np.int64)
-        for i, e in enumerate(entries):
-            if e.request_id in seen:
-                raise StepError(f"request {e.request_id} appears twice in one step")
-            seen.add(e.request_id)
-            n = len(e.tokens)
-            if n < 1:
-                raise StepError(f"request {e.request_id}: an entry needs at least one token")
-            q_lens[i] = n
-            starts[i] = mgr.length(e.request_id)
-            for w in e.want:
-                if not (0 <= w < n):
-                    raise StepError(f"request {e.request_id}: wanted index {w} is outside its {n} tokens")
-        T = int(q_lens.sum())
-        ctx = starts + q_lens
-        if max_pos is not None and int(ctx.max()) > max_pos:
-            i = int(ctx.argmax())
-            raise StepError(f"request {entries[i].request_id}: {int(ctx[i])} tokens exceed the model's "
-                            f"{max_pos} positions")
-        n_logits = sum(len(e.want) for e in entries)
-        G = self.cache.n_groups
-        max_blocks = [max(1, -(-int(ctx.max()) // self.page_size)) for _ in range(G)]
+    def _fill(self, host: np.ndarray, offs, ids: np.ndarray, n_tok: np.ndarray, max_blocks: Sequence[int]):
+        """Fills the packed index arrays (all but token ids and logit rows) natively."""
+        seg = [host[offs[i]:offs[i + 1]] for i in range(len(offs) - 1)]
+        self.manager.fill_step_common(ids, n_tok, seg[1], seg[2], seg[3], seg[5], seg[4], seg[6])
+        for g, mb in enumerate(max_blocks):
+            self.manager.fill_step_group(ids, n_tok, g, mb, seg[8 + 2 * g], seg[9 + 2 * g])
+        return seg
 
-        # one packed int32 buffer: a single host-to-device copy
-        sizes = [T, T, T, B + 1, B, B, B, max(n_logits, 1)]
-        for g in range(G):
-            sizes += [B * max_blocks[g], T]
-        offs = np.concatenate([[0], np.cumsum(sizes)])
-        total = int(offs[-1])
-        self._turn ^= 1
-        stage = self._staging[self._turn]
-        if stage[0] is None or stage[0].numel() < total:
-            cap = max(total, 4096) * 2
-            on_gpu = self.device.type == "cuda"
-            stage[0] = torch.empty(cap, dtype=torch.int32, pin_memory=on_gpu)
-            stage[1] = torch.empty(cap, dtype=torch.int32, device=self.device)
-            stage[2] = torch.cuda.Event() if on_gpu else None
-        elif stage[2] is not None:
-            stage[2].synchronize()        # the copy that last read this buffer is done
-        host = stage[0].numpy()
-        host[:total] = 0
-        seg = [host[offs[i]:offs[i + 1]] for i in range(len(sizes))]
-        tok, pos, tseq, cu_q, ctxl, st, slot_ids, lrows = seg[:8]
-        cu_q[0] = 0
-        np.cumsum(q_lens, out=cu_q[1:])
-        ctxl[:] = ctx
-        st[:] = starts
-        r = 0
-        for i, e in enumerate(entries):
-            a, b = int(cu_q[i]), int(cu_q[i + 1])
-            tok[a:b] = np.asarray(e.tokens, dtype=np.int64)
-            pos[a:b] = np.arange(starts[i], ctx[i])
-            tseq[a:b] = i
-            slot_ids[i] = mgr.state_slot(e.request_id)
-            for w in e.want:
-                lrows[r] = a + w
-                r += 1
-        if T and (tok[:T].min() < 0 or tok[:T].max() >= vocab):
-            raise StepError(f"token ids must lie in [0, {vocab})")
-        for g in range(G):
-            tab = seg[8 + 2 * g].reshape(B, max_blocks[g])
-            slots = seg[9 + 2 * g]
-            for i, e in enumerate(entries):
-                row = mgr.block_table(e.request_id, g, out=tab[i])
-                a, b = int(cu_q[i]), int(cu_q[i + 1])
-                p = pos[a:b]
-                blk = p // self.page_size
-                if len(row) * self.page_size < int(ctx[i]) or (tab[i][blk] < 0).any():
-                    raise StepError(f"request {e.request_id}: no pages are reserved for positions "
-                                    f"[{int(starts[i])}, {int(ctx[i])}) (reserve before the step)")
-                slots[a:b] = tab[i][blk] * self.page_size + p % self.page_size
-        dev = stage[1]
-        dev[:total].copy_(stage[0][:total], non_blocking=True)
-        if stage[2] is not None:
-            stage[2].record()
-        d = [dev[int(offs[i]):int(offs[i + 1])] for i in range(len(sizes))]
+    def _context(self, dev: torch.Tensor, offs, T, B, n_logits, max_blocks, max_q_len, max_ctx_len,
+                 seg=None, request_ids=()) -> StepContext:
+        d = [dev[offs[i]:offs[i + 1]] for i in range(len(offs) - 1)]
+        G = len(max_blocks)
         return StepContext(
             n_tokens=T, n_seqs=B, n_logits=n_logits,
             token_ids=d[0], positions=d[1], token_seq=d[2], cu_q=d[3], ctx_len=d[4], starts=d[5],
             state_slots=d[6], logit_rows=d[7][:n_logits],
             block_tables=[d[8 + 2 * g].view(B, max_blocks[g]) for g in range(G)],
             slots=[d[9 + 2 * g] for g in range(G)],
-            max_q_len=int(q_lens.max()), max_ctx_len=int(ctx.max()),
-            h_cu_q=cu_q.copy(), h_starts=starts.astype(np.int32), h_state_slots=slot_ids.copy(),
-            request_ids=[e.request_id for e in entries])
+            max_q_len=max_q_len, max_ctx_len=max_ctx_len,
+            h_cu_q=None if seg is None else seg[3].copy(),
+            h_starts=None if seg is None else seg[5].copy(),
+            h_state_slots=None if seg is None else seg[6].copy(),
+            request_ids=list(request_ids))
+
+    def build_context(self, entries: Sequence[StepEntry]) -> StepContext:
+        B = len(entries)
+        if B == 0:
+            raise StepError("a step needs at least one entry")
+        vocab, max_pos = self.model.vocab_size, self.model.max_positions
+        ids = np.fromiter((e.request_id for e in entries), dtype=np.int64, count=B)
+        if len(set(ids.tolist())) != B:
+            dup = [r for r in ids.tolist() if (ids == r).sum() > 1][0]
+            raise StepError(f"request {dup} appears twice in one step")
+        n_tok = np.fromiter((len(e.tokens) for e in entries), dtype=np.int32, count=B)
+        if n_tok.min() < 1:
+            raise StepError(f"request {entries[int(n_tok.argmin())].request_id}: an entry needs at least one token")
+        T = int(n_tok.sum())
+        n_logits = 0
+        for e in entries:
+            for w in e.want:
+                if not (0 <= w < len(e.tokens)):
+                    raise StepError(f"request {e.request_id}: wanted index {w} is outside its "
+                                    f"{len(e.tokens)} tokens")
+            n_logits += len(e.want)
+        lengths = np.fromiter((self.manager.length(int(r)) for r in ids), dtype=np.int64, count=B)
+        ctx = lengths + n_tok
+        if max_pos is not None and int(ctx.max()) > max_pos:
+            i = int(ctx.argmax())
+            raise StepError(f"request {entries[i].request_id}: {int(ctx[i])} tokens exceed the model's "
+                            f"{max_pos} positions")
+        G = self.cache.n_groups
+        max_blocks = [max(1, -(-int(ctx.max()) // self.page_size))] * G
+        offs = _layout(T, B, n_logits, max_blocks)
+        host, buf = self._staging.take(offs[-1])
+        try:
+            seg = self._fill(host, offs, ids, n_tok, max_blocks)
+        except KeyError as err:
+            raise StepError(str(err.args[0])) from None
+        tok, lrows = seg[0], seg[7]
+        r = t = 0
+        for e in entries:
+            n = len(e.tokens)
+            tok[t:t + n] = e.tokens
+            for w in e.want:
+                lrows[r] = t + w
+                r += 1
+            t += n
+        if tok.min() < 0 or tok.max() >= vocab:
+            raise StepError(f"token ids must lie in [0, {vocab})")
+        dev = self._staging.upload(buf, offs[-1])
+        return self._context(dev, offs, T, B, n_logits, max_blocks, int(n_tok.max()), int(ctx.max()), seg,
+                             ids.tolist())
 
     def step(self, entries: Sequence[StepEntry], manage_cache: bool = True) -> Optional[torch.Tensor]:
         """Runs one batch. With ``manage_cache`` the runner registers new requests, takes
@@ -200,3 +223,98 @@ class ModelRunner:
             for e in entries:
                 mgr.commit(e.request_id, mgr.length(e.request_id) + len(e.tokens))
         return logits
+
+    # -- decode steps through a captured HIP graph ------------------------------------------
+    def decode_step(self, request_ids: Sequence[int], tokens: Sequence[int],
+                    temperatures: Optional[Sequence[float]] = None,
+                    uniforms: Optional[Sequence[float]] = None) -> List[int]:
+        """One decoded token for each request (pages already reserved, lengths committed by the
+        caller afterwards): runs the model and the sampler as one HIP graph and returns the sampled
+        token of each request. The graph for a batch size is captured at its first use."""
+        B = len(request_ids)
+        greedy = temperatures is None or all(t <= 0 for t in temperatures)
+        bucket = B if B <= 8 else -(-B // 8) * 8
+        key = (bucket, greedy)
+        g = self._graphs.get(key)
+        if g is None:
+            g = self._graphs[key] = DecodeGraph(self, bucket, greedy)
+        return g.run(request_ids, tokens, temperatures, uniforms)
+
+
+class DecodeGraph:
+    """A decode step of fixed batch size captured as a HIP graph: embedding, every layer, the
+    head and the sampler replay from static buffers; per step the host only refreshes the index
+    arrays (one copy) and reads the sampled tokens back.
+
+    Rows beyond the live batch repeat row 0 without writing to the cache, so one graph serves
+    every batch size up to its own.
+    """
+
+    def __init__(self, runner: ModelRunner, batch: int, greedy: bool):
+        from ..kernels import ops
+        self.runner, self.batch, self.greedy = runner, batch, greedy
+        model, cache = runner.model, runner.cache
+        dev = runner.device
+        max_pos = model.max_positions
+        cap_blocks = runner.n_pages if max_pos is None else min(runner.n_pages, -(-max_pos // runner.page_size))
+        self.max_blocks = [max(1, cap_blocks)] * cache.n_groups
+        B = batch
+        self.offs = _layout(B, B, B, self.max_blocks)
+        self.n_ints = self.offs[-1]
+        self.dev_ints = torch.zeros(self.n_ints, dtype=torch.int32, device=dev)
+        self.ctx = runner._context(self.dev_ints, self.offs, B, B, B, self.max_blocks, 1,
+                                   self.max_blocks[0] * runner.page_size if self.max_blocks else 1)
+        self.h_float = torch.zeros((2, B), dtype=torch.float32, pin_memory=True)
+        self.d_float = torch.zeros((2, B), dtype=torch.float32, device=dev)
+        self.out = torch.zeros(B, dtype=torch.int32, device=dev)
+        self.h_out = torch.zeros(B, dtype=torch.int32, pin_memory=True)
+        self.graph: Optional[torch.cuda.CUDAGraph] = None
+        self._ops = ops
+
+    def _forward(self) -> None:
+        logits = self.runner.model.forward(self.ctx, self.runner.cache)
+        if self.greedy:
+            self._ops.argmax(logits, self.out)
+        else:
+            self._ops.sample(logits, self.d_float[0], self.d_float[1], self.out)
+
+    def _fill(self, request_ids, tokens) -> None:
+        r, B, n = self.runner, self.batch, len(request_ids)
+        ids = np.empty(B, dtype=np.int64)
+        ids[:n] = request_ids
+        ids[n:] = request_ids[0]
+        n_tok = np.ones(B, dtype=np.int32)
+        host, buf = r._staging.take(self.n_ints)
+        seg = r._fill(host, self.offs, ids, n_tok, self.max_blocks)
+        tok = seg[0]
+        tok[:n] = tokens
+        tok[n:] = tokens[0]
+        if tok.min() < 0 or tok.max() >= r.model.vocab_size:
+            raise StepError(f"token ids must lie in [0, {r.model.vocab_size})")
+        seg[7][:] = np.arange(B, dtype=np.int32)
+        for g in range(len(self.max_blocks)):
+            seg[9 + 2 * g][n:] = -1              # padding rows write nothing to the cache
+        self.h_cu_q, self.h_starts, self.h_state_slots = seg[3], seg[5], seg[6]
+        _Staging.upload(buf, self.n_ints, self.dev_ints)
+
+    def run(self, request_ids, tokens, temperatures, uniforms) -> List[int]:
+        n = len(request_ids)
+        self._fill(request_ids, tokens)
+        if not self.greedy:
+            h = self.h_float.numpy()
+            h[0, :n] = temperatures
+            h[1, :n] = uniforms
+            h[0, n:] = 0.0
+            self.d_float.copy_(self.h_float, non_blocking=True)
+        if self.graph is None:
+            # First use: run once eagerly (loads the kernels, sizes their scratch), then capture.
+            # Running the same step twice is harmless: it writes the same keys and values.
+            self._forward()
+            torch.cuda.synchronize()
+            self.graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(self.graph):
+                self._forward()
+        self.graph.replay()
+        self.h_out.copy_(self.out, non_blocking=True)
+        torch.cuda.current_stream().synchronize()
+        return self.h_out[:n].tolist()

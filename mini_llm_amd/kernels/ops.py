@@ -169,7 +169,8 @@ def ln_linear(x: torch.Tensor, gamma: torch.Tensor, beta: Optional[torch.Tensor]
     _gpu(x, gamma, beta, w, bias, out)
     M, K = x.shape
     N = w.shape[0]
-    if w.dtype == torch.bfloat16 and M <= 16 and x.dtype == torch.float32 and x.is_contiguous():
+    if (w.dtype == torch.bfloat16 and M <= 16 and x.dtype == torch.float32 and x.is_contiguous()
+            and gamma.data_ptr() % 16 == 0 and (beta is None or beta.data_ptr() % 16 == 0)):
         _rows2d(w, "w")
         _rows2d(out, "out")
         if w.shape[1] != K or gamma.numel() != K or gamma.dtype != torch.float32:
@@ -255,13 +256,13 @@ def paged_attention(q: torch.Tensor, q_col: int, n_heads: int, n_kv_heads: int, 
     if max_q_len == 1 and lpk >= 2 and (lpk & (lpk - 1)) == 0:
         # every query is a single decoded token: split its keys over workgroups
         pairs = T * n_heads
-        nsplit = max(1, min(16, 1024 // pairs, -(-max(max_ctx_len, 1) // 64)))
+        nsplit, waves = _decode_launch_shape(pairs, max_ctx_len)
         ws, counters = _decode_workspace(q.device, pairs, nsplit, head_dim)
         lib = load_library("attention_decode")
         _check(lib.mllm_decode_attention(
             _p(q), q.stride(0), q_col, _p(k_pages), _p(v_pages), kv_dim, _p(block_tables), block_tables.shape[1],
             _p(token_seq), _p(positions), T, n_heads, n_kv_heads, head_dim, page_size, ctypes.c_float(scale),
-            int(window or 0), nsplit, _p(out), out.stride(0), _p(ws), _p(counters), _dt(q), _stream()),
+            int(window or 0), nsplit, waves, _p(out), out.stride(0), _p(ws), _p(counters), _dt(q), _stream()),
             "decode_attention")
         return out
     lib = load_library("attention")
@@ -273,6 +274,16 @@ def paged_attention(q: torch.Tensor, q_col: int, n_heads: int, n_kv_heads: int, 
 
 
 _DECODE_WS = {}
+DECODE_SHAPE_OVERRIDE = None      # (nsplit, waves): set by tuning scripts only
+
+
+def _decode_launch_shape(pairs: int, max_ctx_len: int):
+    """How many workgroups share one (token, head) pair's keys, and wavefronts per workgroup."""
+    if DECODE_SHAPE_OVERRIDE is not None:
+        return DECODE_SHAPE_OVERRIDE
+    nsplit = max(1, min(16, 1024 // pairs, -(-max(max_ctx_len, 1) // 64)))
+    return nsplit, 4
+
 
 
 def _decode_workspace(device, pairs: int, nsplit: int, head_dim: int):
@@ -289,6 +300,9 @@ def _decode_workspace(device, pairs: int, nsplit: int, head_dim: int):
     return ws, counters
 
 
+_ARGMAX_WS = {}
+
+
 def argmax(logits: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
     """out[i] = index of the largest logits[i,:], the lowest index on ties."""
     _gpu(logits, out)
@@ -298,7 +312,14 @@ def argmax(logits: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
     n, V = logits.shape
     _i32(out, "out", n)
     lib = load_library("sampling")
-    _check(lib.mllm_argmax(_p(logits), logits.stride(0), n, V, _p(out), _stream()), "argmax")
+    chunks = lib.mllm_argmax_chunks(V)
+    key = logits.device
+    pv, pi = _ARGMAX_WS.get(key, (None, None))
+    if pv is None or pv.numel() < n * chunks:
+        pv = torch.empty(max(n * chunks, 4096), dtype=torch.float32, device=logits.device)
+        pi = torch.empty(max(n * chunks, 4096), dtype=torch.int32, device=logits.device)
+        _ARGMAX_WS[key] = (pv, pi)
+    _check(lib.mllm_argmax(_p(logits), logits.stride(0), n, V, _p(out), _p(pv), _p(pi), _stream()), "argmax")
     return out
 
 

@@ -52,6 +52,11 @@ class DecoderModel:
     def max_positions(self) -> Optional[int]:
         return self.config.max_positions
 
+    @property
+    def graph_safe(self) -> bool:
+        """True when a decode step of this model may be captured and replayed as a HIP graph."""
+        return all(layer.graph_safe for layer in self.layers)
+
     def cache_specs(self) -> List[object]:
         return list(self._cache_specs)
 

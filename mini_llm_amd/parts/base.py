@@ -82,6 +82,8 @@ class NormedInput:
 
 class Mixer(Part):
     accepts_normed_input = False     # True: forward() takes a NormedInput instead of a tensor
+    graph_safe = True                # False: forward() plans on the host (reads ctx.h_*), so a decode
+                                     # step that contains it cannot be replayed as a HIP graph
 
     def cache_spec(self):
         """KVCacheSpec, StateCacheSpec or None."""
@@ -93,6 +95,7 @@ class Mixer(Part):
 
 class FeedForward(Part):
     accepts_normed_input = False
+    graph_safe = True
 
     def forward(self, h, ctx, x) -> None:
         raise NotImplementedError
@@ -111,6 +114,10 @@ class PositionEncoding(Part):
 class Block(Part):
     def forward(self, x, ctx, cache_view, write: bool = True) -> None:
         raise NotImplementedError
+
+    @property
+    def graph_safe(self) -> bool:
+        return all(getattr(getattr(self, name, None), "graph_safe", True) for name in ("mixer", "feed_forward"))
 
     def cache_spec(self):
         return None

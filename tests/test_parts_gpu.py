@@ -152,6 +152,7 @@ def _define_toy():
     @register_mixer("toy_running_mean", replace=True)
     class RunningMean(Mixer):
         """state <- decay * state + (1 - decay) * h_t, token by token; x_t += gain * state."""
+        graph_safe = False           # it walks the batch on the host
 
         def __init__(self, size, decay, dtype, device):
             super().__init__(dtype, device)
@@ -292,6 +293,7 @@ def test_toy_architecture_with_a_stateful_mixer(tmp_path, dtype):
         assert fed[r] == len(ids)
         ref = _toy_plain(w, cfg, ids)
         assert (torch.cat(got[r]).double() - ref).abs().max() <= tol, r
+    assert not model.graph_safe and not runner.use_graphs
     # a slot that is used again starts from an empty state
     runner.end_request(3)
     out = runner.step([StepEntry(4, seqs[3], list(range(9)))]).float().cpu()
