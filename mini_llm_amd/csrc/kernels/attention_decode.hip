@@ -51,7 +51,9 @@ decode_attention_kernel(const T* __restrict__ q, int q_stride, int q_col,
                         const int* __restrict__ token_seq, const int* __restrict__ positions,
                         int n_heads, int n_kv_heads, int page_size, float scale_log2e, int window,
                         int nsplit, T* __restrict__ out, int out_stride,
-                        float* __restrict__ ws_o, float* __restrict__ ws_ml, int* __restrict__ counters) {
+                        float* __restrict__ ws_o, float* __restrict__ ws_ml, int* __restrict__ counters,
+                        T* __restrict__ k_pages_w, T* __restrict__ v_pages_w, int k_col, int v_col,
+                        const int* __restrict__ slots) {
     constexpr int EPL = Vec16<T>::N;        // elements per lane
     constexpr int DH = LPK * EPL;           // head size
     constexpr int KPW = MLLM_WAVE / LPK;    // keys per wavefront and load instruction
@@ -85,6 +87,11 @@ decode_attention_kernel(const T* __restrict__ q, int q_stride, int q_col,
 #pragma unroll
     for (int e = 0; e < EPL; ++e) o[e] = 0.f;
     const size_t col = static_cast<size_t>(hk) * DH + c * EPL;
+    // With `slots`, the token's own key and value are not in the pages yet: they are read from
+    // its row of q (columns k_col, v_col) and written to the pages here, by the first query head
+    // of each key/value head.
+    const bool append = slots != nullptr;
+    const bool writer = append && (h % (n_heads / n_kv_heads) == 0) && slots[t] >= 0;
 
     for (int j0 = kb + wave * KPW; j0 < ke; j0 += n_waves * KPW * DEC_UNROLL) {
         float kf[DEC_UNROLL][EPL], vf[DEC_UNROLL][EPL];
@@ -94,10 +101,23 @@ decode_attention_kernel(const T* __restrict__ q, int q_stride, int q_col,
             const int j = j0 + u * n_waves * KPW + g;
             valid[u] = j < ke;
             if (valid[u]) {
-                const size_t row = pow2 ? ((static_cast<size_t>(table[j >> shift]) << shift) + (j & (page_size - 1)))
-                                        : (static_cast<size_t>(table[j / page_size]) * page_size + j % page_size);
-                Vec16<T>::load(k_pages + row * kv_dim + col, kf[u]);
-                Vec16<T>::load(v_pages + row * kv_dim + col, vf[u]);
+                if (append && j == p) {
+                    const T* src = q + static_cast<size_t>(t) * q_stride + col;
+                    const uint4 kraw = *reinterpret_cast<const uint4*>(src + k_col);
+                    const uint4 vraw = *reinterpret_cast<const uint4*>(src + v_col);
+                    if (writer) {
+                        const size_t wrow = static_cast<size_t>(slots[t]) * kv_dim + col;
+                        *reinterpret_cast<uint4*>(k_pages_w + wrow) = kraw;
+                        *reinterpret_cast<uint4*>(v_pages_w + wrow) = vraw;
+                    }
+                    Vec16<T>::load(src + k_col, kf[u]);
+                    Vec16<T>::load(src + v_col, vf[u]);
+                } else {
+                    const size_t row = pow2 ? ((static_cast<size_t>(table[j >> shift]) << shift) + (j & (page_size - 1)))
+                                            : (static_cast<size_t>(table[j / page_size]) * page_size + j % page_size);
+                    Vec16<T>::load(k_pages + row * kv_dim + col, kf[u]);
+                    Vec16<T>::load(v_pages + row * kv_dim + col, vf[u]);
+                }
             }
         }
 #pragma unroll
@@ -201,13 +221,14 @@ static int launch_decode(int lpk, dim3 grid, int waves, hipStream_t stream, cons
                          const T* k_pages, const T* v_pages, int kv_dim, const int* block_tables,
                          int max_blocks, const int* token_seq, const int* positions, int n_heads,
                          int n_kv_heads, int page_size, float scale_log2e, int window, int nsplit, T* out,
-                         int out_stride, float* ws_o, float* ws_ml, int* counters) {
+                         int out_stride, float* ws_o, float* ws_ml, int* counters, T* k_pages_w, T* v_pages_w,
+                         int k_col, int v_col, const int* slots) {
 #define DEC_CASE(L)                                                                                    \
     case L:                                                                                            \
         decode_attention_kernel<T, L><<<grid, waves * MLLM_WAVE, 0, stream>>>(                     \
             q, q_stride, q_col, k_pages, v_pages, kv_dim, block_tables, max_blocks, token_seq,         \
             positions, n_heads, n_kv_heads, page_size, scale_log2e, window, nsplit, out, out_stride,   \
-            ws_o, ws_ml, counters);                                                                    \
+            ws_o, ws_ml, counters, k_pages_w, v_pages_w, k_col, v_col, slots);                          \
         return 0;
     switch (lpk) {
         DEC_CASE(2) DEC_CASE(4) DEC_CASE(8) DEC_CASE(16) DEC_CASE(32) DEC_CASE(64)
@@ -225,12 +246,15 @@ long mllm_decode_attention_ws_floats(int n_q, int n_heads, int head_dim, int nsp
 
 // Returns 0, a HIP error code, or -1 for sizes the kernel refuses: head_dim * element size / 16
 // must be a power of two in [2, 64]. `counters` holds n_q*n_heads ints that are zero before the
-// first launch (the kernel leaves them zero).
+// first launch (the kernel leaves them zero). With `slots` (n_q rows of the page pools, < 0: none) the
+// tokens' own keys/values are taken from columns k_col/v_col of q and written to the pages by this
+// kernel; without, they must be in the pages already.
 int mllm_decode_attention(const void* q, int q_stride, int q_col, const void* k_pages, const void* v_pages,
                           int kv_dim, const int* block_tables, int max_blocks, const int* token_seq,
                           const int* positions, int n_q, int n_heads, int n_kv_heads, int head_dim,
                           int page_size, float scale, int window, int nsplit, int waves, void* out,
-                          int out_stride, float* ws, int* counters, int dtype, hipStream_t stream) {
+                          int out_stride, float* ws, int* counters, int k_col, int v_col, const int* slots,
+                          int dtype, hipStream_t stream) {
     if (n_q <= 0) return 0;
     const int esz = dtype == MLLM_F32 ? 4 : 2;
     const int lpk = head_dim * esz / 16;
@@ -245,12 +269,12 @@ int mllm_decode_attention(const void* q, int q_stride, int q_col, const void* k_
         rc = launch_decode<float>(lpk, grid, waves, stream, (const float*)q, q_stride, q_col, (const float*)k_pages,
                                   (const float*)v_pages, kv_dim, block_tables, max_blocks, token_seq, positions,
                                   n_heads, n_kv_heads, page_size, sl2, window, nsplit, (float*)out, out_stride,
-                                  ws_o, ws_ml, counters);
+                                  ws_o, ws_ml, counters, (float*)k_pages, (float*)v_pages, k_col, v_col, slots);
     else
         rc = launch_decode<bf16_t>(lpk, grid, waves, stream, (const bf16_t*)q, q_stride, q_col, (const bf16_t*)k_pages,
                                    (const bf16_t*)v_pages, kv_dim, block_tables, max_blocks, token_seq, positions,
                                    n_heads, n_kv_heads, page_size, sl2, window, nsplit, (bf16_t*)out, out_stride,
-                                   ws_o, ws_ml, counters);
+                                   ws_o, ws_ml, counters, (bf16_t*)k_pages, (bf16_t*)v_pages, k_col, v_col, slots);
     if (rc != 0) return rc;
     MLLM_LAUNCH_CHECK();
     return 0;

@@ -127,7 +127,8 @@ template <int MT, bool LN_FUSED>
 __global__ void __launch_bounds__(1024)
 gemm_bf16_skinny(const void* __restrict__ Ain, int lda, const bf16_t* __restrict__ W, int ldw,
                  const float* __restrict__ bias, void* __restrict__ C, int ldc, int M, int N, int K, int mode,
-                 const float* __restrict__ gamma, const float* __restrict__ beta, float eps) {
+                 const float* __restrict__ gamma, const float* __restrict__ beta, float eps,
+                 const int* __restrict__ rows) {
     extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
     const int tid = threadIdx.x, wave = tid / 64, lane = tid % 64;
     const int nw = blockDim.x / 64;
@@ -136,6 +137,25 @@ gemm_bf16_skinny(const void* __restrict__ Ain, int lda, const bf16_t* __restrict
     float* red = reinterpret_cast<float*>(smem_raw);                       // [nw][MT][256]
     bf16_t* a_s = reinterpret_cast<bf16_t*>(smem_raw + static_cast<size_t>(nw) * MT * 256 * sizeof(float));
     const int a_stride = K + 8;
+    const int n = n0 + row16;
+    const bf16_t* wrow = W + static_cast<size_t>(n < N ? n : 0) * ldw;
+    const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
+
+    f32x4 acc[MT];
+#pragma unroll
+    for (int i = 0; i < MT; ++i) acc[i] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+    // The first weight fragments of this wavefront are requested before the norm, so that their
+    // latency overlaps it.
+    constexpr int PRE = 4;
+    bf16x8 bpre[PRE];
+    if (LN_FUSED) {
+#pragma unroll
+        for (int u = 0; u < PRE; ++u) {
+            const int k = (wave + u * nw) * 32 + 8 * kq;
+            bpre[u] = (k < K && n < N) ? *reinterpret_cast<const bf16x8*>(wrow + k) : zero;
+        }
+    }
 
     if (LN_FUSED) {
         // one wavefront per row: mean, then variance of the centred values, all in fp32
@@ -144,7 +164,7 @@ gemm_bf16_skinny(const void* __restrict__ Ain, int lda, const bf16_t* __restrict
             bf16_t* dst = a_s + static_cast<size_t>(m) * a_stride;
             if (m < M) {
                 // the row lives in registers: one pass over memory (K <= 2048, K % 4 == 0)
-                const float4* xr = reinterpret_cast<const float4*>(x + static_cast<size_t>(m) * lda);
+                const float4* xr = reinterpret_cast<const float4*>(x + static_cast<size_t>(rows ? rows[m] : m) * lda);
                 const int nq = K / 4;
                 float4 v[8];
                 float s = 0.f;
@@ -189,16 +209,27 @@ gemm_bf16_skinny(const void* __restrict__ Ain, int lda, const bf16_t* __restrict
         __syncthreads();
     }
 
-    f32x4 acc[MT];
-#pragma unroll
-    for (int i = 0; i < MT; ++i) acc[i] = f32x4{0.f, 0.f, 0.f, 0.f};
-    const int n = n0 + row16;
-    const bf16_t* wrow = W + static_cast<size_t>(n < N ? n : 0) * ldw;
     const bf16_t* A = static_cast<const bf16_t*>(Ain);
-    const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
 
+    int k_start = wave * 32;
+    if (LN_FUSED) {
+#pragma unroll
+        for (int u = 0; u < PRE; ++u) {
+            const int k = (wave + u * nw) * 32 + 8 * kq;
+            if ((wave + u * nw) * 32 < K) {
+                const bool kin = k < K;
+#pragma unroll
+                for (int i = 0; i < MT; ++i) {
+                    const int m = i * 16 + row16;
+                    bf16x8 a = kin ? *reinterpret_cast<const bf16x8*>(a_s + static_cast<size_t>(m) * a_stride + k) : zero;
+                    acc[i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, bpre[u], acc[i], 0, 0, 0);
+                }
+            }
+        }
+        k_start = (wave + PRE * nw) * 32;
+    }
 #pragma unroll 4
-    for (int k0 = wave * 32; k0 < K; k0 += nw * 32) {
+    for (int k0 = k_start; k0 < K; k0 += nw * 32) {
         const int k = k0 + 8 * kq;
         const bool kin = k < K;
         bf16x8 b = (kin && n < N) ? *reinterpret_cast<const bf16x8*>(wrow + k) : zero;
@@ -236,7 +267,7 @@ static int skinny_waves(int N, int K) {
 template <bool LN_FUSED>
 static int launch_skinny(const void* A, int lda, const bf16_t* W, int ldw, const float* bias, void* C, int ldc,
                          int M, int N, int K, int mode, const float* gamma, const float* beta, float eps,
-                         hipStream_t stream) {
+                         const int* rows, hipStream_t stream) {
     const int mt = (M + 15) / 16, nw = skinny_waves(N, K);
     const dim3 grid((N + 15) / 16), block(nw * 64);
     size_t smem = static_cast<size_t>(nw) * mt * 256 * sizeof(float);
@@ -248,7 +279,7 @@ static int launch_skinny(const void* A, int lda, const bf16_t* W, int ldw, const
 #define SKINNY_CASE(MTV)                                                                                  \
     case MTV:                                                                                             \
         gemm_bf16_skinny<MTV, LN_FUSED><<<grid, block, smem, stream>>>(A, lda, W, ldw, bias, C, ldc, M, N, K, \
-                                                                       mode, gamma, beta, eps);           \
+                                                                       mode, gamma, beta, eps, rows);     \
         break;
     switch (mt) {
         SKINNY_CASE(1) SKINNY_CASE(2) SKINNY_CASE(3) SKINNY_CASE(4)
@@ -271,7 +302,7 @@ int mllm_gemm_bf16(const void* A, int lda, const void* W, int ldw, const float* 
     const bf16_t* w = static_cast<const bf16_t*>(W);
     auto blocks = [&](int bm, int bn) { return static_cast<long>((M + bm - 1) / bm) * ((N + bn - 1) / bn); };
     if (M <= 64 && launch_skinny<false>(A, lda, w, ldw, bias, C, ldc, M, N, K, mode, nullptr, nullptr, 0.f,
-                                        stream) == 0) {
+                                        nullptr, stream) == 0) {
         // few rows: weight-streaming kernel
     } else if (M <= 32) {
         dim3 grid((N + 127) / 128, (M + 31) / 32);
@@ -287,17 +318,18 @@ int mllm_gemm_bf16(const void* A, int lda, const void* W, int ldw, const float* 
     return 0;
 }
 
-// LayerNorm of the fp32 rows x[M,K] fused into the product with W[N,K]: C = epilogue(LN(x) W^T + bias).
+// LayerNorm of the fp32 rows x[M,K] (row m taken from x[rows[m]] when `rows` is given) fused into the
+// product with W[N,K]: C = epilogue(LN(x) W^T + bias).
 // Returns 0, a HIP error code, -1 for misaligned operands, or -2 when M or K is too large for the
 // fused kernel (the caller then runs the norm and the product separately).
-int mllm_ln_gemm_bf16(const float* x, int ldx, const float* gamma, const float* beta, float eps, const void* W,
-                      int ldw, const float* bias, void* C, int ldc, int M, int N, int K, int mode,
+int mllm_ln_gemm_bf16(const float* x, int ldx, const int* rows, const float* gamma, const float* beta, float eps,
+                      const void* W, int ldw, const float* bias, void* C, int ldc, int M, int N, int K, int mode,
                       hipStream_t stream) {
     if (M <= 0 || N <= 0) return 0;
     if (K % 8 != 0 || ldw % 8 != 0 || (reinterpret_cast<uintptr_t>(W) & 15)) return -1;
     if (M > 16) return -2;
     int rc = launch_skinny<true>(x, ldx, static_cast<const bf16_t*>(W), ldw, bias, C, ldc, M, N, K, mode, gamma,
-                                 beta, eps, stream);
+                                 beta, eps, rows, stream);
     if (rc != 0) return rc;
     MLLM_LAUNCH_CHECK();
     return 0;

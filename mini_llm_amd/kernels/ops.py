@@ -159,16 +159,21 @@ def linear(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], out: 
 
 
 def ln_linear(x: torch.Tensor, gamma: torch.Tensor, beta: Optional[torch.Tensor], eps: float,
-              w: torch.Tensor, bias: Optional[torch.Tensor], out: torch.Tensor, epilogue: str = "store") -> torch.Tensor:
-    """out = epilogue(LayerNorm(x) @ w.T + bias) with x the fp32 stream [M,K] and w [N,K].
+              w: torch.Tensor, bias: Optional[torch.Tensor], out: torch.Tensor, epilogue: str = "store",
+              rows: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """out = epilogue(LayerNorm(x) @ w.T + bias) with x the fp32 stream [*,K] and w [N,K]; with
+    ``rows`` (int32 [M]) row m of the input is x[rows[m]].
 
     For bfloat16 weights and at most 16 rows the norm is fused into the product (one kernel);
     otherwise the norm and the product run one after the other. Same numerics either way:
     statistics in fp32, the normalised rows rounded to w's dtype before the product.
     """
-    _gpu(x, gamma, beta, w, bias, out)
-    M, K = x.shape
+    _gpu(x, gamma, beta, w, bias, out, rows)
+    K = x.shape[1]
+    M = x.shape[0] if rows is None else rows.numel()
     N = w.shape[0]
+    if rows is not None:
+        _i32(rows, "rows")
     if (w.dtype == torch.bfloat16 and M <= 16 and x.dtype == torch.float32 and x.is_contiguous()
             and gamma.data_ptr() % 16 == 0 and (beta is None or beta.data_ptr() % 16 == 0)):
         _rows2d(w, "w")
@@ -185,7 +190,7 @@ def ln_linear(x: torch.Tensor, gamma: torch.Tensor, beta: Optional[torch.Tensor]
         if bias is not None and (bias.dtype != torch.float32 or bias.numel() != N or not bias.is_contiguous()):
             raise KernelError(f"bias must be contiguous fp32 [{N}]")
         lib = load_library("gemm_bf16")
-        rc = lib.mllm_ln_gemm_bf16(_p(x), x.stride(0), _p(gamma), _p(beta), ctypes.c_float(eps), _p(w),
+        rc = lib.mllm_ln_gemm_bf16(_p(x), x.stride(0), _p(rows), _p(gamma), _p(beta), ctypes.c_float(eps), _p(w),
                                    w.stride(0), _p(bias), _p(out), out.stride(0), M, N, K, EPILOGUES[epilogue],
                                    _stream())
         if rc == 0:
@@ -193,7 +198,7 @@ def ln_linear(x: torch.Tensor, gamma: torch.Tensor, beta: Optional[torch.Tensor]
         if rc != -2:
             _check(rc, "ln_linear")
     h = torch.empty((M, K), dtype=w.dtype, device=x.device)
-    layernorm(x, gamma, beta, eps, h)
+    layernorm(x, gamma, beta, eps, h, rows)
     return linear(h, w, bias, out, epilogue)
 
 
@@ -219,13 +224,18 @@ def paged_attention(q: torch.Tensor, q_col: int, n_heads: int, n_kv_heads: int, 
                     k_pages: torch.Tensor, v_pages: torch.Tensor, page_size: int,
                     block_tables: torch.Tensor, token_seq: torch.Tensor, positions: torch.Tensor,
                     scale: float, window: int, out: torch.Tensor, *, cu_q: Optional[torch.Tensor] = None,
-                    ctx_len: Optional[torch.Tensor] = None, max_q_len: int = 0, max_ctx_len: int = 0) -> torch.Tensor:
+                    ctx_len: Optional[torch.Tensor] = None, max_q_len: int = 0, max_ctx_len: int = 0,
+                    append: Optional[tuple] = None) -> torch.Tensor:
     """Causal attention of the step's queries over the pages.
 
     q: [T, >= q_col + n_heads*head_dim] (queries of token t start at column q_col);
     block_tables: int32 [B, max_blocks]; token_seq[t]: row of block_tables; positions[t]:
     position of token t in its sequence. A query at position p sees keys
     [max(0, p-window+1) if window else 0, p]. out: [T, n_heads*head_dim].
+
+    ``append=(k_col, v_col, slots)``: the step's own keys and values are still in q's rows
+    (columns k_col, v_col) and this op writes them to row ``slots[t]`` of the pages first
+    (fused into the decode kernel where that runs); without it they are in the pages already.
     """
     _gpu(q, k_pages, v_pages, block_tables, token_seq, positions, out)
     _rows2d(q, "q")
@@ -253,7 +263,19 @@ def paged_attention(q: torch.Tensor, q_col: int, n_heads: int, n_kv_heads: int, 
     if (q.stride(0) * esz) % 16 or (q_col * esz) % 16 or (head_dim * esz) % 16 or q.data_ptr() % 16:
         raise KernelError("query rows and heads must be 16-byte aligned")
     lpk = head_dim * esz // 16
-    if max_q_len == 1 and lpk >= 2 and (lpk & (lpk - 1)) == 0:
+    decode = max_q_len == 1 and lpk >= 2 and (lpk & (lpk - 1)) == 0
+    k_col = v_col = 0
+    slots = None
+    if append is not None:
+        k_col, v_col, slots = append
+        if not decode:
+            kv_append(q, k_col, v_col, kv_dim, k_pages, v_pages, slots)
+            slots = None
+        else:
+            _i32(slots, "slots", T)
+            if max(k_col, v_col) + kv_dim > q.shape[1] or min(k_col, v_col) < 0 or (k_col * esz) % 16 or (v_col * esz) % 16:
+                raise KernelError("key/value columns lie outside q's rows or are not 16-byte aligned")
+    if decode:
         # every query is a single decoded token: split its keys over workgroups
         pairs = T * n_heads
         nsplit, waves = _decode_launch_shape(pairs, max_ctx_len)
@@ -262,7 +284,8 @@ def paged_attention(q: torch.Tensor, q_col: int, n_heads: int, n_kv_heads: int, 
         _check(lib.mllm_decode_attention(
             _p(q), q.stride(0), q_col, _p(k_pages), _p(v_pages), kv_dim, _p(block_tables), block_tables.shape[1],
             _p(token_seq), _p(positions), T, n_heads, n_kv_heads, head_dim, page_size, ctypes.c_float(scale),
-            int(window or 0), nsplit, waves, _p(out), out.stride(0), _p(ws), _p(counters), _dt(q), _stream()),
+            int(window or 0), nsplit, waves, _p(out), out.stride(0), _p(ws), _p(counters), k_col, v_col, _p(slots),
+            _dt(q), _stream()),
             "decode_attention")
         return out
     lib = load_library("attention")
@@ -281,8 +304,9 @@ def _decode_launch_shape(pairs: int, max_ctx_len: int):
     """How many workgroups share one (token, head) pair's keys, and wavefronts per workgroup."""
     if DECODE_SHAPE_OVERRIDE is not None:
         return DECODE_SHAPE_OVERRIDE
-    nsplit = max(1, min(16, 1024 // pairs, -(-max(max_ctx_len, 1) // 64)))
-    return nsplit, 4
+    # One workgroup per pair: merging splits needs a device-wide fence, which costs more than the
+    # parallelism gains at these context lengths. Few pairs get more wavefronts each instead.
+    return 1, (4 if pairs >= 512 else 8)
 
 
 

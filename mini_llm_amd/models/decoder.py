@@ -80,8 +80,9 @@ class DecoderModel:
             self.layers[call.layer].forward(x, ctx, cache.view(call.cache), call.write)
         if ctx.n_logits == 0:
             return None
-        h = self.final_norm.forward(x, rows=ctx.logit_rows)
-        return self.head.forward(h)
+        if hasattr(self.head, "forward_normed"):
+            return self.head.forward_normed(self.final_norm, x, ctx.logit_rows)
+        return self.head.forward(self.final_norm.forward(x, rows=ctx.logit_rows))
 
 
 def build_layers(specs: Sequence[LayerSpec], dtype, device, position: Optional[PositionEncoding] = None):

@@ -53,9 +53,10 @@ class Norm(Part):
     def forward(self, x: torch.Tensor, rows: Optional[torch.Tensor] = None) -> torch.Tensor:
         raise NotImplementedError
 
-    def linear(self, x: torch.Tensor, lin, out: torch.Tensor, epilogue: str = "store") -> torch.Tensor:
-        """out = epilogue(lin(norm(x))). A norm with a fused kernel overrides this."""
-        return lin(self.forward(x), out, epilogue)
+    def linear(self, x: torch.Tensor, lin, out: torch.Tensor, epilogue: str = "store",
+               rows: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """out = epilogue(lin(norm(x[rows]))). A norm with a fused kernel overrides this."""
+        return lin(self.forward(x, rows), out, epilogue)
 
 
 class NormedInput:

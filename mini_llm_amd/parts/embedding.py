@@ -73,6 +73,28 @@ class TiedHead(Part):
         super().__init__(dtype, device)
         self.embedding = embedding
 
+        self.weight_view = _HeadWeights(embedding)
+
     def forward(self, h: torch.Tensor) -> torch.Tensor:
         logits = torch.empty((h.shape[0], self.embedding.vocab_size), dtype=torch.float32, device=h.device)
         return ops.linear(h, self.embedding.weight, None, logits, "store_f32")
+
+    def forward_normed(self, norm, x: torch.Tensor, rows: torch.Tensor) -> torch.Tensor:
+        """logits of norm(x[rows]): lets the final norm fuse into the head's product."""
+        logits = torch.empty((rows.numel(), self.embedding.vocab_size), dtype=torch.float32, device=x.device)
+        return norm.linear(x, self.weight_view, logits, "store_f32", rows)
+
+
+class _HeadWeights:
+    """The tied head seen as a linear map without bias (weight = the embedding matrix)."""
+
+    def __init__(self, embedding: TokenEmbedding):
+        self._embedding = embedding
+        self.bias = None
+
+    @property
+    def weight(self):
+        return self._embedding.weight
+
+    def __call__(self, a, out, epilogue="store"):
+        return ops.linear(a, self.weight, None, out, epilogue)

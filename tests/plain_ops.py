@@ -58,8 +58,9 @@ def linear(a, w, bias, out, epilogue="store"):
     return out
 
 
-def ln_linear(x, gamma, beta, eps, w, bias, out, epilogue="store"):
-    h = layernorm(x, gamma, beta, eps, torch.empty(x.shape, dtype=w.dtype))
+def ln_linear(x, gamma, beta, eps, w, bias, out, epilogue="store", rows=None):
+    n = x.shape[0] if rows is None else rows.numel()
+    h = layernorm(x, gamma, beta, eps, torch.empty((n, x.shape[1]), dtype=w.dtype), rows)
     return linear(h, w, bias, out, epilogue)
 
 
@@ -72,8 +73,10 @@ def kv_append(src, k_col, v_col, kv_dim, k_pages, v_pages, slots):
 
 
 def paged_attention(q, q_col, n_heads, n_kv_heads, head_dim, k_pages, v_pages, page_size, block_tables,
-                    token_seq, positions, scale, window, out, **_):
+                    token_seq, positions, scale, window, out, append=None, **_):
     T = q.shape[0]
+    if append is not None:
+        kv_append(q, append[0], append[1], n_kv_heads * head_dim, k_pages, v_pages, append[2])
     rep = n_heads // n_kv_heads
     for t in range(T):
         b, p = int(token_seq[t]), int(positions[t])

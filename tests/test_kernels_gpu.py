@@ -149,9 +149,11 @@ def test_ln_linear(ops, dtype, M, N, K, epi):
     ref = plain_ops.linear(h, w, bias, torch.zeros(M, N, dtype=torch.float64), epi)
     tol = 3e-5 if dtype == torch.float32 else (2e-2 if epi == "store_f32" else 4e-2)
     assert (out.cpu().double() - ref).abs().max().item() <= tol
+    # no bias, rows gathered in another order
+    sel = torch.tensor(list(range(M - 1, -1, -1)), dtype=torch.int32)
     out2 = torch.zeros(M, N, dtype=odt, device=DEV)
-    ops.ln_linear(x.to(DEV), gamma.to(DEV), None, 1e-5, w.to(DEV), None, out2, epi)
-    h = plain_ops.layernorm(x, gamma, None, 1e-5, torch.empty(M, K, dtype=dtype))
+    ops.ln_linear(x.to(DEV), gamma.to(DEV), None, 1e-5, w.to(DEV), None, out2, epi, rows=sel.to(DEV))
+    h = plain_ops.layernorm(x, gamma, None, 1e-5, torch.empty(M, K, dtype=dtype), rows=sel)
     ref = plain_ops.linear(h, w, None, torch.zeros(M, N, dtype=torch.float64), epi)
     assert (out2.cpu().double() - ref).abs().max().item() <= tol
 
@@ -270,6 +272,52 @@ def test_paged_attention_decode_only(ops, dtype, H, Hkv, dh, page, window):
     # run twice in a row: the split counters must be back at zero
     out, ref = _attention_case(ops, dtype, H, Hkv, dh, page, [(700, 1), (2, 1)], window, g)
     assert (out - ref).abs().max() <= _tol(dtype, 2)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("H,Hkv,dh,page,qlens", [(12, 12, 64, 16, (1, 1, 1)), (6, 2, 32, 8, (1, 1, 1)),
+                                                   (5, 5, 48, 16, (1, 1, 1)), (4, 2, 64, 4, (3, 1, 9))])
+def test_paged_attention_appends_own_keys(ops, dtype, H, Hkv, dh, page, qlens):
+    """With append=..., the step's keys/values come from the q rows and land in the pages:
+    fused into the decode kernel (single-token queries, power-of-two heads) or copied first."""
+    g = torch.Generator().manual_seed(H + dh + sum(qlens))
+    starts = (200, 0, 31)
+    kv_dim, qd = Hkv * dh, H * dh
+    n_pages = sum(-(-(s + n) // page) for s, n in zip(starts, qlens)) + 2
+    kp = torch.full((n_pages * page, kv_dim), float("nan"), dtype=dtype)
+    vp = torch.full((n_pages * page, kv_dim), float("nan"), dtype=dtype)
+    ref_kp, ref_vp = kp.clone(), vp.clone()
+    maxb = max(-(-(s + n) // page) for s, n in zip(starts, qlens))
+    tables = torch.zeros(3, maxb, dtype=torch.int32)
+    T = sum(qlens)
+    qkv = _rand((T, qd + 2 * kv_dim), dtype, g)
+    token_seq, positions, slots = [], [], []
+    used = t = 0
+    for b, (s, n) in enumerate(zip(starts, qlens)):
+        nb = -(-(s + n) // page)
+        tables[b, :nb] = torch.arange(used, used + nb, dtype=torch.int32)
+        used += nb
+        js = torch.arange(s + n)
+        rows = tables[b].long()[js // page] * page + js % page
+        k, v = _rand((s + n, kv_dim), dtype, g), _rand((s + n, kv_dim), dtype, g)
+        k[s:], v[s:] = qkv[t:t + n, qd:qd + kv_dim], qkv[t:t + n, qd + kv_dim:]
+        ref_kp[rows], ref_vp[rows] = k, v
+        kp[rows[:s]], vp[rows[:s]] = k[:s], v[:s]             # the step's own rows are still empty
+        token_seq += [b] * n
+        positions += list(range(s, s + n))
+        slots += rows[s:].tolist()
+        t += n
+    token_seq, positions, slots = (torch.tensor(a, dtype=torch.int32) for a in (token_seq, positions, slots))
+    kp_d, vp_d = kp.to(DEV), vp.to(DEV)
+    out = torch.zeros(T, qd, dtype=dtype, device=DEV)
+    ops.paged_attention(qkv.to(DEV), 0, H, Hkv, dh, kp_d, vp_d, page, tables.to(DEV), token_seq.to(DEV),
+                        positions.to(DEV), dh ** -0.5, 0, out, max_q_len=max(qlens), max_ctx_len=210,
+                        append=(qd, qd + kv_dim, slots.to(DEV)))
+    ref = torch.zeros(T, qd, dtype=torch.float64)
+    plain_ops.paged_attention(qkv, 0, H, Hkv, dh, ref_kp, ref_vp, page, tables, token_seq, positions, dh ** -0.5, 0, ref)
+    assert (out.cpu().double() - ref).abs().max() <= _tol(dtype, 2)
+    written = slots.long()
+    assert torch.equal(kp_d.cpu()[written], ref_kp[written]) and torch.equal(vp_d.cpu()[written], ref_vp[written])
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
