@@ -16,20 +16,29 @@
 #include "common.h"
 
 #define DEC_MAX_WAVES 16
-#define DEC_UNROLL 4
+#define DEC_TABLE_LDS 1024   // block-table entries staged in LDS (longer tables are read from memory)
+#define DEC_UNROLL 8
 
+// 16 bytes of a row: kept raw in registers while the load is in flight, widened to fp32 when used.
 template <typename T> struct Vec16;
 template <> struct Vec16<bf16_t> {
     static constexpr int N = 8;
-    __device__ static void load(const bf16_t* p, float (&v)[8]) { load8(p, v); }
+    __device__ static void widen(const uint4& a, float (&v)[8]) {
+        v[0] = __uint_as_float(a.x << 16); v[1] = __uint_as_float(a.x & 0xffff0000u);
+        v[2] = __uint_as_float(a.y << 16); v[3] = __uint_as_float(a.y & 0xffff0000u);
+        v[4] = __uint_as_float(a.z << 16); v[5] = __uint_as_float(a.z & 0xffff0000u);
+        v[6] = __uint_as_float(a.w << 16); v[7] = __uint_as_float(a.w & 0xffff0000u);
+    }
 };
 template <> struct Vec16<float> {
     static constexpr int N = 4;
-    __device__ static void load(const float* p, float (&v)[4]) {
-        float4 a = *reinterpret_cast<const float4*>(p);
-        v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w;
+    __device__ static void widen(const uint4& a, float (&v)[4]) {
+        v[0] = __uint_as_float(a.x); v[1] = __uint_as_float(a.y);
+        v[2] = __uint_as_float(a.z); v[3] = __uint_as_float(a.w);
     }
 };
+template <typename T>
+__device__ __forceinline__ uint4 load_raw16(const T* p) { return *reinterpret_cast<const uint4*>(p); }
 
 template <int N>
 __device__ __forceinline__ void merge_state(float& m, float& l, float (&o)[N], float m2, float l2,
@@ -60,6 +69,7 @@ decode_attention_kernel(const T* __restrict__ q, int q_stride, int q_col,
     __shared__ float sm_m[DEC_MAX_WAVES], sm_l[DEC_MAX_WAVES];
     __shared__ float sm_o[DEC_MAX_WAVES][DH];
     __shared__ int sm_last;
+    __shared__ int sm_table[DEC_TABLE_LDS];
     const int n_waves = blockDim.x / MLLM_WAVE;
 
     const int pair = blockIdx.x, split = blockIdx.y;
@@ -73,13 +83,21 @@ decode_attention_kernel(const T* __restrict__ q, int q_stride, int q_col,
     const int per = (n_keys + nsplit - 1) / nsplit;
     const int kb = lo + split * per;
     const int ke = min(p + 1, kb + per);
-    const int* table = block_tables + static_cast<size_t>(b) * max_blocks;
+    const int* gtable = block_tables + static_cast<size_t>(b) * max_blocks;
+    // The sequence's block table goes to LDS first, so that no key load waits for a table load.
+    const int n_blocks_needed = p / page_size + 1;
+    const bool lds_table = n_blocks_needed <= DEC_TABLE_LDS;
+    if (lds_table) {
+        for (int i = threadIdx.x; i < n_blocks_needed; i += blockDim.x) sm_table[i] = gtable[i];
+        __syncthreads();
+    }
+    const int* table = lds_table ? sm_table : gtable;
     // pages of a power-of-two size are addressed with a shift and a mask
     const bool pow2 = (page_size & (page_size - 1)) == 0;
     const int shift = pow2 ? __ffs(page_size) - 1 : 0;
 
     float qf[EPL];
-    Vec16<T>::load(q + static_cast<size_t>(t) * q_stride + q_col + h * DH + c * EPL, qf);
+    Vec16<T>::widen(load_raw16(q + static_cast<size_t>(t) * q_stride + q_col + h * DH + c * EPL), qf);
 #pragma unroll
     for (int e = 0; e < EPL; ++e) qf[e] *= scale_log2e;
 
@@ -94,7 +112,7 @@ decode_attention_kernel(const T* __restrict__ q, int q_stride, int q_col,
     const bool writer = append && (h % (n_heads / n_kv_heads) == 0) && slots[t] >= 0;
 
     for (int j0 = kb + wave * KPW; j0 < ke; j0 += n_waves * KPW * DEC_UNROLL) {
-        float kf[DEC_UNROLL][EPL], vf[DEC_UNROLL][EPL];
+        uint4 kraw[DEC_UNROLL], vraw[DEC_UNROLL];
         bool valid[DEC_UNROLL];
 #pragma unroll
         for (int u = 0; u < DEC_UNROLL; ++u) {
@@ -103,20 +121,18 @@ decode_attention_kernel(const T* __restrict__ q, int q_stride, int q_col,
             if (valid[u]) {
                 if (append && j == p) {
                     const T* src = q + static_cast<size_t>(t) * q_stride + col;
-                    const uint4 kraw = *reinterpret_cast<const uint4*>(src + k_col);
-                    const uint4 vraw = *reinterpret_cast<const uint4*>(src + v_col);
+                    kraw[u] = load_raw16(src + k_col);
+                    vraw[u] = load_raw16(src + v_col);
                     if (writer) {
                         const size_t wrow = static_cast<size_t>(slots[t]) * kv_dim + col;
-                        *reinterpret_cast<uint4*>(k_pages_w + wrow) = kraw;
-                        *reinterpret_cast<uint4*>(v_pages_w + wrow) = vraw;
+                        *reinterpret_cast<uint4*>(k_pages_w + wrow) = kraw[u];
+                        *reinterpret_cast<uint4*>(v_pages_w + wrow) = vraw[u];
                     }
-                    Vec16<T>::load(src + k_col, kf[u]);
-                    Vec16<T>::load(src + v_col, vf[u]);
                 } else {
                     const size_t row = pow2 ? ((static_cast<size_t>(table[j >> shift]) << shift) + (j & (page_size - 1)))
                                             : (static_cast<size_t>(table[j / page_size]) * page_size + j % page_size);
-                    Vec16<T>::load(k_pages + row * kv_dim + col, kf[u]);
-                    Vec16<T>::load(v_pages + row * kv_dim + col, vf[u]);
+                    kraw[u] = load_raw16(k_pages + row * kv_dim + col);
+                    vraw[u] = load_raw16(v_pages + row * kv_dim + col);
                 }
             }
         }
@@ -124,17 +140,21 @@ decode_attention_kernel(const T* __restrict__ q, int q_stride, int q_col,
         for (int u = 0; u < DEC_UNROLL; ++u) {
             float dot = 0.f;
             if (valid[u]) {
+                float kf[EPL];
+                Vec16<T>::widen(kraw[u], kf);
 #pragma unroll
-                for (int e = 0; e < EPL; ++e) dot = fmaf(qf[e], kf[u][e], dot);
+                for (int e = 0; e < EPL; ++e) dot = fmaf(qf[e], kf[e], dot);
             }
 #pragma unroll
             for (int off = 1; off < LPK; off <<= 1) dot += __shfl_xor(dot, off, MLLM_WAVE);
             if (valid[u]) {
+                float vf[EPL];
+                Vec16<T>::widen(vraw[u], vf);
                 const float mn = fmaxf(m, dot);
                 const float a = exp2f(m - mn), pj = exp2f(dot - mn);
                 l = l * a + pj;
 #pragma unroll
-                for (int e = 0; e < EPL; ++e) o[e] = o[e] * a + pj * vf[u][e];
+                for (int e = 0; e < EPL; ++e) o[e] = o[e] * a + pj * vf[e];
                 m = mn;
             }
         }

@@ -112,19 +112,21 @@ gemm_bf16_mfma(const bf16_t* __restrict__ A, int lda, const bf16_t* __restrict__
 
 
 // ---------------------------------------------------------------------------------------------
-// Few rows (decode): M <= 64. The product is bound by streaming W once, so the grid is
-// one workgroup per 16 output columns and the wavefronts of a workgroup split K
-// (wavefront w takes the 32-wide k steps w, w+NW, ...), each lane loading 16 contiguous
-// bytes of a weight row straight from global memory into the B operand of
-// v_mfma_f32_16x16x32_bf16. The activations (a few KB, shared by all workgroups) are read
-// from L2, or, with LN_FUSED, normalised from the fp32 stream into LDS first: LayerNorm
+// Few rows (decode): M <= 64. The product is bound by streaming W once. Each lane loads 16
+// contiguous bytes of a weight row straight from global memory into the B operand of
+// v_mfma_f32_16x16x32_bf16; a 16-column tile of the output is one MFMA accumulator per 16 rows.
+//   SPLIT_K:  one workgroup per 16-column tile, its wavefronts split K (wavefront w takes the
+//             32-wide k steps w, w+NW, ...) and their partial sums are added in LDS in a fixed
+//             order: for the narrow products, where tiles alone are too few to fill the chip.
+//   !SPLIT_K: one wavefront per tile over the whole of K (wide products such as the logits head).
+// The activations (a few KB, shared by all workgroups) are read from L2, or, with LN_FUSED,
+// normalised from the fp32 stream into LDS first: LayerNorm
 // (/root/reference/src/kernels/layernorm.cu:32-49) fused into the product that follows it.
-// Partial sums of the wavefronts are added in LDS in a fixed order.
 // ---------------------------------------------------------------------------------------------
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 
-template <int MT, bool LN_FUSED>
-__global__ void __launch_bounds__(1024)
+template <int MT, bool LN_FUSED, bool SPLIT_K>
+__global__ void __launch_bounds__(LN_FUSED ? 512 : 1024)
 gemm_bf16_skinny(const void* __restrict__ Ain, int lda, const bf16_t* __restrict__ W, int ldw,
                  const float* __restrict__ bias, void* __restrict__ C, int ldc, int M, int N, int K, int mode,
                  const float* __restrict__ gamma, const float* __restrict__ beta, float eps,
@@ -132,13 +134,17 @@ gemm_bf16_skinny(const void* __restrict__ Ain, int lda, const bf16_t* __restrict
     extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
     const int tid = threadIdx.x, wave = tid / 64, lane = tid % 64;
     const int nw = blockDim.x / 64;
-    const int n0 = blockIdx.x * 16;
     const int row16 = lane % 16, kq = lane / 16;
+    const int n0 = (SPLIT_K ? blockIdx.x : blockIdx.x * nw + wave) * 16;
+    const int k_first = SPLIT_K ? wave * 32 : 0;      // first k step of this wavefront
+    const int k_step = SPLIT_K ? nw * 32 : 32;
+    const size_t red_bytes = SPLIT_K ? static_cast<size_t>(nw) * MT * 256 * sizeof(float) : 0;
     float* red = reinterpret_cast<float*>(smem_raw);                       // [nw][MT][256]
-    bf16_t* a_s = reinterpret_cast<bf16_t*>(smem_raw + static_cast<size_t>(nw) * MT * 256 * sizeof(float));
+    bf16_t* a_s = reinterpret_cast<bf16_t*>(smem_raw + red_bytes);         // [16*MT][K+8]
     const int a_stride = K + 8;
     const int n = n0 + row16;
-    const bf16_t* wrow = W + static_cast<size_t>(n < N ? n : 0) * ldw;
+    const bool n_ok = n < N;
+    const bf16_t* wrow = W + static_cast<size_t>(n_ok ? n : 0) * ldw;
     const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
 
     f32x4 acc[MT];
@@ -152,26 +158,28 @@ gemm_bf16_skinny(const void* __restrict__ Ain, int lda, const bf16_t* __restrict
     if (LN_FUSED) {
 #pragma unroll
         for (int u = 0; u < PRE; ++u) {
-            const int k = (wave + u * nw) * 32 + 8 * kq;
-            bpre[u] = (k < K && n < N) ? *reinterpret_cast<const bf16x8*>(wrow + k) : zero;
+            const int k = k_first + u * k_step + 8 * kq;
+            bpre[u] = (k < K && n_ok) ? *reinterpret_cast<const bf16x8*>(wrow + k) : zero;
         }
-    }
-
-    if (LN_FUSED) {
-        // one wavefront per row: mean, then variance of the centred values, all in fp32
+        // one wavefront per row: the row lives in registers (K <= 2048, K % 4 == 0), mean, then
+        // variance of the centred values, all in fp32
         const float* x = static_cast<const float*>(Ain);
+        const int nq = K / 4;
+        const float4* g4 = reinterpret_cast<const float4*>(gamma);
+        const float4* b4 = reinterpret_cast<const float4*>(beta);
         for (int m = wave; m < 16 * MT; m += nw) {
             bf16_t* dst = a_s + static_cast<size_t>(m) * a_stride;
             if (m < M) {
-                // the row lives in registers: one pass over memory (K <= 2048, K % 4 == 0)
                 const float4* xr = reinterpret_cast<const float4*>(x + static_cast<size_t>(rows ? rows[m] : m) * lda);
-                const int nq = K / 4;
-                float4 v[8];
+                float4 v[8], gg[8], bb[8];
                 float s = 0.f;
 #pragma unroll
                 for (int u = 0; u < 8; ++u) {
                     const int i = lane + 64 * u;
-                    v[u] = i < nq ? xr[i] : make_float4(0.f, 0.f, 0.f, 0.f);
+                    const bool in = i < nq;
+                    v[u] = in ? xr[i] : make_float4(0.f, 0.f, 0.f, 0.f);
+                    gg[u] = in ? g4[i] : make_float4(0.f, 0.f, 0.f, 0.f);
+                    bb[u] = (in && beta) ? b4[i] : make_float4(0.f, 0.f, 0.f, 0.f);
                     s += (v[u].x + v[u].y) + (v[u].z + v[u].w);
                 }
                 const float mean = wave_sum(s) / static_cast<float>(K);
@@ -184,18 +192,14 @@ gemm_bf16_skinny(const void* __restrict__ Ain, int lda, const bf16_t* __restrict
                     }
                 }
                 const float inv = 1.0f / sqrtf(wave_sum(q) / static_cast<float>(K) + eps);
-                const float4* g4 = reinterpret_cast<const float4*>(gamma);
-                const float4* b4 = reinterpret_cast<const float4*>(beta);
 #pragma unroll
                 for (int u = 0; u < 8; ++u) {
                     const int i = lane + 64 * u;
                     if (i < nq) {
-                        const float4 gg = g4[i];
-                        const float4 bb = beta ? b4[i] : make_float4(0.f, 0.f, 0.f, 0.f);
-                        bf16_t r0 = float_to_bf16((v[u].x - mean) * inv * gg.x + bb.x);
-                        bf16_t r1 = float_to_bf16((v[u].y - mean) * inv * gg.y + bb.y);
-                        bf16_t r2 = float_to_bf16((v[u].z - mean) * inv * gg.z + bb.z);
-                        bf16_t r3 = float_to_bf16((v[u].w - mean) * inv * gg.w + bb.w);
+                        bf16_t r0 = float_to_bf16((v[u].x - mean) * inv * gg[u].x + bb[u].x);
+                        bf16_t r1 = float_to_bf16((v[u].y - mean) * inv * gg[u].y + bb[u].y);
+                        bf16_t r2 = float_to_bf16((v[u].z - mean) * inv * gg[u].z + bb[u].z);
+                        bf16_t r3 = float_to_bf16((v[u].w - mean) * inv * gg[u].w + bb[u].w);
                         uint2 pk;
                         pk.x = static_cast<uint32_t>(r0.bits) | (static_cast<uint32_t>(r1.bits) << 16);
                         pk.y = static_cast<uint32_t>(r2.bits) | (static_cast<uint32_t>(r3.bits) << 16);
@@ -210,13 +214,13 @@ gemm_bf16_skinny(const void* __restrict__ Ain, int lda, const bf16_t* __restrict
     }
 
     const bf16_t* A = static_cast<const bf16_t*>(Ain);
-
-    int k_start = wave * 32;
+    int k_start = k_first;
     if (LN_FUSED) {
 #pragma unroll
         for (int u = 0; u < PRE; ++u) {
-            const int k = (wave + u * nw) * 32 + 8 * kq;
-            if ((wave + u * nw) * 32 < K) {
+            const int kb = k_first + u * k_step;
+            if (kb < K) {
+                const int k = kb + 8 * kq;
                 const bool kin = k < K;
 #pragma unroll
                 for (int i = 0; i < MT; ++i) {
@@ -226,13 +230,13 @@ gemm_bf16_skinny(const void* __restrict__ Ain, int lda, const bf16_t* __restrict
                 }
             }
         }
-        k_start = (wave + PRE * nw) * 32;
+        k_start = k_first + PRE * k_step;
     }
-#pragma unroll 4
-    for (int k0 = k_start; k0 < K; k0 += nw * 32) {
+#pragma unroll 8
+    for (int k0 = k_start; k0 < K; k0 += k_step) {
         const int k = k0 + 8 * kq;
         const bool kin = k < K;
-        bf16x8 b = (kin && n < N) ? *reinterpret_cast<const bf16x8*>(wrow + k) : zero;
+        bf16x8 b = (kin && n_ok) ? *reinterpret_cast<const bf16x8*>(wrow + k) : zero;
 #pragma unroll
         for (int i = 0; i < MT; ++i) {
             const int m = i * 16 + row16;
@@ -242,50 +246,71 @@ gemm_bf16_skinny(const void* __restrict__ Ain, int lda, const bf16_t* __restrict
             acc[i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, acc[i], 0, 0, 0);
         }
     }
+    // accumulator layout of the 16x16 tile: register r of lane l holds row 4*(l/16) + r, column l%16
+    if (!SPLIT_K) {
+        if (!n_ok) return;
+        const float bv = bias ? bias[n] : 0.f;
+#pragma unroll
+        for (int i = 0; i < MT; ++i)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int m = i * 16 + 4 * kq + r;
+                if (m < M) epilogue<bf16_t>(mode, acc[i][r], bv, C, static_cast<size_t>(m) * ldc + n);
+            }
+        return;
+    }
 #pragma unroll
     for (int i = 0; i < MT; ++i)
 #pragma unroll
         for (int r = 0; r < 4; ++r) red[(static_cast<size_t>(wave) * MT + i) * 256 + r * 64 + lane] = acc[i][r];
     __syncthreads();
-    // accumulator layout of the 16x16 tile: register r of lane l holds row 4*(l/16) + r, column l%16
     for (int idx = tid; idx < MT * 256; idx += blockDim.x) {
         const int i = idx / 256, r = (idx % 256) / 64, l = idx % 64;
+        const int m = i * 16 + 4 * (l / 16) + r, nn = n0 + l % 16;
+        if (m >= M || nn >= N) continue;
+        const float bv = bias ? bias[nn] : 0.f;
         float v = 0.f;
         for (int w = 0; w < nw; ++w) v += red[(static_cast<size_t>(w) * MT + i) * 256 + r * 64 + l];
-        const int m = i * 16 + 4 * (l / 16) + r, nn = n0 + l % 16;
-        if (m < M && nn < N) epilogue<bf16_t>(mode, v, bias ? bias[nn] : 0.f, C, static_cast<size_t>(m) * ldc + nn);
+        epilogue<bf16_t>(mode, v, bv, C, static_cast<size_t>(m) * ldc + nn);
     }
-}
-
-static int skinny_waves(int N, int K) {
-    const int blocks = (N + 15) / 16, steps = (K + 31) / 32;
-    int nw = 16;
-    while (nw > 1 && (nw * 3 > steps || blocks * nw > 4096)) nw >>= 1;
-    return nw;
 }
 
 template <bool LN_FUSED>
 static int launch_skinny(const void* A, int lda, const bf16_t* W, int ldw, const float* bias, void* C, int ldc,
                          int M, int N, int K, int mode, const float* gamma, const float* beta, float eps,
                          const int* rows, hipStream_t stream) {
-    const int mt = (M + 15) / 16, nw = skinny_waves(N, K);
-    const dim3 grid((N + 15) / 16), block(nw * 64);
-    size_t smem = static_cast<size_t>(nw) * mt * 256 * sizeof(float);
+    const int mt = (M + 15) / 16;
+    const int tiles = (N + 15) / 16, steps = (K + 31) / 32;
+    const bool split_k = tiles < 1024;
+    int nw;
+    if (split_k) {
+        nw = LN_FUSED ? 8 : 16;
+        while (nw > 1 && nw * 3 > steps) nw >>= 1;
+    } else {
+        nw = 4;
+    }
+    const dim3 grid(split_k ? tiles : (tiles + nw - 1) / nw), block(nw * 64);
+    size_t smem = split_k ? static_cast<size_t>(nw) * mt * 256 * sizeof(float) : 0;
     if (LN_FUSED) {
         smem += static_cast<size_t>(16) * mt * (K + 8) * sizeof(bf16_t);
-        if (K > 2048 || (reinterpret_cast<uintptr_t>(A) & 15) || lda % 4 != 0) return -2;
+        if (K > 2048 || (reinterpret_cast<uintptr_t>(A) & 15) || lda % 4 != 0 ||
+            (reinterpret_cast<uintptr_t>(gamma) & 15) || (reinterpret_cast<uintptr_t>(beta) & 15))
+            return -2;
     }
     if (smem > 64 * 1024) return -2;
-#define SKINNY_CASE(MTV)                                                                                  \
-    case MTV:                                                                                             \
-        gemm_bf16_skinny<MTV, LN_FUSED><<<grid, block, smem, stream>>>(A, lda, W, ldw, bias, C, ldc, M, N, K, \
-                                                                       mode, gamma, beta, eps, rows);     \
+#define SKINNY_LAUNCH(MTV, SK)                                                                              \
+    gemm_bf16_skinny<MTV, LN_FUSED, SK><<<grid, block, smem, stream>>>(A, lda, W, ldw, bias, C, ldc, M, N, K, \
+                                                                       mode, gamma, beta, eps, rows)
+#define SKINNY_CASE(MTV)                                                   \
+    case MTV:                                                              \
+        if (split_k) SKINNY_LAUNCH(MTV, true); else SKINNY_LAUNCH(MTV, false); \
         break;
     switch (mt) {
         SKINNY_CASE(1) SKINNY_CASE(2) SKINNY_CASE(3) SKINNY_CASE(4)
         default: return -2;
     }
 #undef SKINNY_CASE
+#undef SKINNY_LAUNCH
     return 0;
 }
 
