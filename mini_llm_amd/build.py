@@ -47,6 +47,7 @@ LIBRARIES: Dict[str, dict] = {
     "gemm_bf16": {"kind": "hip", "sources": ["kernels/gemm_bf16.hip"], "headers": ["kernels/common.h"]},
     "attention": {"kind": "hip", "sources": ["kernels/attention.hip"], "headers": ["kernels/common.h"]},
     "attention_decode": {"kind": "hip", "sources": ["kernels/attention_decode.hip"], "headers": ["kernels/common.h"]},
+    "attention_prefill": {"kind": "hip", "sources": ["kernels/attention_prefill.hip"], "headers": ["kernels/common.h"]},
     "sampling": {"kind": "hip", "sources": ["kernels/sampling.hip"], "headers": ["kernels/common.h"]},
 }
 

@@ -1,0 +1,229 @@
+// Prefill attention on the MFMA units of gfx950, bf16 with fp32 softmax: causal (optionally
+// windowed) attention of a step's query rows over the paged cache. A workgroup takes 64
+// consecutive queries of one sequence and one head; its four wavefronts take 16 queries each
+// and walk the keys in tiles of 64, which are gathered through the block table into LDS (keys
+// row-major, values transposed), so prompt portions that start anywhere read what earlier steps
+// left in the pages.
+//
+// Everything is computed transposed so that a lane owns ONE query:
+//   S^T = K Q^T   (A = 16 keys x 32 dims from LDS, B = the lane's query fragment, held in registers)
+//   O^T = V^T P^T (A = 16 dims x 32 keys from the transposed values, B = P^T straight from the S^T
+//                  accumulators: the MFMA's k index may be permuted freely as long as both operands
+//                  agree, so no shuffle or LDS round trip is needed)
+// The running maximum and sum are then scalars per lane, merged over the four lane groups with two
+// DPP steps. Recurrence: /root/reference/src/kernels/prefill/flashattention.cu:129-178, in base 2;
+// the reference reads its keys from the step's own qkv buffer (:99-111) and so cannot continue a
+// prompt from the cache.
+#include "common.h"
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+#define PF_BM 64
+#define PF_BN 64
+#define PF_VT_STRIDE 66     // elements per transposed value row: 33 words, so staging writes spread over banks
+
+union Frag8 {
+    bf16x8 v;
+    uint4 q;
+    uint32_t w[4];
+    uint16_t h[8];
+};
+
+__device__ __forceinline__ uint32_t pack_bf16x2(float a, float b) {
+    return static_cast<uint32_t>(float_to_bf16(a).bits) | (static_cast<uint32_t>(float_to_bf16(b).bits) << 16);
+}
+
+template <int DH>
+__global__ void __launch_bounds__(256)
+prefill_attention_kernel(const bf16_t* __restrict__ q, int q_stride, int q_col,
+                         const bf16_t* __restrict__ k_pages, const bf16_t* __restrict__ v_pages, int kv_dim,
+                         const int* __restrict__ block_tables, int max_blocks,
+                         const int* __restrict__ cu_q, const int* __restrict__ ctx_len, int n_seqs,
+                         int n_heads, int n_kv_heads, int page_size, float scale_log2e, int window,
+                         bf16_t* __restrict__ out, int out_stride) {
+    constexpr int KS = DH / 32;            // k steps of S^T
+    constexpr int DT = DH / 16;            // 16-dim tiles of O^T
+    constexpr int KSTRIDE = DH + 8;
+    __shared__ __attribute__((aligned(16))) bf16_t Ks[PF_BN * KSTRIDE];
+    __shared__ __attribute__((aligned(16))) bf16_t Vt[DH * PF_VT_STRIDE];
+
+    // which sequence and which of its 64-query tiles this workgroup has
+    int tile = blockIdx.x, b = 0, q_begin = 0, q_len = 0;
+    for (; b < n_seqs; ++b) {
+        q_begin = cu_q[b];
+        q_len = cu_q[b + 1] - q_begin;
+        const int nt = (q_len + PF_BM - 1) / PF_BM;
+        if (tile < nt) break;
+        tile -= nt;
+    }
+    if (b >= n_seqs) return;               // surplus workgroup; the whole workgroup leaves
+
+    const int h = blockIdx.y, hk = h / (n_heads / n_kv_heads);
+    const int tid = threadIdx.x, wave = tid / 64, lane = tid % 64;
+    const int G = lane / 16, c16 = lane % 16;
+    const int start = ctx_len[b] - q_len;                 // position of the step's first query
+    const int q0 = tile * PF_BM;
+    const int qi = q0 + wave * 16 + c16;                  // this lane's query within the step's rows
+    const bool q_ok = qi < q_len;
+    const int p = start + qi;                             // its position
+    const int p_first = start + q0;
+    const int p_last = start + min(q0 + PF_BM, q_len) - 1;
+    const int k_lo = (window > 0 && p_first - window + 1 > 0) ? p_first - window + 1 : 0;
+    const int* table = block_tables + static_cast<size_t>(b) * max_blocks;
+    const bool pow2 = (page_size & (page_size - 1)) == 0;
+    const int shift = pow2 ? __ffs(page_size) - 1 : 0;
+    auto page_row = [&](int j) -> size_t {
+        return pow2 ? ((static_cast<size_t>(table[j >> shift]) << shift) + (j & (page_size - 1)))
+                    : (static_cast<size_t>(table[j / page_size]) * page_size + j % page_size);
+    };
+
+    Frag8 qf[KS];
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+        qf[ks].q = make_uint4(0, 0, 0, 0);
+        if (q_ok)
+            qf[ks].q = *reinterpret_cast<const uint4*>(q + static_cast<size_t>(q_begin + qi) * q_stride + q_col +
+                                                       h * DH + 32 * ks + 8 * G);
+    }
+
+    float m = -INFINITY, l = 0.f;
+    f32x4 o[DT];
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) o[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
+    const size_t kv_col = static_cast<size_t>(hk) * DH;
+
+    for (int kt = k_lo / PF_BN; kt <= p_last / PF_BN; ++kt) {
+        const int j_base = kt * PF_BN;
+        __syncthreads();                     // the previous tile's readers are done
+        // keys, row-major: 16-byte chunks
+        for (int it = tid; it < PF_BN * (DH / 8); it += 256) {
+            const int row = it / (DH / 8), ch = it % (DH / 8);
+            const int j = j_base + row;
+            uint4 v = make_uint4(0, 0, 0, 0);
+            if (j >= k_lo && j <= p_last) v = *reinterpret_cast<const uint4*>(k_pages + page_row(j) * kv_dim + kv_col + 8 * ch);
+            *reinterpret_cast<uint4*>(Ks + row * KSTRIDE + 8 * ch) = v;
+        }
+        // values, transposed: a thread takes 8 dims of two neighbouring keys and writes 8 words
+        for (int it = tid; it < (PF_BN / 2) * (DH / 8); it += 256) {
+            const int jp = it / (DH / 8), ch = it % (DH / 8);
+            const int j0 = j_base + 2 * jp;
+            Frag8 v0, v1;
+            v0.q = make_uint4(0, 0, 0, 0);
+            v1.q = make_uint4(0, 0, 0, 0);
+            if (j0 >= k_lo && j0 <= p_last) v0.q = *reinterpret_cast<const uint4*>(v_pages + page_row(j0) * kv_dim + kv_col + 8 * ch);
+            if (j0 + 1 >= k_lo && j0 + 1 <= p_last) v1.q = *reinterpret_cast<const uint4*>(v_pages + page_row(j0 + 1) * kv_dim + kv_col + 8 * ch);
+#pragma unroll
+            for (int i = 0; i < 8; ++i)
+                *reinterpret_cast<uint32_t*>(Vt + (8 * ch + i) * PF_VT_STRIDE + 2 * jp) =
+                    static_cast<uint32_t>(v0.h[i]) | (static_cast<uint32_t>(v1.h[i]) << 16);
+        }
+        __syncthreads();
+
+        // S^T: s[nt][r] is the score of key j_base + 16*nt + 4*G + r with this lane's query
+        float s[4][4];
+        float tile_max = -INFINITY;
+#pragma unroll
+        for (int nt = 0; nt < 4; ++nt) {
+            f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks) {
+                const bf16x8 a = *reinterpret_cast<const bf16x8*>(Ks + (16 * nt + c16) * KSTRIDE + 32 * ks + 8 * G);
+                acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, qf[ks].v, acc, 0, 0, 0);
+            }
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int j = j_base + 16 * nt + 4 * G + r;
+                const bool seen = q_ok && j <= p && (window <= 0 || j > p - window);
+                s[nt][r] = seen ? acc[r] * scale_log2e : -INFINITY;
+                tile_max = fmaxf(tile_max, s[nt][r]);
+            }
+        }
+        // the four lane groups of a query agree on the maximum
+        tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 16, MLLM_WAVE));
+        tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 32, MLLM_WAVE));
+        const float m_new = fmaxf(m, tile_max);
+        const float m_use = (m_new == -INFINITY) ? 0.f : m_new;      // nothing seen yet: all weights are 0
+        const float alpha = exp2f(m - m_use);
+        m = m_new;
+        float psum = 0.f;
+#pragma unroll
+        for (int nt = 0; nt < 4; ++nt)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                s[nt][r] = exp2f(s[nt][r] - m_use);
+                psum += s[nt][r];
+            }
+        l = l * alpha + psum;                 // this lane's share of the sum; merged over groups at the end
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) o[dt][r] *= alpha;
+
+        // O^T += V^T P^T over two slabs of 32 keys. k slot i of lane group G stands for key
+        // 32*slab + 4*G + i (i < 4) or 32*slab + 16 + 4*G + i - 4 (i >= 4) in both operands.
+#pragma unroll
+        for (int slab = 0; slab < 2; ++slab) {
+            Frag8 pf;
+            pf.w[0] = pack_bf16x2(s[2 * slab][0], s[2 * slab][1]);
+            pf.w[1] = pack_bf16x2(s[2 * slab][2], s[2 * slab][3]);
+            pf.w[2] = pack_bf16x2(s[2 * slab + 1][0], s[2 * slab + 1][1]);
+            pf.w[3] = pack_bf16x2(s[2 * slab + 1][2], s[2 * slab + 1][3]);
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt) {
+                const uint32_t* vrow = reinterpret_cast<const uint32_t*>(Vt + (16 * dt + c16) * PF_VT_STRIDE);
+                Frag8 vf;
+                vf.w[0] = vrow[16 * slab + 2 * G];
+                vf.w[1] = vrow[16 * slab + 2 * G + 1];
+                vf.w[2] = vrow[16 * slab + 8 + 2 * G];
+                vf.w[3] = vrow[16 * slab + 8 + 2 * G + 1];
+                o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf.v, pf.v, o[dt], 0, 0, 0);
+            }
+        }
+    }
+    l += __shfl_xor(l, 16, MLLM_WAVE);
+    l += __shfl_xor(l, 32, MLLM_WAVE);
+    if (!q_ok) return;
+    const float inv = 1.0f / l;
+    // o[dt][r] is dimension 16*dt + 4*G + r of this lane's query
+    bf16_t* orow = out + static_cast<size_t>(q_begin + qi) * out_stride + h * DH;
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) {
+        uint2 pk;
+        pk.x = pack_bf16x2(o[dt][0] * inv, o[dt][1] * inv);
+        pk.y = pack_bf16x2(o[dt][2] * inv, o[dt][3] * inv);
+        *reinterpret_cast<uint2*>(orow + 16 * dt + 4 * G) = pk;
+    }
+}
+
+extern "C" {
+
+// n_tiles_upper: an upper bound of the number of 64-query tiles, sum over sequences of
+// ceil(q_len / 64) (e.g. n_tokens / 64 + n_seqs); surplus workgroups leave at once.
+// Returns 0, a HIP error code, or -1 when the head size is not 32, 64 or 128.
+int mllm_prefill_attention_bf16(const void* q, int q_stride, int q_col, const void* k_pages, const void* v_pages,
+                                int kv_dim, const int* block_tables, int max_blocks, const int* cu_q,
+                                const int* ctx_len, int n_seqs, int n_tiles_upper, int n_heads, int n_kv_heads,
+                                int head_dim, int page_size, float scale, int window, void* out, int out_stride,
+                                hipStream_t stream) {
+    if (n_seqs <= 0 || n_tiles_upper <= 0) return 0;
+    if (n_heads % n_kv_heads != 0 || n_heads > 65535) return -1;
+    const dim3 grid(n_tiles_upper, n_heads);
+    const float sl2 = scale * 1.44269504088896340736f;
+#define PF_CASE(D)                                                                                          \
+    case D:                                                                                                 \
+        prefill_attention_kernel<D><<<grid, 256, 0, stream>>>(                                              \
+            (const bf16_t*)q, q_stride, q_col, (const bf16_t*)k_pages, (const bf16_t*)v_pages, kv_dim,      \
+            block_tables, max_blocks, cu_q, ctx_len, n_seqs, n_heads, n_kv_heads, page_size, sl2, window,   \
+            (bf16_t*)out, out_stride);                                                                      \
+        break;
+    switch (head_dim) {
+        PF_CASE(32) PF_CASE(64) PF_CASE(128)
+        default: return -1;
+    }
+#undef PF_CASE
+    MLLM_LAUNCH_CHECK();
+    return 0;
+}
+
+}  // extern "C"

@@ -288,6 +288,20 @@ def paged_attention(q: torch.Tensor, q_col: int, n_heads: int, n_kv_heads: int, 
             _dt(q), _stream()),
             "decode_attention")
         return out
+    if (q.dtype == torch.bfloat16 and head_dim in (32, 64, 128) and max_q_len > 1
+            and cu_q is not None and ctx_len is not None):
+        # prompt portions: tiles of 64 queries on the matrix cores
+        B = block_tables.shape[0]
+        _i32(cu_q, "cu_q", B + 1)
+        _i32(ctx_len, "ctx_len", B)
+        if out.data_ptr() % 16 or (out.stride(0) * esz) % 8:
+            raise KernelError("attention output rows must be 8-byte aligned")
+        lib = load_library("attention_prefill")
+        _check(lib.mllm_prefill_attention_bf16(
+            _p(q), q.stride(0), q_col, _p(k_pages), _p(v_pages), kv_dim, _p(block_tables), block_tables.shape[1],
+            _p(cu_q), _p(ctx_len), B, T // 64 + B, n_heads, n_kv_heads, head_dim, page_size,
+            ctypes.c_float(scale), int(window or 0), _p(out), out.stride(0), _stream()), "prefill_attention")
+        return out
     lib = load_library("attention")
     _check(lib.mllm_paged_attention_generic(
         _p(q), q.stride(0), q_col, _p(k_pages), _p(v_pages), kv_dim, _p(block_tables), block_tables.shape[1],

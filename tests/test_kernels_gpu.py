@@ -237,8 +237,10 @@ def _attention_case(ops, dtype, H, Hkv, dh, page, seqs, window, gen, boost=None)
     positions = torch.tensor(positions, dtype=torch.int32)
     scale = dh ** -0.5
     out = torch.zeros(T, H * dh, dtype=dtype, device=DEV)
+    cu = torch.tensor([0] + list(torch.tensor([n for _, n in seqs]).cumsum(0)), dtype=torch.int32)
     ops.paged_attention(q.to(DEV), 8, H, Hkv, dh, kp.to(DEV), vp.to(DEV), page, tables.to(DEV),
                         token_seq.to(DEV), positions.to(DEV), scale, window, out,
+                        cu_q=cu.to(DEV), ctx_len=torch.tensor(ctx, dtype=torch.int32).to(DEV),
                         max_q_len=max(n for _, n in seqs), max_ctx_len=max(ctx))
     ref = torch.zeros(T, H * dh, dtype=torch.float64)
     plain_ops.paged_attention(q, 8, H, Hkv, dh, kp, vp, page, tables, token_seq, positions, scale, window, ref)
@@ -318,6 +320,18 @@ def test_paged_attention_appends_own_keys(ops, dtype, H, Hkv, dh, page, qlens):
     assert (out.cpu().double() - ref).abs().max() <= _tol(dtype, 2)
     written = slots.long()
     assert torch.equal(kp_d.cpu()[written], ref_kp[written]) and torch.equal(vp_d.cpu()[written], ref_vp[written])
+
+
+@pytest.mark.parametrize("H,Hkv,dh,page", [(12, 12, 64, 16), (3, 3, 32, 8), (4, 1, 128, 16), (6, 2, 64, 4)])
+@pytest.mark.parametrize("window", [0, 1, 50, 64, 200])
+def test_paged_attention_prefill_tiles(ops, H, Hkv, dh, page, window):
+    """The MFMA prefill kernel (bf16, head sizes 32/64/128): query tiles that are full, partial and
+    a single row; portions that start mid-sequence and mid-page; windows that cut inside a key tile."""
+    g = torch.Generator().manual_seed(H + dh + window)
+    seqs = [(0, 64), (0, 150), (37, 2), (100, 129), (511, 1), (64, 64), (5, 63)]
+    out, ref = _attention_case(ops, torch.bfloat16, H, Hkv, dh, page, seqs, window, g)
+    assert torch.isfinite(out).all()
+    assert (out - ref).abs().max() <= _tol(torch.bfloat16, 2)
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
