@@ -45,7 +45,7 @@ __device__ __forceinline__ void merge_state(float& m, float& l, float (&o)[N], f
                                             const float (&o2)[N]) {
     const float mn = fmaxf(m, m2);
     if (mn == -INFINITY) return;          // both empty
-    const float a = exp2f(m - mn), b = exp2f(m2 - mn);
+    const float a = fast_exp2(m - mn), b = fast_exp2(m2 - mn);
     l = l * a + l2 * b;
 #pragma unroll
     for (int e = 0; e < N; ++e) o[e] = o[e] * a + o2[e] * b;
@@ -151,7 +151,7 @@ decode_attention_kernel(const T* __restrict__ q, int q_stride, int q_col,
                 float vf[EPL];
                 Vec16<T>::widen(vraw[u], vf);
                 const float mn = fmaxf(m, dot);
-                const float a = exp2f(m - mn), pj = exp2f(dot - mn);
+                const float a = fast_exp2(m - mn), pj = fast_exp2(dot - mn);
                 l = l * a + pj;
 #pragma unroll
                 for (int e = 0; e < EPL; ++e) o[e] = o[e] * a + pj * vf[e];

@@ -16,11 +16,14 @@
 // prompt from the cache.
 #include "common.h"
 
+#include <type_traits>
+
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 
 #define PF_BM 64
 #define PF_BN 64
+#define PF_TABLE_LDS 2048   // block-table entries staged in LDS (longer tables are read from memory)
 #define PF_VT_STRIDE 66     // elements per transposed value row: 33 words, so staging writes spread over banks
 
 union Frag8 {
@@ -29,10 +32,6 @@ union Frag8 {
     uint32_t w[4];
     uint16_t h[8];
 };
-
-__device__ __forceinline__ uint32_t pack_bf16x2(float a, float b) {
-    return static_cast<uint32_t>(float_to_bf16(a).bits) | (static_cast<uint32_t>(float_to_bf16(b).bits) << 16);
-}
 
 template <int DH>
 __global__ void __launch_bounds__(256)
@@ -47,6 +46,7 @@ prefill_attention_kernel(const bf16_t* __restrict__ q, int q_stride, int q_col,
     constexpr int KSTRIDE = DH + 8;
     __shared__ __attribute__((aligned(16))) bf16_t Ks[PF_BN * KSTRIDE];
     __shared__ __attribute__((aligned(16))) bf16_t Vt[DH * PF_VT_STRIDE];
+    __shared__ int sm_table[PF_TABLE_LDS];
 
     // which sequence and which of its 64-query tiles this workgroup has
     int tile = blockIdx.x, b = 0, q_begin = 0, q_len = 0;
@@ -70,12 +70,16 @@ prefill_attention_kernel(const bf16_t* __restrict__ q, int q_stride, int q_col,
     const int p_first = start + q0;
     const int p_last = start + min(q0 + PF_BM, q_len) - 1;
     const int k_lo = (window > 0 && p_first - window + 1 > 0) ? p_first - window + 1 : 0;
-    const int* table = block_tables + static_cast<size_t>(b) * max_blocks;
-    const bool pow2 = (page_size & (page_size - 1)) == 0;
-    const int shift = pow2 ? __ffs(page_size) - 1 : 0;
+    // The sequence's block table goes to LDS first: the gathers below then depend on an LDS read,
+    // not on a global load that would have to be waited for in front of every key load.
+    // (The host passes page sizes that are powers of two and tables of at most PF_TABLE_LDS blocks.)
+    const int* gtable = block_tables + static_cast<size_t>(b) * max_blocks;
+    const int shift = __ffs(page_size) - 1;
+    const int n_blocks_needed = (p_last >> shift) + 1;
+    for (int i = tid; i < n_blocks_needed; i += 256) sm_table[i] = gtable[i];
+    __syncthreads();
     auto page_row = [&](int j) -> size_t {
-        return pow2 ? ((static_cast<size_t>(table[j >> shift]) << shift) + (j & (page_size - 1)))
-                    : (static_cast<size_t>(table[j / page_size]) * page_size + j % page_size);
+        return (static_cast<size_t>(sm_table[j >> shift]) << shift) + (j & (page_size - 1));
     };
 
     Frag8 qf[KS];
@@ -93,33 +97,81 @@ prefill_attention_kernel(const bf16_t* __restrict__ q, int q_stride, int q_col,
     for (int dt = 0; dt < DT; ++dt) o[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
     const size_t kv_col = static_cast<size_t>(hk) * DH;
 
-    for (int kt = k_lo / PF_BN; kt <= p_last / PF_BN; ++kt) {
+    // Tiles are fetched into registers one tile ahead, so the gather of the next keys and values
+    // is in flight while the matrix cores work on the current ones.
+    constexpr int K_ITEMS = (PF_BN * (DH / 8) + 255) / 256;          // 16-byte key chunks per thread
+    constexpr int V_ITEMS = ((PF_BN / 2) * (DH / 8) + 255) / 256;    // (key pair, 8 dims) items per thread
+    struct TileRegs {
+        uint4 rk[K_ITEMS], rv0[V_ITEMS], rv1[V_ITEMS];
+    };
+    TileRegs regs_a, regs_b;
+    auto fetch = [&](TileRegs& t, int kt) {
+        uint4 (&rk)[K_ITEMS] = t.rk;
+        uint4 (&rv0)[V_ITEMS] = t.rv0;
+        uint4 (&rv1)[V_ITEMS] = t.rv1;
         const int j_base = kt * PF_BN;
-        __syncthreads();                     // the previous tile's readers are done
-        // keys, row-major: 16-byte chunks
-        for (int it = tid; it < PF_BN * (DH / 8); it += 256) {
+#pragma unroll
+        for (int u = 0; u < K_ITEMS; ++u) {
+            const int it = tid + u * 256;
             const int row = it / (DH / 8), ch = it % (DH / 8);
             const int j = j_base + row;
-            uint4 v = make_uint4(0, 0, 0, 0);
-            if (j >= k_lo && j <= p_last) v = *reinterpret_cast<const uint4*>(k_pages + page_row(j) * kv_dim + kv_col + 8 * ch);
-            *reinterpret_cast<uint4*>(Ks + row * KSTRIDE + 8 * ch) = v;
+            // always a held page (clamped); what lies outside [k_lo, p_last] becomes zero afterwards
+            const int jc = min(max(j, k_lo), p_last);
+            rk[u] = make_uint4(0, 0, 0, 0);
+            if (K_ITEMS * 256 == PF_BN * (DH / 8) || it < PF_BN * (DH / 8)) {
+                const uint4 v = *reinterpret_cast<const uint4*>(k_pages + page_row(jc) * kv_dim + kv_col + 8 * ch);
+                if (j == jc) rk[u] = v;
+            }
         }
-        // values, transposed: a thread takes 8 dims of two neighbouring keys and writes 8 words
-        for (int it = tid; it < (PF_BN / 2) * (DH / 8); it += 256) {
+#pragma unroll
+        for (int u = 0; u < V_ITEMS; ++u) {
+            const int it = tid + u * 256;
             const int jp = it / (DH / 8), ch = it % (DH / 8);
             const int j0 = j_base + 2 * jp;
-            Frag8 v0, v1;
-            v0.q = make_uint4(0, 0, 0, 0);
-            v1.q = make_uint4(0, 0, 0, 0);
-            if (j0 >= k_lo && j0 <= p_last) v0.q = *reinterpret_cast<const uint4*>(v_pages + page_row(j0) * kv_dim + kv_col + 8 * ch);
-            if (j0 + 1 >= k_lo && j0 + 1 <= p_last) v1.q = *reinterpret_cast<const uint4*>(v_pages + page_row(j0 + 1) * kv_dim + kv_col + 8 * ch);
-#pragma unroll
-            for (int i = 0; i < 8; ++i)
-                *reinterpret_cast<uint32_t*>(Vt + (8 * ch + i) * PF_VT_STRIDE + 2 * jp) =
-                    static_cast<uint32_t>(v0.h[i]) | (static_cast<uint32_t>(v1.h[i]) << 16);
+            rv0[u] = make_uint4(0, 0, 0, 0);
+            rv1[u] = make_uint4(0, 0, 0, 0);
+            if (V_ITEMS * 256 == (PF_BN / 2) * (DH / 8) || it < (PF_BN / 2) * (DH / 8)) {
+                const int jc0 = min(max(j0, k_lo), p_last), jc1 = min(max(j0 + 1, k_lo), p_last);
+                const uint4 a = *reinterpret_cast<const uint4*>(v_pages + page_row(jc0) * kv_dim + kv_col + 8 * ch);
+                const uint4 c = *reinterpret_cast<const uint4*>(v_pages + page_row(jc1) * kv_dim + kv_col + 8 * ch);
+                if (j0 == jc0) rv0[u] = a;
+                if (j0 + 1 == jc1) rv1[u] = c;
+            }
         }
-        __syncthreads();
+    };
+    auto stage = [&](const TileRegs& t) {
+        // keys row-major; values transposed: 8 dims of two neighbouring keys become 8 words
+        const uint4 (&rk)[K_ITEMS] = t.rk;
+        const uint4 (&rv0)[V_ITEMS] = t.rv0;
+        const uint4 (&rv1)[V_ITEMS] = t.rv1;
+#pragma unroll
+        for (int u = 0; u < K_ITEMS; ++u) {
+            const int it = tid + u * 256;
+            if (it < PF_BN * (DH / 8))
+                *reinterpret_cast<uint4*>(Ks + (it / (DH / 8)) * KSTRIDE + 8 * (it % (DH / 8))) = rk[u];
+        }
+#pragma unroll
+        for (int u = 0; u < V_ITEMS; ++u) {
+            const int it = tid + u * 256;
+            if (it < (PF_BN / 2) * (DH / 8)) {
+                const int jp = it / (DH / 8), ch = it % (DH / 8);
+                Frag8 v0, v1;
+                v0.q = rv0[u];
+                v1.q = rv1[u];
+#pragma unroll
+                for (int i = 0; i < 8; ++i)
+                    *reinterpret_cast<uint32_t*>(Vt + (8 * ch + i) * PF_VT_STRIDE + 2 * jp) =
+                        static_cast<uint32_t>(v0.h[i]) | (static_cast<uint32_t>(v1.h[i]) << 16);
+            }
+        }
+    };
 
+    // Positions of this wavefront's first and last query: a key tile that every one of them sees
+    // in full needs no mask.
+    const int pw_min = start + q0 + wave * 16, pw_max = pw_min + 15;
+    auto compute = [&](int kt, auto masked_tag) {
+        constexpr bool MASKED = decltype(masked_tag)::value;
+        const int j_base = kt * PF_BN;
         // S^T: s[nt][r] is the score of key j_base + 16*nt + 4*G + r with this lane's query
         float s[4][4];
         float tile_max = -INFINITY;
@@ -133,9 +185,12 @@ prefill_attention_kernel(const bf16_t* __restrict__ q, int q_stride, int q_col,
             }
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
-                const int j = j_base + 16 * nt + 4 * G + r;
-                const bool seen = q_ok && j <= p && (window <= 0 || j > p - window);
-                s[nt][r] = seen ? acc[r] * scale_log2e : -INFINITY;
+                s[nt][r] = acc[r] * scale_log2e;
+                if (MASKED) {
+                    const int j = j_base + 16 * nt + 4 * G + r;
+                    const bool seen = q_ok && j <= p && (window <= 0 || j > p - window);
+                    if (!seen) s[nt][r] = -INFINITY;
+                }
                 tile_max = fmaxf(tile_max, s[nt][r]);
             }
         }
@@ -144,14 +199,14 @@ prefill_attention_kernel(const bf16_t* __restrict__ q, int q_stride, int q_col,
         tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 32, MLLM_WAVE));
         const float m_new = fmaxf(m, tile_max);
         const float m_use = (m_new == -INFINITY) ? 0.f : m_new;      // nothing seen yet: all weights are 0
-        const float alpha = exp2f(m - m_use);
+        const float alpha = fast_exp2(m - m_use);
         m = m_new;
         float psum = 0.f;
 #pragma unroll
         for (int nt = 0; nt < 4; ++nt)
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
-                s[nt][r] = exp2f(s[nt][r] - m_use);
+                s[nt][r] = fast_exp2(s[nt][r] - m_use);
                 psum += s[nt][r];
             }
         l = l * alpha + psum;                 // this lane's share of the sum; merged over groups at the end
@@ -180,6 +235,30 @@ prefill_attention_kernel(const bf16_t* __restrict__ q, int q_stride, int q_col,
                 o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf.v, pf.v, o[dt], 0, 0, 0);
             }
         }
+    };
+
+    auto run_tile = [&](int kt) {
+        const int j_base = kt * PF_BN;
+        const bool full = j_base + PF_BN - 1 <= pw_min && (window <= 0 || j_base > pw_max - window);
+        if (full) compute(kt, std::false_type{}); else compute(kt, std::true_type{});
+    };
+
+    // Two register sets, each fetched two tiles ahead of its use.
+    const int kt_first = k_lo / PF_BN, kt_last = p_last / PF_BN;
+    fetch(regs_a, kt_first);
+    if (kt_first + 1 <= kt_last) fetch(regs_b, kt_first + 1);
+    for (int kt = kt_first; kt <= kt_last; kt += 2) {
+        lds_barrier();                     // the previous tile's readers are done
+        stage(regs_a);
+        lds_barrier();
+        if (kt + 2 <= kt_last) fetch(regs_a, kt + 2);
+        run_tile(kt);
+        if (kt + 1 > kt_last) break;
+        lds_barrier();
+        stage(regs_b);
+        lds_barrier();
+        if (kt + 3 <= kt_last) fetch(regs_b, kt + 3);
+        run_tile(kt + 1);
     }
     l += __shfl_xor(l, 16, MLLM_WAVE);
     l += __shfl_xor(l, 32, MLLM_WAVE);
@@ -200,7 +279,8 @@ extern "C" {
 
 // n_tiles_upper: an upper bound of the number of 64-query tiles, sum over sequences of
 // ceil(q_len / 64) (e.g. n_tokens / 64 + n_seqs); surplus workgroups leave at once.
-// Returns 0, a HIP error code, or -1 when the head size is not 32, 64 or 128.
+// Returns 0, a HIP error code, or -1 when the head size is not 32, 64 or 128, the page size is no
+// power of two, or a block table has more than PF_TABLE_LDS entries.
 int mllm_prefill_attention_bf16(const void* q, int q_stride, int q_col, const void* k_pages, const void* v_pages,
                                 int kv_dim, const int* block_tables, int max_blocks, const int* cu_q,
                                 const int* ctx_len, int n_seqs, int n_tiles_upper, int n_heads, int n_kv_heads,
@@ -208,6 +288,7 @@ int mllm_prefill_attention_bf16(const void* q, int q_stride, int q_col, const vo
                                 hipStream_t stream) {
     if (n_seqs <= 0 || n_tiles_upper <= 0) return 0;
     if (n_heads % n_kv_heads != 0 || n_heads > 65535) return -1;
+    if ((page_size & (page_size - 1)) != 0 || max_blocks > PF_TABLE_LDS) return -1;
     const dim3 grid(n_tiles_upper, n_heads);
     const float sl2 = scale * 1.44269504088896340736f;
 #define PF_CASE(D)                                                                                          \

@@ -26,18 +26,21 @@ __device__ __forceinline__ float bf16_to_float(bf16_t v) {
     return __uint_as_float(static_cast<uint32_t>(v.bits) << 16);
 }
 
-// Round to nearest, ties to even; NaN stays NaN.
+// Round to nearest, ties to even (the hardware conversion of gfx950, v_cvt_pk_bf16_f32).
 __device__ __forceinline__ bf16_t float_to_bf16(float f) {
-    uint32_t u = __float_as_uint(f);
     bf16_t r;
-    if ((u & 0x7fffffffu) > 0x7f800000u) {
-        r.bits = static_cast<uint16_t>((u >> 16) | 0x0040u);
-    } else {
-        u += 0x7fffu + ((u >> 16) & 1u);
-        r.bits = static_cast<uint16_t>(u >> 16);
-    }
+    r.bits = __builtin_bit_cast(uint16_t, static_cast<__bf16>(f));
     return r;
 }
+// Two values converted by one instruction; `a` lands in the low half.
+__device__ __forceinline__ uint32_t pack_bf16x2(float a, float b) {
+    typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+    const bf16x2_t v = {static_cast<__bf16>(a), static_cast<__bf16>(b)};
+    return __builtin_bit_cast(uint32_t, v);
+}
+// 2^x by the hardware instruction alone: for arguments <= 0, where results below the normal
+// range may flush to zero (softmax weights).
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
 __device__ __forceinline__ float to_float(float v) { return v; }
 __device__ __forceinline__ float to_float(bf16_t v) { return bf16_to_float(v); }
@@ -78,6 +81,15 @@ __device__ __forceinline__ void wave_lds_sync() {
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
+// Workgroup barrier that orders LDS traffic only. __syncthreads() also waits for every
+// outstanding global load, which would drain the loads a kernel has deliberately in flight for
+// a later tile; this one leaves them in flight (their registers are waited for where first used).
+__device__ __forceinline__ void lds_barrier() {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
 }
 
 // Block-wide sum for blocks of up to 1024 threads; `scratch` holds >= 16 floats of LDS.

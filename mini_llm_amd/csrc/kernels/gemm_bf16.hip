@@ -70,9 +70,9 @@ gemm_bf16_mfma(const bf16_t* __restrict__ A, int lda, const bf16_t* __restrict__
 
     fetch(0);
     for (int k0 = 0; k0 < K; k0 += BK) {
-        __syncthreads();            // readers of the previous tile are done
+        lds_barrier();              // readers of the previous tile are done
         stage();
-        __syncthreads();
+        lds_barrier();
         if (k0 + BK < K) fetch(k0 + BK);
 #pragma unroll
         for (int ks = 0; ks < BK / 16; ++ks) {
@@ -314,7 +314,12 @@ static int launch_skinny(const void* A, int lda, const bf16_t* W, int ldw, const
     return 0;
 }
 
+static int g_big_tile_min_blocks = 512;
+
 extern "C" {
+
+// Tuning knob: the 128x128 tile is used when it yields at least this many workgroups.
+void mllm_gemm_bf16_set_big_tile_min_blocks(int n) { g_big_tile_min_blocks = n; }
 
 // Returns 0, a HIP error code, or -1 when K or the row strides are not multiples of 8
 // elements or a base pointer is not 16-byte aligned.
@@ -332,7 +337,7 @@ int mllm_gemm_bf16(const void* A, int lda, const void* W, int ldw, const float* 
     } else if (M <= 32) {
         dim3 grid((N + 127) / 128, (M + 31) / 32);
         gemm_bf16_mfma<1, 4, 1, 1><<<grid, 256, 0, stream>>>(a, lda, w, ldw, bias, C, ldc, M, N, K, mode);
-    } else if (blocks(128, 128) >= 512) {
+    } else if (blocks(128, 128) >= g_big_tile_min_blocks) {
         dim3 grid((N + 127) / 128, (M + 127) / 128);
         gemm_bf16_mfma<2, 2, 2, 2><<<grid, 256, 0, stream>>>(a, lda, w, ldw, bias, C, ldc, M, N, K, mode);
     } else {
