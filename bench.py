@@ -20,10 +20,15 @@ HBM_PEAK = 8.0e12                                   # bytes/s
 MFMA_PEAK = {"bfloat16": 2.5e15, "float32": 157.3e12}
 
 
-def small_config(n_layer):
-    # BASELINE.json configs[2]: GPT-2 small sizes
-    return dict(architectures=["GPT2LMHeadModel"], model_type="gpt2", n_layer=n_layer, n_embd=768, n_head=12,
-                n_inner=3072, vocab_size=50257, n_positions=1024, layer_norm_epsilon=1e-5,
+SIZES = {   # BASELINE.json configs[2..4]: n_layer, n_embd, n_head, n_inner
+    "gpt2-small": (12, 768, 12, 3072), "gpt2-medium": (24, 1024, 16, 4096), "gpt2-xl": (48, 1600, 25, 6400),
+}
+
+
+def small_config(n_layer, size="gpt2-small"):
+    full_layers, d, h, f = SIZES[size]
+    return dict(architectures=["GPT2LMHeadModel"], model_type="gpt2", n_layer=n_layer or full_layers, n_embd=d,
+                n_head=h, n_inner=f, vocab_size=50257, n_positions=1024, layer_norm_epsilon=1e-5,
                 activation_function="gelu_new", eos_token_id=50256, bos_token_id=50256)
 
 
@@ -112,7 +117,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=32)
     ap.add_argument("--batch", type=int, default=8)
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
-    ap.add_argument("--layers", type=int, default=12, help="fewer layers than GPT-2 small's 12 are named in config")
+    ap.add_argument("--layers", type=int, default=0, help="fewer layers than the size has (named in config)")
+    ap.add_argument("--size", default="gpt2-small", choices=sorted(SIZES), help="layer sizes (default: configs[2])")
     ap.add_argument("--prompt-len", type=int, default=512)
     ap.add_argument("--no-points", action="store_true", help="skip the batch-1/64 and prefill measurements")
     args = ap.parse_args()
@@ -122,7 +128,7 @@ def main():
     import torch
     from mini_llm_amd import write_random_model
 
-    cfg = small_config(args.layers)
+    cfg = small_config(args.layers, args.size)
     esz = 2 if args.dtype == "bfloat16" else 4
     steps = min(args.steps, cfg["n_positions"] - args.prompt_len - args.warmup - 2 - 64)
     with tempfile.TemporaryDirectory() as d:
@@ -131,13 +137,13 @@ def main():
         bytes_step = weight_bytes(cfg, esz) + args.batch * mean_ctx * kv_bytes_per_token(cfg, esz)
         achieved = bytes_step / step_s
         rec = {
-            "metric": "decode tok/s at batch 8 (GPT-2 small sizes, 512-token prompts, context to 1024)",
+            "metric": f"decode tok/s at batch {args.batch} ({args.size} sizes, {args.prompt_len}-token prompts)",
             "value": round(tps, 1), "unit": "tok/s", "n_gpus": 1, "steps": steps, "warmup": args.warmup,
             "ms_per_step": round(step_s * 1e3, 4), "higher_is_better": True, "scaling": "weak",
             "vs_baseline": None, "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
             "data": "synthetic (random weights seed 2, uniform random token ids)",
-            "config": {"model": "gpt2-small-sizes", "n_layer": cfg["n_layer"], "n_layer_full": 12,
-                       "n_embd": cfg["n_embd"], "n_head": cfg["n_head"], "head_dim": 64,
+            "config": {"model": args.size + "-sizes", "n_layer": cfg["n_layer"], "n_layer_full": SIZES[args.size][0],
+                       "n_embd": cfg["n_embd"], "n_head": cfg["n_head"], "head_dim": cfg["n_embd"] // cfg["n_head"],
                        "n_inner": cfg["n_inner"], "vocab_size": cfg["vocab_size"],
                        "n_positions": cfg["n_positions"], "global_batch": args.batch,
                        "prompt_len": args.prompt_len, "seq_len": cfg["n_positions"],

@@ -13,15 +13,13 @@
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 
-#define BK 64
-#define LDS_STRIDE (BK + 8)   // 144-byte rows: 16-byte reads of 32 consecutive rows hit distinct banks
-
-template <int WM, int WN, int TM, int TN>
+template <int WM, int WN, int TM, int TN, int BK, int DEPTH = 3>
 __global__ void __launch_bounds__(256)
 gemm_bf16_mfma(const bf16_t* __restrict__ A, int lda, const bf16_t* __restrict__ W, int ldw,
                const float* __restrict__ bias, void* __restrict__ C, int ldc, int M, int N, int K, int mode) {
     static_assert(WM * WN == 4, "four wavefronts per block");
     constexpr int BM = WM * TM * 32, BN = WN * TN * 32;
+    constexpr int LDS_STRIDE = BK + 8;   // rows of 16-byte reads from 32 consecutive rows hit distinct banks
     constexpr int A_CHUNKS = BM * (BK / 8) / 256, W_CHUNKS = BN * (BK / 8) / 256;
     __shared__ __attribute__((aligned(16))) bf16_t As[BM * LDS_STRIDE];
     __shared__ __attribute__((aligned(16))) bf16_t Ws[BN * LDS_STRIDE];
@@ -38,42 +36,41 @@ gemm_bf16_mfma(const bf16_t* __restrict__ A, int lda, const bf16_t* __restrict__
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
-    uint4 ra[A_CHUNKS], rw[W_CHUNKS];
-    auto fetch = [&](int k0) {
+    // Global loads run DEPTH-1 tiles ahead of the MFMAs in rotating register sets: one tile of
+    // compute is far shorter than the memory latency, so several tiles must be in flight.
+    struct TileRegs {
+        uint4 ra[A_CHUNKS], rw[W_CHUNKS];
+    };
+    TileRegs regs[DEPTH];
+    auto fetch = [&](TileRegs& t, int k0) {
 #pragma unroll
         for (int i = 0; i < A_CHUNKS; ++i) {
             const int c = tid + i * 256, row = c / (BK / 8), kc = c % (BK / 8);
             const int m = m0 + row, k = k0 + kc * 8;
-            ra[i] = (m < M && k < K) ? *reinterpret_cast<const uint4*>(A + static_cast<size_t>(m) * lda + k)
-                                     : make_uint4(0, 0, 0, 0);
+            t.ra[i] = (m < M && k < K) ? *reinterpret_cast<const uint4*>(A + static_cast<size_t>(m) * lda + k)
+                                       : make_uint4(0, 0, 0, 0);
         }
 #pragma unroll
         for (int i = 0; i < W_CHUNKS; ++i) {
             const int c = tid + i * 256, row = c / (BK / 8), kc = c % (BK / 8);
             const int n = n0 + row, k = k0 + kc * 8;
-            rw[i] = (n < N && k < K) ? *reinterpret_cast<const uint4*>(W + static_cast<size_t>(n) * ldw + k)
-                                     : make_uint4(0, 0, 0, 0);
+            t.rw[i] = (n < N && k < K) ? *reinterpret_cast<const uint4*>(W + static_cast<size_t>(n) * ldw + k)
+                                       : make_uint4(0, 0, 0, 0);
         }
     };
-    auto stage = [&]() {
+    auto stage = [&](const TileRegs& t) {
 #pragma unroll
         for (int i = 0; i < A_CHUNKS; ++i) {
             const int c = tid + i * 256, row = c / (BK / 8), kc = c % (BK / 8);
-            *reinterpret_cast<uint4*>(As + row * LDS_STRIDE + kc * 8) = ra[i];
+            *reinterpret_cast<uint4*>(As + row * LDS_STRIDE + kc * 8) = t.ra[i];
         }
 #pragma unroll
         for (int i = 0; i < W_CHUNKS; ++i) {
             const int c = tid + i * 256, row = c / (BK / 8), kc = c % (BK / 8);
-            *reinterpret_cast<uint4*>(Ws + row * LDS_STRIDE + kc * 8) = rw[i];
+            *reinterpret_cast<uint4*>(Ws + row * LDS_STRIDE + kc * 8) = t.rw[i];
         }
     };
-
-    fetch(0);
-    for (int k0 = 0; k0 < K; k0 += BK) {
-        lds_barrier();              // readers of the previous tile are done
-        stage();
-        lds_barrier();
-        if (k0 + BK < K) fetch(k0 + BK);
+    auto compute = [&]() {
 #pragma unroll
         for (int ks = 0; ks < BK / 16; ++ks) {
             const int kofs = ks * 16 + 8 * (lane / 32);
@@ -89,6 +86,24 @@ gemm_bf16_mfma(const bf16_t* __restrict__ A, int lda, const bf16_t* __restrict__
 #pragma unroll
                 for (int j = 0; j < TN; ++j)
                     acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[i], b[j], acc[i][j], 0, 0, 0);
+        }
+    };
+
+    const int nk = (K + BK - 1) / BK;
+#pragma unroll
+    for (int d = 0; d < DEPTH - 1; ++d)
+        if (d < nk) fetch(regs[d], d * BK);
+    for (int kt = 0; kt < nk; kt += DEPTH) {
+#pragma unroll
+        for (int d = 0; d < DEPTH; ++d) {
+            const int t = kt + d;
+            if (t < nk) {
+                lds_barrier();              // readers of the previous tile are done
+                stage(regs[d]);
+                lds_barrier();
+                if (t + DEPTH - 1 < nk) fetch(regs[(d + DEPTH - 1) % DEPTH], (t + DEPTH - 1) * BK);
+                compute();
+            }
         }
     }
 
@@ -315,11 +330,13 @@ static int launch_skinny(const void* A, int lda, const bf16_t* W, int ldw, const
 }
 
 static int g_big_tile_min_blocks = 512;
+static int g_variant = 0;
 
 extern "C" {
 
 // Tuning knob: the 128x128 tile is used when it yields at least this many workgroups.
 void mllm_gemm_bf16_set_big_tile_min_blocks(int n) { g_big_tile_min_blocks = n; }
+void mllm_gemm_bf16_set_variant(int v) { g_variant = v; }
 
 // Returns 0, a HIP error code, or -1 when K or the row strides are not multiples of 8
 // elements or a base pointer is not 16-byte aligned.
@@ -331,18 +348,29 @@ int mllm_gemm_bf16(const void* A, int lda, const void* W, int ldw, const float* 
     const bf16_t* a = static_cast<const bf16_t*>(A);
     const bf16_t* w = static_cast<const bf16_t*>(W);
     auto blocks = [&](int bm, int bn) { return static_cast<long>((M + bm - 1) / bm) * ((N + bn - 1) / bn); };
-    if (M <= 64 && launch_skinny<false>(A, lda, w, ldw, bias, C, ldc, M, N, K, mode, nullptr, nullptr, 0.f,
+    if (g_variant > 0) {
+        // tuning only: force one tile shape
+#define VAR(ID, WM_, WN_, TM_, TN_, BK_, D_)                                                                  \
+        if (g_variant == ID) {                                                                              \
+            dim3 grid((N + WN_ * TN_ * 32 - 1) / (WN_ * TN_ * 32), (M + WM_ * TM_ * 32 - 1) / (WM_ * TM_ * 32)); \
+            gemm_bf16_mfma<WM_, WN_, TM_, TN_, BK_, D_><<<grid, 256, 0, stream>>>(a, lda, w, ldw, bias, C, ldc, M, N, K, mode); \
+        }
+        VAR(1, 2, 2, 1, 1, 64, 2) VAR(2, 2, 2, 1, 1, 64, 3) VAR(3, 2, 2, 1, 1, 64, 4) VAR(4, 2, 2, 2, 1, 64, 3)
+        VAR(5, 2, 2, 1, 2, 64, 3) VAR(6, 2, 2, 2, 2, 64, 3) VAR(7, 2, 2, 2, 2, 32, 4) VAR(8, 2, 2, 2, 2, 64, 2)
+        VAR(9, 2, 2, 2, 1, 32, 4) VAR(10, 2, 2, 1, 1, 32, 4)
+#undef VAR
+    } else if (M <= 64 && launch_skinny<false>(A, lda, w, ldw, bias, C, ldc, M, N, K, mode, nullptr, nullptr, 0.f,
                                         nullptr, stream) == 0) {
         // few rows: weight-streaming kernel
     } else if (M <= 32) {
         dim3 grid((N + 127) / 128, (M + 31) / 32);
-        gemm_bf16_mfma<1, 4, 1, 1><<<grid, 256, 0, stream>>>(a, lda, w, ldw, bias, C, ldc, M, N, K, mode);
+        gemm_bf16_mfma<1, 4, 1, 1, 64><<<grid, 256, 0, stream>>>(a, lda, w, ldw, bias, C, ldc, M, N, K, mode);
     } else if (blocks(128, 128) >= g_big_tile_min_blocks) {
         dim3 grid((N + 127) / 128, (M + 127) / 128);
-        gemm_bf16_mfma<2, 2, 2, 2><<<grid, 256, 0, stream>>>(a, lda, w, ldw, bias, C, ldc, M, N, K, mode);
+        gemm_bf16_mfma<2, 2, 2, 2, 64><<<grid, 256, 0, stream>>>(a, lda, w, ldw, bias, C, ldc, M, N, K, mode);
     } else {
         dim3 grid((N + 63) / 64, (M + 63) / 64);
-        gemm_bf16_mfma<2, 2, 1, 1><<<grid, 256, 0, stream>>>(a, lda, w, ldw, bias, C, ldc, M, N, K, mode);
+        gemm_bf16_mfma<2, 2, 1, 1, 64><<<grid, 256, 0, stream>>>(a, lda, w, ldw, bias, C, ldc, M, N, K, mode);
     }
     MLLM_LAUNCH_CHECK();
     return 0;

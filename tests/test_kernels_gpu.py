@@ -87,7 +87,8 @@ def test_layernorm_constant_row_gives_beta(ops):
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("M,N,K", [(67, 79, 40), (5, 2304, 768), (1, 1000, 96), (130, 320, 96),
-                                   (9, 73, 320), (200, 50257, 64), (33, 96, 3072), (257, 257, 264)])
+                                   (9, 73, 320), (200, 50257, 64), (33, 96, 3072), (257, 257, 264),
+                                   (300, 4800, 1600), (100, 1600, 6400)])
 @pytest.mark.parametrize("epi", ["store", "gelu_tanh", "gelu_erf", "add_residual", "store_f32"])
 def test_linear(ops, dtype, M, N, K, epi):
     if N == 50257 and epi not in ("store_f32", "store"):
@@ -113,7 +114,8 @@ def test_linear(ops, dtype, M, N, K, epi):
 
 
 @pytest.mark.parametrize("M", [1, 8, 16, 17, 48, 64])
-@pytest.mark.parametrize("N,K", [(2304, 768), (768, 3072), (1000, 96), (50257, 768), (72, 1600)])
+@pytest.mark.parametrize("N,K", [(2304, 768), (768, 3072), (1000, 96), (50257, 768), (72, 1600), (4800, 1600),
+                                 (1600, 6400), (1024, 4096)])
 def test_linear_bf16_few_rows(ops, M, N, K):
     """The weight-streaming kernel of decode steps (M <= 64), every wavefront count and m-tile count."""
     g = torch.Generator().manual_seed(M + N + K)
@@ -132,7 +134,7 @@ def test_linear_bf16_few_rows(ops, M, N, K):
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("M,N,K", [(1, 2304, 768), (8, 3072, 768), (16, 320, 96), (5, 200, 1600), (17, 96, 64),
-                                   (3, 64, 4096)])
+                                   (3, 64, 4096), (16, 6400, 1600), (9, 50257, 1024), (16, 3072, 1024)])
 @pytest.mark.parametrize("epi", ["store", "gelu_tanh", "gelu_erf", "store_f32"])
 def test_ln_linear(ops, dtype, M, N, K, epi):
     """LayerNorm fused into the product (bf16, few rows) and its unfused form give the plain result."""
