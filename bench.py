@@ -121,6 +121,7 @@ def main():
     ap.add_argument("--size", default="gpt2-small", choices=sorted(SIZES), help="layer sizes (default: configs[2])")
     ap.add_argument("--prompt-len", type=int, default=512)
     ap.add_argument("--no-points", action="store_true", help="skip the batch-1/64 and prefill measurements")
+    ap.add_argument("--prefill-only", action="store_true", help="measure only the 2,048-token prefill (profiling)")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
@@ -133,6 +134,11 @@ def main():
     steps = min(args.steps, cfg["n_positions"] - args.prompt_len - args.warmup - 2 - 64)
     with tempfile.TemporaryDirectory() as d:
         write_random_model(dict(cfg), d, seed=2)
+        if args.prefill_only:
+            ptps, pdt, flops = prefill_run(d, args.dtype, cfg)
+            print(json.dumps({"metric": "prefill tok/s at 2,048 tokens", "value": round(ptps, 1), "unit": "tok/s",
+                              "ms": round(pdt * 1e3, 4), "frac": round(flops / pdt / MFMA_PEAK[args.dtype], 5)}))
+            return 0
         tps, step_s, mean_ctx = decode_run(d, args.dtype, args.batch, args.prompt_len, steps, args.warmup, cfg)
         bytes_step = weight_bytes(cfg, esz) + args.batch * mean_ctx * kv_bytes_per_token(cfg, esz)
         achieved = bytes_step / step_s

@@ -13,20 +13,71 @@
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 
-template <int WM, int WN, int TM, int TN, int BK, int DEPTH = 3>
-__global__ void __launch_bounds__(256)
+#define N_XCD 8       // accelerator dies of an MI355X, each with its own L2
+
+// ---------------------------------------------------------------------------------------------
+// Many rows (prefill): WM x WN wavefronts, each TM x TN MFMA tiles of 32x32. LDS is double
+// buffered (one barrier per k tile), global loads run DEPTH-1 tiles ahead in rotating register
+// sets, per-thread pointers only advance, and blocks that lie fully inside the matrices take an
+// edge-free path chosen at compile time. The weight fragment is the MFMA's A operand, so a lane's
+// accumulator registers hold 4 consecutive columns of one output row: the epilogue stores them
+// as one 8- or 16-byte access.
+// ---------------------------------------------------------------------------------------------
+template <int MODE>
+__device__ __forceinline__ void store4(void* C, size_t idx, const float (&v)[4], bool vec, int n_left) {
+    // v: 4 consecutive columns of one row, bias already added; n_left: columns that exist (1..4)
+    float o[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e)
+        o[e] = MODE == EPI_GELU_TANH ? gelu_tanh(v[e]) : MODE == EPI_GELU_ERF ? gelu_erf(v[e]) : v[e];
+    if (MODE == EPI_ADD_RESIDUAL || MODE == EPI_STORE_F32) {
+        float* c = static_cast<float*>(C) + idx;
+        if (vec && n_left >= 4) {
+            float4 r = make_float4(o[0], o[1], o[2], o[3]);
+            if (MODE == EPI_ADD_RESIDUAL) {
+                const float4 old = *reinterpret_cast<const float4*>(c);
+                r.x += old.x; r.y += old.y; r.z += old.z; r.w += old.w;
+            }
+            *reinterpret_cast<float4*>(c) = r;
+        } else {
+            for (int e = 0; e < n_left; ++e) c[e] = (MODE == EPI_ADD_RESIDUAL ? c[e] : 0.f) + o[e];
+        }
+    } else {
+        bf16_t* c = static_cast<bf16_t*>(C) + idx;
+        if (vec && n_left >= 4) {
+            uint2 pk;
+            pk.x = pack_bf16x2(o[0], o[1]);
+            pk.y = pack_bf16x2(o[2], o[3]);
+            *reinterpret_cast<uint2*>(c) = pk;
+        } else {
+            for (int e = 0; e < n_left; ++e) c[e] = float_to_bf16(o[e]);
+        }
+    }
+}
+
+template <int WM, int WN, int TM, int TN, int BKP, int DEPTH, bool EDGE, int MODE>
+__global__ void __launch_bounds__(WM * WN * 64)
 gemm_bf16_mfma(const bf16_t* __restrict__ A, int lda, const bf16_t* __restrict__ W, int ldw,
-               const float* __restrict__ bias, void* __restrict__ C, int ldc, int M, int N, int K, int mode) {
-    static_assert(WM * WN == 4, "four wavefronts per block");
+               const float* __restrict__ bias, void* __restrict__ C, int ldc, int M, int N, int K,
+               int tiles_m, int tiles_n, int xm, int xn) {
+    constexpr int NT = WM * WN * 64;
     constexpr int BM = WM * TM * 32, BN = WN * TN * 32;
-    constexpr int LDS_STRIDE = BK + 8;   // rows of 16-byte reads from 32 consecutive rows hit distinct banks
-    constexpr int A_CHUNKS = BM * (BK / 8) / 256, W_CHUNKS = BN * (BK / 8) / 256;
-    __shared__ __attribute__((aligned(16))) bf16_t As[BM * LDS_STRIDE];
-    __shared__ __attribute__((aligned(16))) bf16_t Ws[BN * LDS_STRIDE];
+    constexpr int STRIDE = BKP + 8;
+    constexpr int CPR = BKP / 8;                      // 16-byte chunks per row
+    constexpr int A_CH = (BM * CPR + NT - 1) / NT, W_CH = (BN * CPR + NT - 1) / NT;
+    __shared__ __attribute__((aligned(16))) bf16_t As[2][BM * STRIDE];
+    __shared__ __attribute__((aligned(16))) bf16_t Ws[2][BN * STRIDE];
 
     const int tid = threadIdx.x, wave = tid / 64, lane = tid % 64;
     const int wm = wave / WN, wn = wave % WN;
-    const int m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
+    // Workgroups are handed to the 8 XCDs round-robin and every XCD has an L2 of its own, so the
+    // tiles of one XCD (workgroup id % 8) form one compact rectangle of the output: the rows of A
+    // and W it needs then fit in its L2 instead of every XCD streaming both matrices.
+    const int xcd = blockIdx.x % N_XCD, local = blockIdx.x / N_XCD;
+    const int rect_m = (tiles_m + xm - 1) / xm, rect_n = (tiles_n + xn - 1) / xn;
+    const int tm = (xcd / xn) * rect_m + local / rect_n, tn = (xcd % xn) * rect_n + local % rect_n;
+    if (local >= rect_m * rect_n || tm >= tiles_m || tn >= tiles_n) return;      // padding of the grid
+    const int m0 = tm * BM, n0 = tn * BN;
 
     f32x16 acc[TM][TN];
 #pragma unroll
@@ -36,95 +87,141 @@ gemm_bf16_mfma(const bf16_t* __restrict__ A, int lda, const bf16_t* __restrict__
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
-    // Global loads run DEPTH-1 tiles ahead of the MFMAs in rotating register sets: one tile of
-    // compute is far shorter than the memory latency, so several tiles must be in flight.
+    // per-thread chunk pointers (row fixed, k advances by BKP per tile) and LDS offsets
+    const bf16_t* pa[A_CH];
+    const bf16_t* pw[W_CH];
+    int la[A_CH], lw[W_CH];
+    bool va[A_CH], vw[W_CH];
+#pragma unroll
+    for (int i = 0; i < A_CH; ++i) {
+        const int c = tid + i * NT, row = c / CPR, kc = c % CPR;
+        va[i] = (BM * CPR % NT == 0 || c < BM * CPR) && (!EDGE || m0 + row < M);
+        pa[i] = A + static_cast<size_t>(va[i] ? m0 + row : 0) * lda + kc * 8;
+        la[i] = row * STRIDE + kc * 8;
+    }
+#pragma unroll
+    for (int i = 0; i < W_CH; ++i) {
+        const int c = tid + i * NT, row = c / CPR, kc = c % CPR;
+        vw[i] = (BN * CPR % NT == 0 || c < BN * CPR) && (!EDGE || n0 + row < N);
+        pw[i] = W + static_cast<size_t>(vw[i] ? n0 + row : 0) * ldw + kc * 8;
+        lw[i] = row * STRIDE + kc * 8;
+    }
     struct TileRegs {
-        uint4 ra[A_CHUNKS], rw[W_CHUNKS];
+        uint4 ra[A_CH], rw[W_CH];
     };
     TileRegs regs[DEPTH];
     auto fetch = [&](TileRegs& t, int k0) {
 #pragma unroll
-        for (int i = 0; i < A_CHUNKS; ++i) {
-            const int c = tid + i * 256, row = c / (BK / 8), kc = c % (BK / 8);
-            const int m = m0 + row, k = k0 + kc * 8;
-            t.ra[i] = (m < M && k < K) ? *reinterpret_cast<const uint4*>(A + static_cast<size_t>(m) * lda + k)
-                                       : make_uint4(0, 0, 0, 0);
+        for (int i = 0; i < A_CH; ++i) {
+            const int kc8 = (tid + i * NT) % CPR * 8;
+            const bool ok = va[i] && (!EDGE || k0 + kc8 < K);
+            t.ra[i] = ok ? *reinterpret_cast<const uint4*>(pa[i] + k0) : make_uint4(0, 0, 0, 0);
         }
 #pragma unroll
-        for (int i = 0; i < W_CHUNKS; ++i) {
-            const int c = tid + i * 256, row = c / (BK / 8), kc = c % (BK / 8);
-            const int n = n0 + row, k = k0 + kc * 8;
-            t.rw[i] = (n < N && k < K) ? *reinterpret_cast<const uint4*>(W + static_cast<size_t>(n) * ldw + k)
-                                       : make_uint4(0, 0, 0, 0);
+        for (int i = 0; i < W_CH; ++i) {
+            const int kc8 = (tid + i * NT) % CPR * 8;
+            const bool ok = vw[i] && (!EDGE || k0 + kc8 < K);
+            t.rw[i] = ok ? *reinterpret_cast<const uint4*>(pw[i] + k0) : make_uint4(0, 0, 0, 0);
         }
     };
-    auto stage = [&](const TileRegs& t) {
+    auto stage = [&](const TileRegs& t, int buf) {
 #pragma unroll
-        for (int i = 0; i < A_CHUNKS; ++i) {
-            const int c = tid + i * 256, row = c / (BK / 8), kc = c % (BK / 8);
-            *reinterpret_cast<uint4*>(As + row * LDS_STRIDE + kc * 8) = t.ra[i];
-        }
+        for (int i = 0; i < A_CH; ++i)
+            if (BM * CPR % NT == 0 || tid + i * NT < BM * CPR) *reinterpret_cast<uint4*>(&As[buf][la[i]]) = t.ra[i];
 #pragma unroll
-        for (int i = 0; i < W_CHUNKS; ++i) {
-            const int c = tid + i * 256, row = c / (BK / 8), kc = c % (BK / 8);
-            *reinterpret_cast<uint4*>(Ws + row * LDS_STRIDE + kc * 8) = t.rw[i];
-        }
+        for (int i = 0; i < W_CH; ++i)
+            if (BN * CPR % NT == 0 || tid + i * NT < BN * CPR) *reinterpret_cast<uint4*>(&Ws[buf][lw[i]]) = t.rw[i];
     };
-    auto compute = [&]() {
+    const int a_off = (wm * TM * 32 + lane % 32) * STRIDE + 8 * (lane / 32);
+    const int w_off = (wn * TN * 32 + lane % 32) * STRIDE + 8 * (lane / 32);
+    auto compute = [&](int buf) {
 #pragma unroll
-        for (int ks = 0; ks < BK / 16; ++ks) {
-            const int kofs = ks * 16 + 8 * (lane / 32);
+        for (int ks = 0; ks < BKP / 16; ++ks) {
             bf16x8 a[TM], b[TN];
 #pragma unroll
             for (int i = 0; i < TM; ++i)
-                a[i] = *reinterpret_cast<const bf16x8*>(As + ((wm * TM + i) * 32 + lane % 32) * LDS_STRIDE + kofs);
+                a[i] = *reinterpret_cast<const bf16x8*>(&As[buf][a_off + i * 32 * STRIDE + ks * 16]);
 #pragma unroll
             for (int j = 0; j < TN; ++j)
-                b[j] = *reinterpret_cast<const bf16x8*>(Ws + ((wn * TN + j) * 32 + lane % 32) * LDS_STRIDE + kofs);
+                b[j] = *reinterpret_cast<const bf16x8*>(&Ws[buf][w_off + j * 32 * STRIDE + ks * 16]);
 #pragma unroll
             for (int i = 0; i < TM; ++i)
 #pragma unroll
                 for (int j = 0; j < TN; ++j)
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[i], b[j], acc[i][j], 0, 0, 0);
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(b[j], a[i], acc[i][j], 0, 0, 0);
         }
     };
 
-    const int nk = (K + BK - 1) / BK;
+    const int nk = (K + BKP - 1) / BKP;
+    // tiles 0 .. DEPTH-2 are requested; tile 0 is staged
 #pragma unroll
     for (int d = 0; d < DEPTH - 1; ++d)
-        if (d < nk) fetch(regs[d], d * BK);
+        if (d < nk) fetch(regs[d], d * BKP);
+    stage(regs[0], 0);
+    lds_barrier();
     for (int kt = 0; kt < nk; kt += DEPTH) {
 #pragma unroll
         for (int d = 0; d < DEPTH; ++d) {
             const int t = kt + d;
             if (t < nk) {
-                lds_barrier();              // readers of the previous tile are done
-                stage(regs[d]);
+                // tile t is in LDS buffer t%2; tile t+1 goes to the other buffer (its last readers
+                // passed the barrier that ended the previous iteration)
+                if (t + DEPTH - 1 < nk) fetch(regs[(d + DEPTH - 1) % DEPTH], (t + DEPTH - 1) * BKP);
+                if (t + 1 < nk) stage(regs[(d + 1) % DEPTH], (t + 1) & 1);
+                compute(t & 1);
                 lds_barrier();
-                if (t + DEPTH - 1 < nk) fetch(regs[(d + DEPTH - 1) % DEPTH], (t + DEPTH - 1) * BK);
-                compute();
             }
         }
     }
 
-    // accumulator layout of the 32x32 tile: register r of lane l holds
-    // row 8*(r/4) + 4*(l/32) + r%4, column l%32
+    // With the weights as the A operand, register r of lane l holds output row l%32 and column
+    // 8*(r/4) + 4*(l/32) + r%4 of the 32x32 tile: 4 consecutive columns per register quad.
+    const bool vec = (ldc % 4 == 0) && ((reinterpret_cast<uintptr_t>(C) & 15) == 0);
 #pragma unroll
     for (int i = 0; i < TM; ++i) {
+        const int m = m0 + (wm * TM + i) * 32 + lane % 32;
+        if (EDGE && m >= M) continue;
 #pragma unroll
         for (int j = 0; j < TN; ++j) {
-            const int n = n0 + (wn * TN + j) * 32 + lane % 32;
-            if (n >= N) continue;
-            const float bv = bias ? bias[n] : 0.f;
 #pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                const int m = m0 + (wm * TM + i) * 32 + 8 * (r / 4) + 4 * (lane / 32) + r % 4;
-                if (m < M) epilogue<bf16_t>(mode, acc[i][j][r], bv, C, static_cast<size_t>(m) * ldc + n);
+            for (int g = 0; g < 4; ++g) {
+                const int n = n0 + (wn * TN + j) * 32 + 8 * g + 4 * (lane / 32);
+                if (EDGE && n >= N) continue;
+                const int n_left = EDGE ? min(4, N - n) : 4;
+                float v[4];
+#pragma unroll
+                for (int e = 0; e < 4; ++e) v[e] = acc[i][j][4 * g + e] + ((bias && e < n_left) ? bias[n + e] : 0.f);
+                store4<MODE>(C, static_cast<size_t>(m) * ldc + n, v, vec, n_left);
             }
         }
     }
 }
 
+template <int WM, int WN, int TM, int TN, int BKP, int DEPTH>
+static void launch_tiled(const bf16_t* a, int lda, const bf16_t* w, int ldw, const float* bias, void* C, int ldc,
+                         int M, int N, int K, int mode, hipStream_t stream) {
+    constexpr int BM = WM * TM * 32, BN = WN * TN * 32;
+    const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
+    // split of the output among the XCDs (xm x xn = 8) that keeps the A rows plus W rows of one XCD smallest
+    int xm = 1, xn = N_XCD;
+    double best = 1e300;
+    for (int cand = 1; cand <= N_XCD; cand *= 2) {
+        const int cm = cand, cn = N_XCD / cand;
+        const double rows = static_cast<double>((tiles_m + cm - 1) / cm) * BM + static_cast<double>((tiles_n + cn - 1) / cn) * BN;
+        if (rows < best) { best = rows; xm = cm; xn = cn; }
+    }
+    const int per_xcd = ((tiles_m + xm - 1) / xm) * ((tiles_n + xn - 1) / xn);
+    const dim3 grid(per_xcd * N_XCD), block(WM * WN * 64);
+    const bool edge = !(M % BM == 0 && N % BN == 0 && K % BKP == 0);
+#define TILED(E, MD) gemm_bf16_mfma<WM, WN, TM, TN, BKP, DEPTH, E, MD><<<grid, block, 0, stream>>>(a, lda, w, ldw, bias, C, ldc, M, N, K, tiles_m, tiles_n, xm, xn)
+#define TILED_MODE(MD) case MD: if (edge) TILED(true, MD); else TILED(false, MD); break;
+    switch (mode) {
+        TILED_MODE(EPI_STORE) TILED_MODE(EPI_GELU_TANH) TILED_MODE(EPI_GELU_ERF) TILED_MODE(EPI_ADD_RESIDUAL)
+        default: if (edge) TILED(true, EPI_STORE_F32); else TILED(false, EPI_STORE_F32); break;
+    }
+#undef TILED_MODE
+#undef TILED
+}
 
 // ---------------------------------------------------------------------------------------------
 // Few rows (decode): M <= 64. The product is bound by streaming W once. Each lane loads 16
@@ -168,7 +265,7 @@ gemm_bf16_skinny(const void* __restrict__ Ain, int lda, const bf16_t* __restrict
 
     // The first weight fragments of this wavefront are requested before the norm, so that their
     // latency overlaps it.
-    constexpr int PRE = 4;
+    constexpr int PRE = 6;
     bf16x8 bpre[PRE];
     if (LN_FUSED) {
 #pragma unroll
@@ -302,7 +399,7 @@ static int launch_skinny(const void* A, int lda, const bf16_t* W, int ldw, const
         nw = LN_FUSED ? 8 : 16;
         while (nw > 1 && nw * 3 > steps) nw >>= 1;
     } else {
-        nw = 4;
+        nw = LN_FUSED ? 8 : 4;      // with the norm fused, its rows spread over more wavefronts
     }
     const dim3 grid(split_k ? tiles : (tiles + nw - 1) / nw), block(nw * 64);
     size_t smem = split_k ? static_cast<size_t>(nw) * mt * 256 * sizeof(float) : 0;
@@ -329,14 +426,9 @@ static int launch_skinny(const void* A, int lda, const bf16_t* W, int ldw, const
     return 0;
 }
 
-static int g_big_tile_min_blocks = 512;
-static int g_variant = 0;
 
 extern "C" {
 
-// Tuning knob: the 128x128 tile is used when it yields at least this many workgroups.
-void mllm_gemm_bf16_set_big_tile_min_blocks(int n) { g_big_tile_min_blocks = n; }
-void mllm_gemm_bf16_set_variant(int v) { g_variant = v; }
 
 // Returns 0, a HIP error code, or -1 when K or the row strides are not multiples of 8
 // elements or a base pointer is not 16-byte aligned.
@@ -347,30 +439,17 @@ int mllm_gemm_bf16(const void* A, int lda, const void* W, int ldw, const float* 
     if ((reinterpret_cast<uintptr_t>(A) & 15) || (reinterpret_cast<uintptr_t>(W) & 15)) return -1;
     const bf16_t* a = static_cast<const bf16_t*>(A);
     const bf16_t* w = static_cast<const bf16_t*>(W);
-    auto blocks = [&](int bm, int bn) { return static_cast<long>((M + bm - 1) / bm) * ((N + bn - 1) / bn); };
-    if (g_variant > 0) {
-        // tuning only: force one tile shape
-#define VAR(ID, WM_, WN_, TM_, TN_, BK_, D_)                                                                  \
-        if (g_variant == ID) {                                                                              \
-            dim3 grid((N + WN_ * TN_ * 32 - 1) / (WN_ * TN_ * 32), (M + WM_ * TM_ * 32 - 1) / (WM_ * TM_ * 32)); \
-            gemm_bf16_mfma<WM_, WN_, TM_, TN_, BK_, D_><<<grid, 256, 0, stream>>>(a, lda, w, ldw, bias, C, ldc, M, N, K, mode); \
-        }
-        VAR(1, 2, 2, 1, 1, 64, 2) VAR(2, 2, 2, 1, 1, 64, 3) VAR(3, 2, 2, 1, 1, 64, 4) VAR(4, 2, 2, 2, 1, 64, 3)
-        VAR(5, 2, 2, 1, 2, 64, 3) VAR(6, 2, 2, 2, 2, 64, 3) VAR(7, 2, 2, 2, 2, 32, 4) VAR(8, 2, 2, 2, 2, 64, 2)
-        VAR(9, 2, 2, 2, 1, 32, 4) VAR(10, 2, 2, 1, 1, 32, 4)
-#undef VAR
-    } else if (M <= 64 && launch_skinny<false>(A, lda, w, ldw, bias, C, ldc, M, N, K, mode, nullptr, nullptr, 0.f,
+    if (M <= 64 && launch_skinny<false>(A, lda, w, ldw, bias, C, ldc, M, N, K, mode, nullptr, nullptr, 0.f,
                                         nullptr, stream) == 0) {
         // few rows: weight-streaming kernel
     } else if (M <= 32) {
-        dim3 grid((N + 127) / 128, (M + 31) / 32);
-        gemm_bf16_mfma<1, 4, 1, 1, 64><<<grid, 256, 0, stream>>>(a, lda, w, ldw, bias, C, ldc, M, N, K, mode);
-    } else if (blocks(128, 128) >= g_big_tile_min_blocks) {
-        dim3 grid((N + 127) / 128, (M + 127) / 128);
-        gemm_bf16_mfma<2, 2, 2, 2, 64><<<grid, 256, 0, stream>>>(a, lda, w, ldw, bias, C, ldc, M, N, K, mode);
+        launch_tiled<1, 4, 1, 1, 64, 3>(a, lda, w, ldw, bias, C, ldc, M, N, K, mode, stream);
+    } else if (static_cast<long>((M + 127) / 128) * ((N + 127) / 128) >= 512) {
+        // enough 128x128 tiles to fill 256 CUs twice: 8 wavefronts (4x2), each 32x64 of the tile
+        launch_tiled<4, 2, 1, 2, 32, 4>(a, lda, w, ldw, bias, C, ldc, M, N, K, mode, stream);
     } else {
-        dim3 grid((N + 63) / 64, (M + 63) / 64);
-        gemm_bf16_mfma<2, 2, 1, 1, 64><<<grid, 256, 0, stream>>>(a, lda, w, ldw, bias, C, ldc, M, N, K, mode);
+        // measured on GPT-2 shapes (2048 rows): 64x64 tiles keep more workgroups in flight and win
+        launch_tiled<2, 2, 1, 1, 64, 3>(a, lda, w, ldw, bias, C, ldc, M, N, K, mode, stream);
     }
     MLLM_LAUNCH_CHECK();
     return 0;
