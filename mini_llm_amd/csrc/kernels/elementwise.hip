@@ -74,6 +74,60 @@ __global__ void layernorm_kernel(const float* __restrict__ x, const int* __restr
     }
 }
 
+// Same norm, one wavefront per row (four rows per workgroup), the row in registers as float4:
+// for D % 4 == 0 and D <= 2048. Fewer, fatter workgroups and 16-byte accesses.
+template <typename OutT>
+__global__ void __launch_bounds__(256)
+layernorm_wave_kernel(const float* __restrict__ x, const int* __restrict__ rows,
+                      const float* __restrict__ gamma, const float* __restrict__ beta,
+                      OutT* __restrict__ y, int n, int D, float eps) {
+    const int wave = threadIdx.x / MLLM_WAVE, lane = threadIdx.x % MLLM_WAVE;
+    const int r = blockIdx.x * 4 + wave;
+    if (r >= n) return;
+    const int src = rows ? rows[r] : r;
+    const float4* xr = reinterpret_cast<const float4*>(x + static_cast<size_t>(src) * D);
+    const float4* g4 = reinterpret_cast<const float4*>(gamma);
+    const float4* b4 = reinterpret_cast<const float4*>(beta);
+    const int nq = D / 4;
+    float4 v[8];
+    float s = 0.f;
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+        const int i = lane + 64 * u;
+        v[u] = i < nq ? xr[i] : make_float4(0.f, 0.f, 0.f, 0.f);
+        s += (v[u].x + v[u].y) + (v[u].z + v[u].w);
+    }
+    const float mean = wave_sum(s) / static_cast<float>(D);
+    float q = 0.f;
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+        if (lane + 64 * u < nq) {
+            const float a = v[u].x - mean, b = v[u].y - mean, c = v[u].z - mean, d = v[u].w - mean;
+            q += (a * a + b * b) + (c * c + d * d);
+        }
+    }
+    const float inv = 1.0f / sqrtf(wave_sum(q) / static_cast<float>(D) + eps);
+    OutT* yr = y + static_cast<size_t>(r) * D;
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+        const int i = lane + 64 * u;
+        if (i < nq) {
+            const float4 gg = g4[i];
+            const float4 bb = beta ? b4[i] : make_float4(0.f, 0.f, 0.f, 0.f);
+            const float o0 = (v[u].x - mean) * inv * gg.x + bb.x, o1 = (v[u].y - mean) * inv * gg.y + bb.y;
+            const float o2 = (v[u].z - mean) * inv * gg.z + bb.z, o3 = (v[u].w - mean) * inv * gg.w + bb.w;
+            if (sizeof(OutT) == 2) {
+                uint2 pk;
+                pk.x = pack_bf16x2(o0, o1);
+                pk.y = pack_bf16x2(o2, o3);
+                *reinterpret_cast<uint2*>(yr + 4 * i) = pk;
+            } else {
+                *reinterpret_cast<float4*>(yr + 4 * i) = make_float4(o0, o1, o2, o3);
+            }
+        }
+    }
+}
+
 // ---------------------------------------------------------------------------
 // Key/value write: copies the key and value columns of each token's row into the
 // row `slots[t]` of the page pools (slot = page * page_size + offset; < 0: skip).
@@ -112,6 +166,17 @@ int mllm_embed(const int* ids, const int* pos, const void* wte, const void* wpe,
 int mllm_layernorm(const float* x, const int* rows, const float* gamma, const float* beta, void* y, int n,
                    int D, float eps, int out_dtype, hipStream_t stream) {
     if (n <= 0) return 0;
+    const bool aligned = ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(gamma) |
+                           reinterpret_cast<uintptr_t>(beta) | reinterpret_cast<uintptr_t>(y)) & 15) == 0;
+    if (D % 4 == 0 && D <= 2048 && aligned) {
+        const int blocks = (n + 3) / 4;
+        if (out_dtype == MLLM_F32)
+            layernorm_wave_kernel<float><<<blocks, 256, 0, stream>>>(x, rows, gamma, beta, (float*)y, n, D, eps);
+        else
+            layernorm_wave_kernel<bf16_t><<<blocks, 256, 0, stream>>>(x, rows, gamma, beta, (bf16_t*)y, n, D, eps);
+        MLLM_LAUNCH_CHECK();
+        return 0;
+    }
     const int threads = D >= 1024 ? 512 : 256;
     if (out_dtype == MLLM_F32)
         layernorm_kernel<float><<<n, threads, 0, stream>>>(x, rows, gamma, beta, (float*)y, D, eps);

@@ -226,7 +226,8 @@ static void launch_tiled(const bf16_t* a, int lda, const bf16_t* w, int ldw, con
 // ---------------------------------------------------------------------------------------------
 // Few rows (decode): M <= 64. The product is bound by streaming W once. Each lane loads 16
 // contiguous bytes of a weight row straight from global memory into the B operand of
-// v_mfma_f32_16x16x32_bf16; a 16-column tile of the output is one MFMA accumulator per 16 rows.
+// v_mfma_f32_16x16x32_bf16; a workgroup owns 16 rows of the output (more rows: more workgroups
+// per column range, placed on the same XCD so that the weights they share come from its L2).
 //   SPLIT_K:  one workgroup per 16-column tile, its wavefronts split K (wavefront w takes the
 //             32-wide k steps w, w+NW, ...) and their partial sums are added in LDS in a fixed
 //             order: for the narrow products, where tiles alone are too few to fill the chip.
@@ -242,12 +243,18 @@ __global__ void __launch_bounds__(LN_FUSED ? 512 : 1024)
 gemm_bf16_skinny(const void* __restrict__ Ain, int lda, const bf16_t* __restrict__ W, int ldw,
                  const float* __restrict__ bias, void* __restrict__ C, int ldc, int M, int N, int K, int mode,
                  const float* __restrict__ gamma, const float* __restrict__ beta, float eps,
-                 const int* __restrict__ rows) {
+                 const int* __restrict__ rows, int col_blocks, int row_blocks) {
     extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
     const int tid = threadIdx.x, wave = tid / 64, lane = tid % 64;
     const int nw = blockDim.x / 64;
     const int row16 = lane % 16, kq = lane / 16;
-    const int n0 = (SPLIT_K ? blockIdx.x : blockIdx.x * nw + wave) * 16;
+    // workgroup id -> (column block, row block): the row blocks of one column block have ids that
+    // agree modulo 8, i.e. run on one XCD
+    const int g = blockIdx.x;
+    const int cb = (g / (N_XCD * row_blocks)) * N_XCD + g % N_XCD, rb = (g / N_XCD) % row_blocks;
+    if (cb >= col_blocks) return;
+    const int m_base = rb * 16;
+    const int n0 = (SPLIT_K ? cb : cb * nw + wave) * 16;
     const int k_first = SPLIT_K ? wave * 32 : 0;      // first k step of this wavefront
     const int k_step = SPLIT_K ? nw * 32 : 32;
     const size_t red_bytes = SPLIT_K ? static_cast<size_t>(nw) * MT * 256 * sizeof(float) : 0;
@@ -281,8 +288,9 @@ gemm_bf16_skinny(const void* __restrict__ Ain, int lda, const bf16_t* __restrict
         const float4* b4 = reinterpret_cast<const float4*>(beta);
         for (int m = wave; m < 16 * MT; m += nw) {
             bf16_t* dst = a_s + static_cast<size_t>(m) * a_stride;
-            if (m < M) {
-                const float4* xr = reinterpret_cast<const float4*>(x + static_cast<size_t>(rows ? rows[m] : m) * lda);
+            if (m_base + m < M) {
+                const float4* xr = reinterpret_cast<const float4*>(
+                    x + static_cast<size_t>(rows ? rows[m_base + m] : m_base + m) * lda);
                 float4 v[8], gg[8], bb[8];
                 float s = 0.f;
 #pragma unroll
@@ -354,7 +362,7 @@ gemm_bf16_skinny(const void* __restrict__ Ain, int lda, const bf16_t* __restrict
             const int m = i * 16 + row16;
             bf16x8 a;
             if (LN_FUSED) a = kin ? *reinterpret_cast<const bf16x8*>(a_s + static_cast<size_t>(m) * a_stride + k) : zero;
-            else a = (kin && m < M) ? *reinterpret_cast<const bf16x8*>(A + static_cast<size_t>(m) * lda + k) : zero;
+            else a = (kin && m_base + m < M) ? *reinterpret_cast<const bf16x8*>(A + static_cast<size_t>(m_base + m) * lda + k) : zero;
             acc[i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, acc[i], 0, 0, 0);
         }
     }
@@ -366,7 +374,7 @@ gemm_bf16_skinny(const void* __restrict__ Ain, int lda, const bf16_t* __restrict
         for (int i = 0; i < MT; ++i)
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
-                const int m = i * 16 + 4 * kq + r;
+                const int m = m_base + i * 16 + 4 * kq + r;
                 if (m < M) epilogue<bf16_t>(mode, acc[i][r], bv, C, static_cast<size_t>(m) * ldc + n);
             }
         return;
@@ -378,7 +386,7 @@ gemm_bf16_skinny(const void* __restrict__ Ain, int lda, const bf16_t* __restrict
     __syncthreads();
     for (int idx = tid; idx < MT * 256; idx += blockDim.x) {
         const int i = idx / 256, r = (idx % 256) / 64, l = idx % 64;
-        const int m = i * 16 + 4 * (l / 16) + r, nn = n0 + l % 16;
+        const int m = m_base + i * 16 + 4 * (l / 16) + r, nn = n0 + l % 16;
         if (m >= M || nn >= N) continue;
         const float bv = bias ? bias[nn] : 0.f;
         float v = 0.f;
@@ -391,9 +399,13 @@ template <bool LN_FUSED>
 static int launch_skinny(const void* A, int lda, const bf16_t* W, int ldw, const float* bias, void* C, int ldc,
                          int M, int N, int K, int mode, const float* gamma, const float* beta, float eps,
                          const int* rows, hipStream_t stream) {
-    const int mt = (M + 15) / 16;
     const int tiles = (N + 15) / 16, steps = (K + 31) / 32;
     const bool split_k = tiles < 1024;
+    // Narrow products: 16 rows per workgroup and one workgroup per 16 rows (more workgroups, each
+    // reading only its rows). Wide products: every wavefront keeps all rows of its tile in
+    // registers (up to 4 accumulators), so the weights are streamed once.
+    const int row_blocks = split_k ? (M + 15) / 16 : 1;
+    const int mt = split_k ? 1 : (M + 15) / 16;
     int nw;
     if (split_k) {
         nw = LN_FUSED ? 8 : 16;
@@ -401,7 +413,8 @@ static int launch_skinny(const void* A, int lda, const bf16_t* W, int ldw, const
     } else {
         nw = LN_FUSED ? 8 : 4;      // with the norm fused, its rows spread over more wavefronts
     }
-    const dim3 grid(split_k ? tiles : (tiles + nw - 1) / nw), block(nw * 64);
+    const int col_blocks = split_k ? tiles : (tiles + nw - 1) / nw;
+    const dim3 grid((col_blocks + N_XCD - 1) / N_XCD * N_XCD * row_blocks), block(nw * 64);
     size_t smem = split_k ? static_cast<size_t>(nw) * mt * 256 * sizeof(float) : 0;
     if (LN_FUSED) {
         smem += static_cast<size_t>(16) * mt * (K + 8) * sizeof(bf16_t);
@@ -410,19 +423,21 @@ static int launch_skinny(const void* A, int lda, const bf16_t* W, int ldw, const
             return -2;
     }
     if (smem > 64 * 1024) return -2;
-#define SKINNY_LAUNCH(MTV, SK)                                                                              \
-    gemm_bf16_skinny<MTV, LN_FUSED, SK><<<grid, block, smem, stream>>>(A, lda, W, ldw, bias, C, ldc, M, N, K, \
-                                                                       mode, gamma, beta, eps, rows)
-#define SKINNY_CASE(MTV)                                                   \
-    case MTV:                                                              \
-        if (split_k) SKINNY_LAUNCH(MTV, true); else SKINNY_LAUNCH(MTV, false); \
+#define SKINNY_WIDE(MTV)                                                                              \
+    case MTV:                                                                                         \
+        gemm_bf16_skinny<MTV, LN_FUSED, false><<<grid, block, smem, stream>>>(                        \
+            A, lda, W, ldw, bias, C, ldc, M, N, K, mode, gamma, beta, eps, rows, col_blocks, row_blocks); \
         break;
-    switch (mt) {
-        SKINNY_CASE(1) SKINNY_CASE(2) SKINNY_CASE(3) SKINNY_CASE(4)
-        default: return -2;
+    if (split_k) {
+        gemm_bf16_skinny<1, LN_FUSED, true><<<grid, block, smem, stream>>>(
+            A, lda, W, ldw, bias, C, ldc, M, N, K, mode, gamma, beta, eps, rows, col_blocks, row_blocks);
+    } else {
+        switch (mt) {
+            SKINNY_WIDE(1) SKINNY_WIDE(2) SKINNY_WIDE(3) SKINNY_WIDE(4)
+            default: return -2;
+        }
     }
-#undef SKINNY_CASE
-#undef SKINNY_LAUNCH
+#undef SKINNY_WIDE
     return 0;
 }
 
@@ -457,7 +472,7 @@ int mllm_gemm_bf16(const void* A, int lda, const void* W, int ldw, const float* 
 
 // LayerNorm of the fp32 rows x[M,K] (row m taken from x[rows[m]] when `rows` is given) fused into the
 // product with W[N,K]: C = epilogue(LN(x) W^T + bias).
-// Returns 0, a HIP error code, -1 for misaligned operands, or -2 when M or K is too large for the
+// M <= 16. Returns 0, a HIP error code, -1 for misaligned operands, or -2 when M or K is too large for the
 // fused kernel (the caller then runs the norm and the product separately).
 int mllm_ln_gemm_bf16(const float* x, int ldx, const int* rows, const float* gamma, const float* beta, float eps,
                       const void* W, int ldw, const float* bias, void* C, int ldc, int M, int N, int K, int mode,

@@ -75,81 +75,145 @@ __global__ void argmax_stage2(const float* __restrict__ part_val, const int* __r
 }
 
 // ---------------------------------------------------------------------------
-// Temperature sampling: p = softmax(logits / temperature) in fp32, then the
-// inverse CDF at u in [0,1): the first index whose cumulative mass exceeds u * total.
-// Rows with temperature <= 0 take the argmax. One block per row; every thread owns a
-// contiguous chunk of the vocabulary so that the cumulative order is the index order.
+// Temperature sampling: p = softmax(logits / temperature) in fp32, then the inverse CDF at
+// u in [0,1): the first index whose cumulative mass exceeds u * total. Rows with
+// temperature <= 0 take the argmax (lowest index on ties). One workgroup per row:
+//   1. row maximum (and its lowest index), coalesced strided loads;
+//   2. the mass of every tile of SAMPLE_TILE consecutive entries, one wavefront per tile;
+//   3. a scan over the few tile masses finds the tile that holds u * total;
+//   4. inside that tile every thread owns 8 consecutive entries; a workgroup scan finds the thread
+//      and it walks its 8 entries.
+// The cumulative order is the index order and every sum has a fixed order, so a draw depends on
+// (logits, temperature, u) only.
 // ---------------------------------------------------------------------------
-__global__ void sample_kernel(const float* __restrict__ logits, int ld, int V,
-                              const float* __restrict__ temperature, const float* __restrict__ u,
-                              int* __restrict__ out) {
-    __shared__ float scratch[16];
-    __shared__ float part[SAMPLE_THREADS];
-    __shared__ int chosen_thread;
-    __shared__ float chosen_before;
-    const int r = blockIdx.x;
+#define SAMPLE_TILE 2048
+#define SAMPLE_MAX_TILES 1024      // vocabularies up to 2M entries
+#define SAMPLE_BLOCK 1024          // threads of the sampling workgroup
+
+__global__ void __launch_bounds__(SAMPLE_BLOCK)
+sample_kernel(const float* __restrict__ logits, int ld, int V, const float* __restrict__ temperature,
+              const float* __restrict__ u, int* __restrict__ out) {
+    __shared__ float sv[SAMPLE_BLOCK / MLLM_WAVE];
+    __shared__ int si[SAMPLE_BLOCK / MLLM_WAVE];
+    __shared__ float tile_mass[SAMPLE_MAX_TILES];
+    __shared__ float wave_mass[SAMPLE_TILE / 8 / MLLM_WAVE];
+    __shared__ int sh_tile;
+    __shared__ float sh_rest;
+    const int r = blockIdx.x, tid = threadIdx.x, wave = tid / MLLM_WAVE, lane = tid % MLLM_WAVE;
     const float* row = logits + static_cast<size_t>(r) * ld;
     const float temp = temperature[r];
-    const int chunk = (V + blockDim.x - 1) / blockDim.x;
-    const int lo = min(V, static_cast<int>(threadIdx.x) * chunk), hi = min(V, lo + chunk);
 
-    float m = -INFINITY;
-    int mi = 0x7fffffff;
-    for (int i = lo; i < hi; ++i) {
-        float v = row[i];
-        if (better(v, i, m, mi)) { m = v; mi = i; }
-    }
-    if (temp <= 0.f) {
-        // greedy: reduce (value, index) pairs
-        __shared__ float gv[SAMPLE_THREADS];
-        __shared__ int gi[SAMPLE_THREADS];
-        gv[threadIdx.x] = m;
-        gi[threadIdx.x] = mi;
-        __syncthreads();
-        if (threadIdx.x == 0) {
-            float bv = gv[0];
-            int bi = gi[0];
-            for (int t = 1; t < blockDim.x; ++t)
-                if (better(gv[t], gi[t], bv, bi)) { bv = gv[t]; bi = gi[t]; }
-            out[r] = (bi == 0x7fffffff) ? 0 : bi;
+    // 1. maximum and its lowest index
+    float bv = -INFINITY;
+    int bi = 0x7fffffff;
+    for (int i0 = 0; i0 < V; i0 += SAMPLE_BLOCK * 8) {
+        float v[8];
+#pragma unroll
+        for (int k = 0; k < 8; ++k) {
+            const int i = i0 + k * SAMPLE_BLOCK + tid;
+            v[k] = row[min(i, V - 1)];           // unconditional (clamped) loads stay in flight together
         }
+#pragma unroll
+        for (int k = 0; k < 8; ++k) {
+            const int i = i0 + k * SAMPLE_BLOCK + tid;
+            if (i < V && better(v[k], i, bv, bi)) { bv = v[k]; bi = i; }
+        }
+    }
+#pragma unroll
+    for (int off = MLLM_WAVE / 2; off > 0; off >>= 1) {
+        const float ov = __shfl_xor(bv, off, MLLM_WAVE);
+        const int oi = __shfl_xor(bi, off, MLLM_WAVE);
+        if (better(ov, oi, bv, bi)) { bv = ov; bi = oi; }
+    }
+    if (lane == 0) { sv[wave] = bv; si[wave] = bi; }
+    __syncthreads();
+    bv = sv[0]; bi = si[0];
+    for (int w = 1; w < SAMPLE_BLOCK / MLLM_WAVE; ++w)
+        if (better(sv[w], si[w], bv, bi)) { bv = sv[w]; bi = si[w]; }
+    if (temp <= 0.f) {                       // greedy row (uniform over the workgroup)
+        if (tid == 0) out[r] = (bi == 0x7fffffff) ? 0 : bi;
         return;
     }
-    const float row_max = block_max(m, scratch);
-    const float inv_t = 1.0f / temp;
-    float s = 0.f;
-    for (int i = lo; i < hi; ++i) s += expf((row[i] - row_max) * inv_t);
-    part[threadIdx.x] = s;
-    __syncthreads();
-    if (threadIdx.x == 0) {
-        float total = 0.f;
-        for (int t = 0; t < blockDim.x; ++t) total += part[t];
-        const float target = u[r] * total;
-        float before = 0.f;
-        int pick = -1;
-        float pick_before = 0.f;
-        int last_nonempty = 0;
-        float last_before = 0.f;
-        for (int t = 0; t < blockDim.x; ++t) {
-            if (part[t] > 0.f) { last_nonempty = t; last_before = before; }
-            if (pick < 0 && target < before + part[t]) { pick = t; pick_before = before; }
-            before += part[t];
+    // e^((x - max)/T) as 2^((x - max) * log2(e)/T)
+    const float row_max = bv, inv_t = 1.44269504088896340736f / temp;
+
+    // 2. mass of every tile; wavefront w takes tiles w, w+16, ...
+    const int n_tiles = (V + SAMPLE_TILE - 1) / SAMPLE_TILE;
+    for (int t = wave; t < n_tiles; t += SAMPLE_BLOCK / MLLM_WAVE) {
+        float s = 0.f;
+        const int base = t * SAMPLE_TILE;
+        for (int k0 = 0; k0 < SAMPLE_TILE / MLLM_WAVE; k0 += 8) {
+            float v[8];
+#pragma unroll
+            for (int k = 0; k < 8; ++k) v[k] = row[min(base + (k0 + k) * MLLM_WAVE + lane, V - 1)];
+#pragma unroll
+            for (int k = 0; k < 8; ++k)
+                if (base + (k0 + k) * MLLM_WAVE + lane < V) s += exp2f((v[k] - row_max) * inv_t);
         }
-        if (pick < 0) { pick = last_nonempty; pick_before = last_before; }   // rounding at the top end
-        chosen_thread = pick;
-        chosen_before = pick_before;
-        part[0] = target;   // thread 0's own sum is no longer needed
+        s = wave_sum(s);
+        if (lane == 0) tile_mass[t] = s;
     }
     __syncthreads();
-    if (static_cast<int>(threadIdx.x) == chosen_thread) {
-        const float target = part[0];
-        float c = chosen_before;
-        int pick = -1, last = lo;
-        for (int i = lo; i < hi; ++i) {
-            float p = expf((row[i] - row_max) * inv_t);
-            if (p > 0.f) last = i;
-            c += p;
-            if (target < c) { pick = i; break; }
+
+    // 3. the tile that holds the target
+    if (tid == 0) {
+        float total = 0.f;
+        for (int t = 0; t < n_tiles; ++t) total += tile_mass[t];
+        const float target = u[r] * total;
+        float before = 0.f;
+        int pick = -1, last = 0;
+        float rest = 0.f;
+        for (int t = 0; t < n_tiles; ++t) {
+            if (tile_mass[t] > 0.f) last = t;
+            if (pick < 0 && target < before + tile_mass[t]) { pick = t; rest = target - before; }
+            before += tile_mass[t];
+        }
+        if (pick < 0) { pick = last; rest = INFINITY; }      // rounding at the top end: last entry with mass
+        sh_tile = pick;
+        sh_rest = rest;
+    }
+    __syncthreads();
+
+    // 4. inside the tile: 8 consecutive entries per thread; the first SAMPLE_TILE/8 threads suffice
+    const bool worker = tid < SAMPLE_TILE / 8;
+    const int base = sh_tile * SAMPLE_TILE + (worker ? tid : 0) * 8;
+    const float rest = sh_rest;
+    float p[8], local = 0.f;
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+        p[k] = (worker && base + k < V) ? exp2f((row[min(base + k, V - 1)] - row_max) * inv_t) : 0.f;
+        local += p[k];
+    }
+    // exclusive prefix of `local` over the workgroup, in thread order
+    float incl = local;
+#pragma unroll
+    for (int off = 1; off < MLLM_WAVE; off <<= 1) {
+        const float o = __shfl_up(incl, off, MLLM_WAVE);
+        if (lane >= off) incl += o;
+    }
+    if (worker && lane == MLLM_WAVE - 1) wave_mass[wave] = incl;
+    __syncthreads();
+    float before = incl - local;
+    for (int w = 0; w < wave && w < SAMPLE_TILE / 8 / MLLM_WAVE; ++w) before += wave_mass[w];
+    // the first thread (in order) whose range reaches the target; if none does, the last with mass
+    const bool hit = worker && rest < before + local && local > 0.f;
+    const bool has_mass = worker && local > 0.f;
+    // lowest hitting thread / highest thread with mass, through LDS atomics
+    __shared__ int first_hit, last_mass;
+    if (tid == 0) { first_hit = 0x7fffffff; last_mass = -1; }
+    __syncthreads();
+    if (hit) atomicMin(&first_hit, tid);
+    if (has_mass) atomicMax(&last_mass, tid);
+    __syncthreads();
+    const int chosen = first_hit != 0x7fffffff ? first_hit : last_mass;
+    if (tid == chosen) {
+        float c = before;
+        int pick = -1, last = base;
+#pragma unroll
+        for (int k = 0; k < 8; ++k) {
+            if (p[k] > 0.f) last = base + k;
+            c += p[k];
+            if (pick < 0 && rest < c && p[k] > 0.f) pick = base + k;
         }
         out[r] = pick >= 0 ? pick : last;
     }
@@ -177,7 +241,8 @@ int mllm_argmax(const float* logits, int ld, int n, int V, int* out, float* part
 int mllm_sample(const float* logits, int ld, int n, int V, const float* temperature, const float* u, int* out,
                 hipStream_t stream) {
     if (n <= 0) return 0;
-    sample_kernel<<<n, SAMPLE_THREADS, 0, stream>>>(logits, ld, V, temperature, u, out);
+    if (V <= 0 || V > SAMPLE_TILE * SAMPLE_MAX_TILES) return -1;
+    sample_kernel<<<n, SAMPLE_BLOCK, 0, stream>>>(logits, ld, V, temperature, u, out);
     MLLM_LAUNCH_CHECK();
     return 0;
 }

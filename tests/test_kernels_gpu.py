@@ -58,7 +58,8 @@ def test_embed_reference_vector(ops, dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("rows,D,eps", [(17, 768, 1e-5), (5, 100, 1e-6), (3, 1600, 1e-5), (1, 16, 1e-3)])
+@pytest.mark.parametrize("rows,D,eps", [(17, 768, 1e-5), (5, 100, 1e-6), (3, 1600, 1e-5), (1, 16, 1e-3),
+                                        (2050, 768, 1e-5), (6, 2048, 1e-5), (5, 2052, 1e-5), (4, 98, 1e-6)])
 def test_layernorm(ops, dtype, rows, D, eps):
     g = torch.Generator().manual_seed(0)
     x = _rand((rows, D), torch.float32, g) + 0.5
@@ -134,7 +135,8 @@ def test_linear_bf16_few_rows(ops, M, N, K):
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("M,N,K", [(1, 2304, 768), (8, 3072, 768), (16, 320, 96), (5, 200, 1600), (17, 96, 64),
-                                   (3, 64, 4096), (16, 6400, 1600), (9, 50257, 1024), (16, 3072, 1024)])
+                                   (3, 64, 4096), (16, 6400, 1600), (9, 50257, 1024), (16, 3072, 1024), (33, 2304, 768),
+                                   (64, 50257, 768), (64, 104, 1600), (65, 96, 64)])
 @pytest.mark.parametrize("epi", ["store", "gelu_tanh", "gelu_erf", "store_f32"])
 def test_ln_linear(ops, dtype, M, N, K, epi):
     """LayerNorm fused into the product (bf16, few rows) and its unfused form give the plain result."""
@@ -388,6 +390,25 @@ def test_sample_inverse_cdf(ops, V):
         lo = float(c[got[i] - 1]) if got[i] > 0 else 0.0
         hi = float(c[got[i]])
         assert lo - 1e-5 <= float(u[i]) <= hi + 1e-5, (i, got[i], lo, float(u[i]), hi)
+
+
+def test_sample_edge_rows(ops):
+    """All mass on one entry, a flat row, u at both ends, masses that underflow to zero."""
+    V = 5000
+    logits = torch.full((6, V), -50.0)
+    logits[0, 4321] = 30.0
+    logits[1] = 0.0
+    logits[2] = 0.0
+    logits[3, V - 1] = 30.0
+    logits[4, 0] = 30.0
+    logits[5, 2047:2050] = 5.0                      # the mass straddles a tile edge
+    u = torch.tensor([0.5, 0.0, 0.99999994, 0.99999994, 0.0, 0.5])
+    temps = torch.full((6,), 1.0)
+    out = torch.empty(6, dtype=torch.int32, device=DEV)
+    ops.sample(logits.to(DEV), temps.to(DEV), u.to(DEV), out)
+    got = out.cpu().tolist()
+    assert got[0] == 4321 and got[1] == 0 and got[2] == V - 1 and got[3] == V - 1 and got[4] == 0
+    assert got[5] == 2048
 
 
 def test_sample_frequencies_follow_softmax(ops):
