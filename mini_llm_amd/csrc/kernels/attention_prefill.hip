@@ -1,7 +1,7 @@
 // Prefill attention on the MFMA units of gfx950, bf16 with fp32 softmax: causal (optionally
 // windowed) attention of a step's query rows over the paged cache. A workgroup takes 64
 // consecutive queries of one sequence and one head; its four wavefronts take 16 queries each
-// and walk the keys in tiles of 64, which are gathered through the block table into LDS (keys
+// and walk the keys in tiles of 128, which are gathered through the block table into LDS (keys
 // row-major, values transposed), so prompt portions that start anywhere read what earlier steps
 // left in the pages.
 //
@@ -22,9 +22,9 @@ typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 
 #define PF_BM 64
-#define PF_BN 64
+#define PF_BN 128
 #define PF_TABLE_LDS 2048   // block-table entries staged in LDS (longer tables are read from memory)
-#define PF_VT_STRIDE 66     // elements per transposed value row: 33 words, so staging writes spread over banks
+#define PF_VT_STRIDE (PF_BN + 2)   // elements per transposed value row: an odd number of words, so staging writes spread over banks
 
 union Frag8 {
     bf16x8 v;
@@ -48,8 +48,10 @@ prefill_attention_kernel(const bf16_t* __restrict__ q, int q_stride, int q_col,
     __shared__ __attribute__((aligned(16))) bf16_t Vt[DH * PF_VT_STRIDE];
     __shared__ int sm_table[PF_TABLE_LDS];
 
-    // which sequence and which of its 64-query tiles this workgroup has
-    int tile = blockIdx.x, b = 0, q_begin = 0, q_len = 0;
+    // Which sequence and which of its 64-query tiles this workgroup has. Heads vary fastest and the
+    // tiles are handed out last-first: a causal tile's work grows with its position, so the long
+    // ones start in the first wave of workgroups and the short ones fill the tail.
+    int tile = gridDim.y - 1 - blockIdx.y, b = 0, q_begin = 0, q_len = 0;
     for (; b < n_seqs; ++b) {
         q_begin = cu_q[b];
         q_len = cu_q[b + 1] - q_begin;
@@ -59,7 +61,7 @@ prefill_attention_kernel(const bf16_t* __restrict__ q, int q_stride, int q_col,
     }
     if (b >= n_seqs) return;               // surplus workgroup; the whole workgroup leaves
 
-    const int h = blockIdx.y, hk = h / (n_heads / n_kv_heads);
+    const int h = blockIdx.x, hk = h / (n_heads / n_kv_heads);
     const int tid = threadIdx.x, wave = tid / 64, lane = tid % 64;
     const int G = lane / 16, c16 = lane % 16;
     const int start = ctx_len[b] - q_len;                 // position of the step's first query
@@ -173,10 +175,10 @@ prefill_attention_kernel(const bf16_t* __restrict__ q, int q_stride, int q_col,
         constexpr bool MASKED = decltype(masked_tag)::value;
         const int j_base = kt * PF_BN;
         // S^T: s[nt][r] is the score of key j_base + 16*nt + 4*G + r with this lane's query
-        float s[4][4];
+        float s[PF_BN / 16][4];
         float tile_max = -INFINITY;
 #pragma unroll
-        for (int nt = 0; nt < 4; ++nt) {
+        for (int nt = 0; nt < PF_BN / 16; ++nt) {
             f32x4 acc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
             for (int ks = 0; ks < KS; ++ks) {
@@ -203,7 +205,7 @@ prefill_attention_kernel(const bf16_t* __restrict__ q, int q_stride, int q_col,
         m = m_new;
         float psum = 0.f;
 #pragma unroll
-        for (int nt = 0; nt < 4; ++nt)
+        for (int nt = 0; nt < PF_BN / 16; ++nt)
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
                 s[nt][r] = fast_exp2(s[nt][r] - m_use);
@@ -215,10 +217,10 @@ prefill_attention_kernel(const bf16_t* __restrict__ q, int q_stride, int q_col,
 #pragma unroll
             for (int r = 0; r < 4; ++r) o[dt][r] *= alpha;
 
-        // O^T += V^T P^T over two slabs of 32 keys. k slot i of lane group G stands for key
+        // O^T += V^T P^T over slabs of 32 keys. k slot i of lane group G stands for key
         // 32*slab + 4*G + i (i < 4) or 32*slab + 16 + 4*G + i - 4 (i >= 4) in both operands.
 #pragma unroll
-        for (int slab = 0; slab < 2; ++slab) {
+        for (int slab = 0; slab < PF_BN / 32; ++slab) {
             Frag8 pf;
             pf.w[0] = pack_bf16x2(s[2 * slab][0], s[2 * slab][1]);
             pf.w[1] = pack_bf16x2(s[2 * slab][2], s[2 * slab][3]);
@@ -287,9 +289,9 @@ int mllm_prefill_attention_bf16(const void* q, int q_stride, int q_col, const vo
                                 int head_dim, int page_size, float scale, int window, void* out, int out_stride,
                                 hipStream_t stream) {
     if (n_seqs <= 0 || n_tiles_upper <= 0) return 0;
-    if (n_heads % n_kv_heads != 0 || n_heads > 65535) return -1;
+    if (n_heads % n_kv_heads != 0 || n_tiles_upper > 65535) return -1;
     if ((page_size & (page_size - 1)) != 0 || max_blocks > PF_TABLE_LDS) return -1;
-    const dim3 grid(n_tiles_upper, n_heads);
+    const dim3 grid(n_heads, n_tiles_upper);
     const float sl2 = scale * 1.44269504088896340736f;
 #define PF_CASE(D)                                                                                          \
     case D:                                                                                                 \
