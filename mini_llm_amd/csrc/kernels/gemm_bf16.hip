@@ -270,6 +270,22 @@ gemm_bf16_skinny(const void* __restrict__ Ain, int lda, const bf16_t* __restrict
 #pragma unroll
     for (int i = 0; i < MT; ++i) acc[i] = f32x4{0.f, 0.f, 0.f, 0.f};
 
+    // Split-K epilogue operands (thread tid < 256 owns output element tid of the 16x16 tile, in
+    // accumulator order): requested now so that their latency hides behind the product.
+    bool ep_ok = false;
+    size_t ep_idx = 0;
+    float ep_bias = 0.f, ep_old = 0.f;
+    if (SPLIT_K && MT == 1 && tid < 256) {
+        const int r = tid / 64, l = tid % 64;
+        const int m = m_base + 4 * (l / 16) + r, nn = n0 + l % 16;
+        ep_ok = m < M && nn < N;
+        if (ep_ok) {
+            ep_idx = static_cast<size_t>(m) * ldc + nn;
+            if (bias) ep_bias = bias[nn];
+            if (mode == EPI_ADD_RESIDUAL) ep_old = static_cast<const float*>(C)[ep_idx];
+        }
+    }
+
     // The first weight fragments of this wavefront are requested before the norm, so that their
     // latency overlaps it.
     constexpr int PRE = 6;
@@ -384,6 +400,18 @@ gemm_bf16_skinny(const void* __restrict__ Ain, int lda, const bf16_t* __restrict
 #pragma unroll
         for (int r = 0; r < 4; ++r) red[(static_cast<size_t>(wave) * MT + i) * 256 + r * 64 + lane] = acc[i][r];
     __syncthreads();
+    if (MT == 1) {
+        // one output per thread (the first 256); its bias and old residual value were requested
+        // before the MFMA loop
+        if (ep_ok) {
+            float v = 0.f;
+            for (int w = 0; w < nw; ++w) v += red[static_cast<size_t>(w) * 256 + tid];
+            v += ep_bias;
+            if (mode == EPI_ADD_RESIDUAL) static_cast<float*>(C)[ep_idx] = ep_old + v;
+            else epilogue<bf16_t>(mode, v, 0.f, C, ep_idx);
+        }
+        return;
+    }
     for (int idx = tid; idx < MT * 256; idx += blockDim.x) {
         const int i = idx / 256, r = (idx % 256) / 64, l = idx % 64;
         const int m = m_base + i * 16 + 4 * (l / 16) + r, nn = n0 + l % 16;
@@ -409,7 +437,7 @@ static int launch_skinny(const void* A, int lda, const bf16_t* W, int ldw, const
     int nw;
     if (split_k) {
         nw = LN_FUSED ? 8 : 16;
-        while (nw > 1 && nw * 3 > steps) nw >>= 1;
+        while (nw > 4 && nw * 3 > steps) nw >>= 1;      // at least 256 threads: one per output of the tile
     } else {
         nw = LN_FUSED ? 8 : 4;      // with the norm fused, its rows spread over more wavefronts
     }

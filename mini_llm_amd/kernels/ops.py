@@ -321,7 +321,7 @@ def _decode_launch_shape(pairs: int, max_ctx_len: int):
         return DECODE_SHAPE_OVERRIDE
     # One workgroup per pair: merging splits needs a device-wide fence, which costs more than the
     # parallelism gains at these context lengths. Few pairs get more wavefronts each instead.
-    return 1, (4 if pairs >= 512 else 8 if pairs >= 192 else 16)
+    return 1, (4 if pairs >= 512 else 8)
 
 
 
