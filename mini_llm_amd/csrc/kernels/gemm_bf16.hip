@@ -110,27 +110,40 @@ gemm_bf16_mfma(const bf16_t* __restrict__ A, int lda, const bf16_t* __restrict__
         uint4 ra[A_CH], rw[W_CH];
     };
     TileRegs regs[DEPTH];
+    // Every thread issues every load of every fetch, with the address clamped into the matrix:
+    // the number of loads in flight is then the same on every path through the loop, and only so
+    // does the compiler wait for exactly the tile that is staged next while later ones stay in
+    // flight (a skipped load on any path makes it wait for all of them). What lies outside the
+    // matrices is zeroed when the tile is staged.
     auto fetch = [&](TileRegs& t, int k0) {
 #pragma unroll
         for (int i = 0; i < A_CH; ++i) {
             const int kc8 = (tid + i * NT) % CPR * 8;
-            const bool ok = va[i] && (!EDGE || k0 + kc8 < K);
-            t.ra[i] = ok ? *reinterpret_cast<const uint4*>(pa[i] + k0) : make_uint4(0, 0, 0, 0);
+            const int k = EDGE ? min(k0 + kc8, K - 8) - kc8 : k0;
+            t.ra[i] = *reinterpret_cast<const uint4*>(pa[i] + k);
         }
 #pragma unroll
         for (int i = 0; i < W_CH; ++i) {
             const int kc8 = (tid + i * NT) % CPR * 8;
-            const bool ok = vw[i] && (!EDGE || k0 + kc8 < K);
-            t.rw[i] = ok ? *reinterpret_cast<const uint4*>(pw[i] + k0) : make_uint4(0, 0, 0, 0);
+            const int k = EDGE ? min(k0 + kc8, K - 8) - kc8 : k0;
+            t.rw[i] = *reinterpret_cast<const uint4*>(pw[i] + k);
         }
     };
-    auto stage = [&](const TileRegs& t, int buf) {
+    auto stage = [&](const TileRegs& t, int buf, int k0) {
 #pragma unroll
-        for (int i = 0; i < A_CH; ++i)
-            if (BM * CPR % NT == 0 || tid + i * NT < BM * CPR) *reinterpret_cast<uint4*>(&As[buf][la[i]]) = t.ra[i];
+        for (int i = 0; i < A_CH; ++i) {
+            const int kc8 = (tid + i * NT) % CPR * 8;
+            const bool ok = !EDGE || (va[i] && k0 + kc8 < K);
+            if (BM * CPR % NT == 0 || tid + i * NT < BM * CPR)
+                *reinterpret_cast<uint4*>(&As[buf][la[i]]) = ok ? t.ra[i] : make_uint4(0, 0, 0, 0);
+        }
 #pragma unroll
-        for (int i = 0; i < W_CH; ++i)
-            if (BN * CPR % NT == 0 || tid + i * NT < BN * CPR) *reinterpret_cast<uint4*>(&Ws[buf][lw[i]]) = t.rw[i];
+        for (int i = 0; i < W_CH; ++i) {
+            const int kc8 = (tid + i * NT) % CPR * 8;
+            const bool ok = !EDGE || (vw[i] && k0 + kc8 < K);
+            if (BN * CPR % NT == 0 || tid + i * NT < BN * CPR)
+                *reinterpret_cast<uint4*>(&Ws[buf][lw[i]]) = ok ? t.rw[i] : make_uint4(0, 0, 0, 0);
+        }
     };
     const int a_off = (wm * TM * 32 + lane % 32) * STRIDE + 8 * (lane / 32);
     const int w_off = (wn * TN * 32 + lane % 32) * STRIDE + 8 * (lane / 32);
@@ -153,24 +166,35 @@ gemm_bf16_mfma(const bf16_t* __restrict__ A, int lda, const bf16_t* __restrict__
     };
 
     const int nk = (K + BKP - 1) / BKP;
-    // tiles 0 .. DEPTH-2 are requested; tile 0 is staged
+    // tiles 0 .. DEPTH-2 are requested (past the last tile: the last one again, never used);
+    // tile 0 is staged
 #pragma unroll
-    for (int d = 0; d < DEPTH - 1; ++d)
-        if (d < nk) fetch(regs[d], d * BKP);
-    stage(regs[0], 0);
+    for (int d = 0; d < DEPTH - 1; ++d) fetch(regs[d], min(d, nk - 1) * BKP);
+    stage(regs[0], 0, 0);
     lds_barrier();
-    for (int kt = 0; kt < nk; kt += DEPTH) {
+    // Whole groups of DEPTH tiles run without a branch in the body (a load or a use of it under a
+    // condition would be moved or waited for conservatively); the last nk % DEPTH tiles, which
+    // fetch nothing any more, follow under conditions.
+    const int n_groups = nk / DEPTH, n_tail = nk % DEPTH;
+    for (int g = 0; g < n_groups; ++g) {
 #pragma unroll
         for (int d = 0; d < DEPTH; ++d) {
-            const int t = kt + d;
-            if (t < nk) {
-                // tile t is in LDS buffer t%2; tile t+1 goes to the other buffer (its last readers
-                // passed the barrier that ended the previous iteration)
-                if (t + DEPTH - 1 < nk) fetch(regs[(d + DEPTH - 1) % DEPTH], (t + DEPTH - 1) * BKP);
-                if (t + 1 < nk) stage(regs[(d + 1) % DEPTH], (t + 1) & 1);
-                compute(t & 1);
-                lds_barrier();
-            }
+            const int t = g * DEPTH + d;
+            // tile t is in LDS buffer t%2; tile t+1 goes to the other buffer (its last readers
+            // passed the barrier that ended the previous iteration)
+            fetch(regs[(d + DEPTH - 1) % DEPTH], min(t + DEPTH - 1, nk - 1) * BKP);
+            stage(regs[(d + 1) % DEPTH], (t + 1) & 1, (t + 1) * BKP);
+            compute(t & 1);
+            lds_barrier();
+        }
+    }
+#pragma unroll
+    for (int d = 0; d < DEPTH - 1; ++d) {
+        const int t = n_groups * DEPTH + d;
+        if (d < n_tail) {
+            if (d + 1 < n_tail) stage(regs[(d + 1) % DEPTH], (t + 1) & 1, (t + 1) * BKP);
+            compute(t & 1);
+            lds_barrier();
         }
     }
 
@@ -238,13 +262,17 @@ static void launch_tiled(const bf16_t* a, int lda, const bf16_t* w, int ldw, con
 // ---------------------------------------------------------------------------------------------
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 
-template <int MT, bool LN_FUSED, bool SPLIT_K>
-__global__ void __launch_bounds__(LN_FUSED ? 512 : 1024)
+enum { A_GLOBAL = 0, A_NORMED = 1, A_STAGED = 2 };
+
+template <int MT, int ASRC, bool SPLIT_K>
+__global__ void __launch_bounds__(ASRC == A_NORMED ? 512 : 1024)
 gemm_bf16_skinny(const void* __restrict__ Ain, int lda, const bf16_t* __restrict__ W, int ldw,
                  const float* __restrict__ bias, void* __restrict__ C, int ldc, int M, int N, int K, int mode,
                  const float* __restrict__ gamma, const float* __restrict__ beta, float eps,
                  const int* __restrict__ rows, int col_blocks, int row_blocks) {
     extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
+    constexpr bool LN_FUSED = ASRC == A_NORMED;
+    constexpr bool IN_LDS = ASRC != A_GLOBAL;
     const int tid = threadIdx.x, wave = tid / 64, lane = tid % 64;
     const int nw = blockDim.x / 64;
     const int row16 = lane % 16, kq = lane / 16;
@@ -253,7 +281,7 @@ gemm_bf16_skinny(const void* __restrict__ Ain, int lda, const bf16_t* __restrict
     const int g = blockIdx.x;
     const int cb = (g / (N_XCD * row_blocks)) * N_XCD + g % N_XCD, rb = (g / N_XCD) % row_blocks;
     if (cb >= col_blocks) return;
-    const int m_base = rb * 16;
+    const int m_base = rb * 16 * MT;
     const int n0 = (SPLIT_K ? cb : cb * nw + wave) * 16;
     const int k_first = SPLIT_K ? wave * 32 : 0;      // first k step of this wavefront
     const int k_step = SPLIT_K ? nw * 32 : 32;
@@ -290,12 +318,27 @@ gemm_bf16_skinny(const void* __restrict__ Ain, int lda, const bf16_t* __restrict
     // latency overlaps it.
     constexpr int PRE = 6;
     bf16x8 bpre[PRE];
-    if (LN_FUSED) {
+    if (IN_LDS) {
 #pragma unroll
         for (int u = 0; u < PRE; ++u) {
             const int k = k_first + u * k_step + 8 * kq;
             bpre[u] = (k < K && n_ok) ? *reinterpret_cast<const bf16x8*>(wrow + k) : zero;
         }
+    }
+    if (ASRC == A_STAGED) {
+        // the workgroup's rows of A, copied once into LDS for all its wavefronts
+        const bf16_t* A = static_cast<const bf16_t*>(Ain);
+        const int kv = K / 8;
+        for (int idx = tid; idx < 16 * MT * kv; idx += blockDim.x) {
+            const int m = idx / kv, c = idx % kv;
+            const bf16x8 v = (m_base + m < M)
+                                 ? *reinterpret_cast<const bf16x8*>(A + static_cast<size_t>(m_base + m) * lda + 8 * c)
+                                 : zero;
+            *reinterpret_cast<bf16x8*>(a_s + static_cast<size_t>(m) * a_stride + 8 * c) = v;
+        }
+        __syncthreads();
+    }
+    if (LN_FUSED) {
         // one wavefront per row: the row lives in registers (K <= 2048, K % 4 == 0), mean, then
         // variance of the centred values, all in fp32
         const float* x = static_cast<const float*>(Ain);
@@ -351,7 +394,7 @@ gemm_bf16_skinny(const void* __restrict__ Ain, int lda, const bf16_t* __restrict
 
     const bf16_t* A = static_cast<const bf16_t*>(Ain);
     int k_start = k_first;
-    if (LN_FUSED) {
+    if (IN_LDS) {
 #pragma unroll
         for (int u = 0; u < PRE; ++u) {
             const int kb = k_first + u * k_step;
@@ -377,7 +420,7 @@ gemm_bf16_skinny(const void* __restrict__ Ain, int lda, const bf16_t* __restrict
         for (int i = 0; i < MT; ++i) {
             const int m = i * 16 + row16;
             bf16x8 a;
-            if (LN_FUSED) a = kin ? *reinterpret_cast<const bf16x8*>(a_s + static_cast<size_t>(m) * a_stride + k) : zero;
+            if (IN_LDS) a = kin ? *reinterpret_cast<const bf16x8*>(a_s + static_cast<size_t>(m) * a_stride + k) : zero;
             else a = (kin && m_base + m < M) ? *reinterpret_cast<const bf16x8*>(A + static_cast<size_t>(m_base + m) * lda + k) : zero;
             acc[i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, acc[i], 0, 0, 0);
         }
@@ -432,18 +475,55 @@ static int launch_skinny(const void* A, int lda, const bf16_t* W, int ldw, const
     // Narrow products: 16 rows per workgroup and one workgroup per 16 rows (more workgroups, each
     // reading only its rows). Wide products: every wavefront keeps all rows of its tile in
     // registers (up to 4 accumulators), so the weights are streamed once.
-    const int row_blocks = split_k ? (M + 15) / 16 : 1;
-    const int mt = split_k ? 1 : (M + 15) / 16;
+    int row_blocks = split_k ? (M + 15) / 16 : 1;
+    int mt = split_k ? 1 : (M + 15) / 16;
+    // Wide products without the fused norm: every wavefront needs all rows of A for its tile, as
+    // many bytes as the tile's weights or more, so the workgroup copies its rows into LDS once
+    // (at most 160 KB: more rows than fit are split over row blocks).
+    const bool staged = !LN_FUSED && !split_k;
+    size_t staged_bytes = 0;
+    if (staged) {
+        const size_t row16_bytes = static_cast<size_t>(16) * (K + 8) * sizeof(bf16_t);
+        int fit = static_cast<int>(160 * 1024 / row16_bytes);
+        if (fit < 1) return -2;
+        if (fit > 4) fit = 4;
+        row_blocks = (mt + fit - 1) / fit;
+        mt = (mt + row_blocks - 1) / row_blocks;
+        staged_bytes = row16_bytes * mt;
+    }
     int nw;
     if (split_k) {
         nw = LN_FUSED ? 8 : 16;
         while (nw > 4 && nw * 3 > steps) nw >>= 1;      // at least 256 threads: one per output of the tile
     } else {
-        nw = LN_FUSED ? 8 : 4;      // with the norm fused, its rows spread over more wavefronts
+        // one round of workgroups over the 256 compute units, each wavefront one tile
+        // (the fused norm holds a row in registers: at most 8 wavefronts)
+        const int nw_max = LN_FUSED ? 8 : 16;
+        nw = (tiles * row_blocks + 255) / 256;
+        nw = nw < 4 ? 4 : (nw > nw_max ? nw_max : nw);
     }
     const int col_blocks = split_k ? tiles : (tiles + nw - 1) / nw;
     const dim3 grid((col_blocks + N_XCD - 1) / N_XCD * N_XCD * row_blocks), block(nw * 64);
     size_t smem = split_k ? static_cast<size_t>(nw) * mt * 256 * sizeof(float) : 0;
+    if (staged) {
+#define SKINNY_STAGED(MTV)                                                                             \
+    case MTV: {                                                                                        \
+        auto kernel = gemm_bf16_skinny<MTV, A_STAGED, false>;                                          \
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),                      \
+                                           hipFuncAttributeMaxDynamicSharedMemorySize,                 \
+                                           static_cast<int>(staged_bytes));                            \
+        if (e != hipSuccess) return static_cast<int>(e);                                               \
+        kernel<<<grid, block, staged_bytes, stream>>>(A, lda, W, ldw, bias, C, ldc, M, N, K, mode, gamma, beta, \
+                                                      eps, rows, col_blocks, row_blocks);              \
+        break;                                                                                         \
+    }
+        switch (mt) {
+            SKINNY_STAGED(1) SKINNY_STAGED(2) SKINNY_STAGED(3) SKINNY_STAGED(4)
+            default: return -2;
+        }
+#undef SKINNY_STAGED
+        return 0;
+    }
     if (LN_FUSED) {
         smem += static_cast<size_t>(16) * mt * (K + 8) * sizeof(bf16_t);
         if (K > 2048 || (reinterpret_cast<uintptr_t>(A) & 15) || lda % 4 != 0 ||
@@ -453,11 +533,11 @@ static int launch_skinny(const void* A, int lda, const bf16_t* W, int ldw, const
     if (smem > 64 * 1024) return -2;
 #define SKINNY_WIDE(MTV)                                                                              \
     case MTV:                                                                                         \
-        gemm_bf16_skinny<MTV, LN_FUSED, false><<<grid, block, smem, stream>>>(                        \
+        gemm_bf16_skinny<MTV, LN_FUSED ? A_NORMED : A_GLOBAL, false><<<grid, block, smem, stream>>>(                        \
             A, lda, W, ldw, bias, C, ldc, M, N, K, mode, gamma, beta, eps, rows, col_blocks, row_blocks); \
         break;
     if (split_k) {
-        gemm_bf16_skinny<1, LN_FUSED, true><<<grid, block, smem, stream>>>(
+        gemm_bf16_skinny<1, LN_FUSED ? A_NORMED : A_GLOBAL, true><<<grid, block, smem, stream>>>(
             A, lda, W, ldw, bias, C, ldc, M, N, K, mode, gamma, beta, eps, rows, col_blocks, row_blocks);
     } else {
         switch (mt) {
@@ -487,12 +567,21 @@ int mllm_gemm_bf16(const void* A, int lda, const void* W, int ldw, const float* 
         // few rows: weight-streaming kernel
     } else if (M <= 32) {
         launch_tiled<1, 4, 1, 1, 64, 3>(a, lda, w, ldw, bias, C, ldc, M, N, K, mode, stream);
-    } else if (static_cast<long>((M + 127) / 128) * ((N + 127) / 128) >= 512) {
-        // enough 128x128 tiles to fill 256 CUs twice: 8 wavefronts (4x2), each 32x64 of the tile
-        launch_tiled<4, 2, 1, 2, 32, 4>(a, lda, w, ldw, bias, C, ldc, M, N, K, mode, stream);
     } else {
-        // measured on GPT-2 shapes (2048 rows): 64x64 tiles keep more workgroups in flight and win
-        launch_tiled<2, 2, 1, 1, 64, 3>(a, lda, w, ldw, bias, C, ldc, M, N, K, mode, stream);
+        // Tile choice, measured at 2048 rows on GPT-2 shapes: a large tile moves fewer bytes per
+        // flop, but pays only when its workgroups fill the 256 compute units in one round (or in
+        // many); otherwise 64x64 tiles, several of them resident per unit, balance best.
+        auto blocks = [&](int bm, int bn) { return static_cast<long>((M + bm - 1) / bm) * ((N + bn - 1) / bn); };
+        auto one_round = [](long n) { return n >= 192 && n <= 256; };
+        if (one_round(blocks(128, 192))) {
+            launch_tiled<4, 2, 1, 3, 32, 4>(a, lda, w, ldw, bias, C, ldc, M, N, K, mode, stream);     // 128x192
+        } else if (blocks(128, 128) >= 512 || one_round(blocks(128, 128))) {
+            launch_tiled<2, 2, 2, 2, 32, 6>(a, lda, w, ldw, bias, C, ldc, M, N, K, mode, stream);     // 128x128
+        } else if (one_round(blocks(64, 96))) {
+            launch_tiled<2, 3, 1, 1, 64, 3>(a, lda, w, ldw, bias, C, ldc, M, N, K, mode, stream);     // 64x96
+        } else {
+            launch_tiled<2, 2, 1, 1, 64, 4>(a, lda, w, ldw, bias, C, ldc, M, N, K, mode, stream);     // 64x64
+        }
     }
     MLLM_LAUNCH_CHECK();
     return 0;

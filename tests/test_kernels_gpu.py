@@ -114,6 +114,30 @@ def test_linear(ops, dtype, M, N, K, epi):
     assert (out.cpu().double() - ref).abs().max().item() <= tol
 
 
+@pytest.mark.parametrize("M,N,K", [(2000, 2300, 776),      # 128x192 tiles, one round, ragged in M, N and K
+                                   (2048, 3072, 768),      # 128x192 tiles, no edge
+                                   (2040, 1800, 200),      # 128x128 tiles, one round, ragged
+                                   (2900, 3000, 72),       # 128x128 tiles, many rounds, ragged
+                                   (2040, 760, 136),       # 64x96 tiles, one round, ragged
+                                   (2048, 768, 3072),      # 64x96 tiles, long K
+                                   (1000, 1000, 40),       # 64x64 tiles, K below one k tile
+                                   (512, 2304, 768)])      # 64x64 tiles
+@pytest.mark.parametrize("epi", ["store", "add_residual"])
+def test_linear_bf16_tile_choices(ops, M, N, K, epi):
+    """Every tile shape of the many-row product, with edges in all three dimensions."""
+    g = torch.Generator().manual_seed(M + 3 * N + 7 * K)
+    a = _rand((M, K), torch.bfloat16, g)
+    w = _rand((N, K), torch.bfloat16, g, std=1.0 / math.sqrt(K))
+    bias = 0.5 * _rand((N,), torch.float32, g)
+    f32_out = epi == "add_residual"
+    out0 = _rand((M, N), torch.float32 if f32_out else torch.bfloat16, g)
+    out = out0.clone().to(DEV)
+    ops.linear(a.to(DEV), w.to(DEV), bias.to(DEV), out, epi)
+    ref = plain_ops.linear(a, w, bias, out0.double().clone(), epi)
+    err = (out.cpu().double() - ref).abs().max().item()
+    assert err <= (2e-5 + 2e-5 * math.sqrt(K) if f32_out else 4e-2), err
+
+
 @pytest.mark.parametrize("M", [1, 8, 16, 17, 48, 64])
 @pytest.mark.parametrize("N,K", [(2304, 768), (768, 3072), (1000, 96), (50257, 768), (72, 1600), (4800, 1600),
                                  (1600, 6400), (1024, 4096)])
