@@ -16,7 +16,7 @@
 #include "common.h"
 
 #define DEC_MAX_WAVES 16
-#define DEC_TABLE_LDS 1024   // block-table entries staged in LDS (longer tables are read from memory)
+#define DEC_TABLE_LDS 4096   // block-table entries staged in LDS: the most pages one workgroup's keys may span
 #define DEC_UNROLL 8
 
 // 16 bytes of a row: kept raw in registers while the load is in flight, widened to fp32 when used.
@@ -43,8 +43,9 @@ __device__ __forceinline__ uint4 load_raw16(const T* p) { return *reinterpret_ca
 template <int N>
 __device__ __forceinline__ void merge_state(float& m, float& l, float (&o)[N], float m2, float l2,
                                             const float (&o2)[N]) {
+    // empty states carry a large negative finite maximum and zero sums: their weight is 0 or
+    // (both empty) irrelevant
     const float mn = fmaxf(m, m2);
-    if (mn == -INFINITY) return;          // both empty
     const float a = fast_exp2(m - mn), b = fast_exp2(m2 - mn);
     l = l * a + l2 * b;
 #pragma unroll
@@ -83,81 +84,110 @@ decode_attention_kernel(const T* __restrict__ q, int q_stride, int q_col,
     const int per = (n_keys + nsplit - 1) / nsplit;
     const int kb = lo + split * per;
     const int ke = min(p + 1, kb + per);
-    const int* gtable = block_tables + static_cast<size_t>(b) * max_blocks;
-    // The sequence's block table goes to LDS first, so that no key load waits for a table load.
-    const int n_blocks_needed = p / page_size + 1;
-    const bool lds_table = n_blocks_needed <= DEC_TABLE_LDS;
-    if (lds_table) {
-        for (int i = threadIdx.x; i < n_blocks_needed; i += blockDim.x) sm_table[i] = gtable[i];
-        __syncthreads();
+    // With `slots`, the token's own key and value are not in the pages yet: they are read from
+    // its row of q (columns k_col, v_col), and written to the pages by the first query head of
+    // each key/value head. That key is taken by one lane group after the loop over the pages.
+    const bool append = slots != nullptr;
+    const bool own_here = append && ke == p + 1 && kb <= p;     // this workgroup's range holds the token itself
+    const int ke_pages = own_here ? p : ke;                     // keys [kb, ke_pages) come from the pages
+    const size_t col = static_cast<size_t>(hk) * DH + c * EPL;
+    const int shift = __ffs(page_size) - 1;                     // page sizes are powers of two
+
+    // The block table entries of this workgroup's keys go to LDS first, so that no key load waits
+    // for a table load.
+    const int first_blk = kb >> shift;
+    const int n_blk = ke_pages > kb ? ((ke_pages - 1) >> shift) - first_blk + 1 : 0;
+    {
+        const int* gtable = block_tables + static_cast<size_t>(b) * max_blocks + first_blk;
+        for (int i = threadIdx.x; i < n_blk; i += blockDim.x) sm_table[i] = gtable[i];
     }
-    const int* table = lds_table ? sm_table : gtable;
-    // pages of a power-of-two size are addressed with a shift and a mask
-    const bool pow2 = (page_size & (page_size - 1)) == 0;
-    const int shift = pow2 ? __ffs(page_size) - 1 : 0;
 
     float qf[EPL];
     Vec16<T>::widen(load_raw16(q + static_cast<size_t>(t) * q_stride + q_col + h * DH + c * EPL), qf);
 #pragma unroll
     for (int e = 0; e < EPL; ++e) qf[e] *= scale_log2e;
+    uint4 k_own = make_uint4(0, 0, 0, 0), v_own = make_uint4(0, 0, 0, 0);
+    const bool own_lanes = own_here && wave == 0 && g == 0;
+    if (own_lanes) {
+        const T* src = q + static_cast<size_t>(t) * q_stride + col;
+        k_own = load_raw16(src + k_col);
+        v_own = load_raw16(src + v_col);
+        const int slot = slots[t];
+        if (slot >= 0 && h % (n_heads / n_kv_heads) == 0) {
+            const size_t wrow = static_cast<size_t>(slot) * kv_dim + col;
+            *reinterpret_cast<uint4*>(k_pages_w + wrow) = k_own;
+            *reinterpret_cast<uint4*>(v_pages_w + wrow) = v_own;
+        }
+    }
+    __syncthreads();       // the table is in LDS
 
-    float m = -INFINITY, l = 0.f, o[EPL];
+    // Running state (maximum in base 2, sum, output slice). The maximum starts at a large
+    // negative finite number, so that no difference of two of them is NaN.
+    constexpr float NEG = -1.0e30f;
+    float m = NEG, l = 0.f, o[EPL];
 #pragma unroll
     for (int e = 0; e < EPL; ++e) o[e] = 0.f;
-    const size_t col = static_cast<size_t>(hk) * DH + c * EPL;
-    // With `slots`, the token's own key and value are not in the pages yet: they are read from
-    // its row of q (columns k_col, v_col) and written to the pages here, by the first query head
-    // of each key/value head.
-    const bool append = slots != nullptr;
-    const bool writer = append && (h % (n_heads / n_kv_heads) == 0) && slots[t] >= 0;
 
-    for (int j0 = kb + wave * KPW; j0 < ke; j0 += n_waves * KPW * DEC_UNROLL) {
+    // A wavefront takes DEC_UNROLL groups of 64/LPK keys at a time. All their loads are issued
+    // first, unconditionally (a key beyond the range loads the last key of the range again and is
+    // masked when used): a load under a condition would make every later one wait for it.
+    const int mask = page_size - 1;
+    for (int j0 = kb + wave * KPW; j0 < ke_pages; j0 += n_waves * KPW * DEC_UNROLL) {
         uint4 kraw[DEC_UNROLL], vraw[DEC_UNROLL];
-        bool valid[DEC_UNROLL];
 #pragma unroll
         for (int u = 0; u < DEC_UNROLL; ++u) {
-            const int j = j0 + u * n_waves * KPW + g;
-            valid[u] = j < ke;
-            if (valid[u]) {
-                if (append && j == p) {
-                    const T* src = q + static_cast<size_t>(t) * q_stride + col;
-                    kraw[u] = load_raw16(src + k_col);
-                    vraw[u] = load_raw16(src + v_col);
-                    if (writer) {
-                        const size_t wrow = static_cast<size_t>(slots[t]) * kv_dim + col;
-                        *reinterpret_cast<uint4*>(k_pages_w + wrow) = kraw[u];
-                        *reinterpret_cast<uint4*>(v_pages_w + wrow) = vraw[u];
-                    }
-                } else {
-                    const size_t row = pow2 ? ((static_cast<size_t>(table[j >> shift]) << shift) + (j & (page_size - 1)))
-                                            : (static_cast<size_t>(table[j / page_size]) * page_size + j % page_size);
-                    kraw[u] = load_raw16(k_pages + row * kv_dim + col);
-                    vraw[u] = load_raw16(v_pages + row * kv_dim + col);
-                }
-            }
+            const int j = min(j0 + u * n_waves * KPW + g, ke_pages - 1);
+            const size_t row = (static_cast<size_t>(sm_table[(j >> shift) - first_blk]) << shift) + (j & mask);
+            kraw[u] = load_raw16(k_pages + row * kv_dim + col);
+            vraw[u] = load_raw16(v_pages + row * kv_dim + col);
         }
+        float dot[DEC_UNROLL];
+        float mx = NEG;
 #pragma unroll
         for (int u = 0; u < DEC_UNROLL; ++u) {
-            float dot = 0.f;
-            if (valid[u]) {
-                float kf[EPL];
-                Vec16<T>::widen(kraw[u], kf);
+            float kf[EPL];
+            Vec16<T>::widen(kraw[u], kf);
+            float d = 0.f;
 #pragma unroll
-                for (int e = 0; e < EPL; ++e) dot = fmaf(qf[e], kf[e], dot);
-            }
+            for (int e = 0; e < EPL; ++e) d = fmaf(qf[e], kf[e], d);
 #pragma unroll
-            for (int off = 1; off < LPK; off <<= 1) dot += __shfl_xor(dot, off, MLLM_WAVE);
-            if (valid[u]) {
-                float vf[EPL];
-                Vec16<T>::widen(vraw[u], vf);
-                const float mn = fmaxf(m, dot);
-                const float a = fast_exp2(m - mn), pj = fast_exp2(dot - mn);
-                l = l * a + pj;
-#pragma unroll
-                for (int e = 0; e < EPL; ++e) o[e] = o[e] * a + pj * vf[e];
-                m = mn;
-            }
+            for (int off = 1; off < LPK; off <<= 1) d += __shfl_xor(d, off, MLLM_WAVE);
+            const bool valid = j0 + u * n_waves * KPW + g < ke_pages;
+            dot[u] = valid ? d : NEG;
+            mx = fmaxf(mx, dot[u]);
         }
+        // one rescale of the state for the whole batch of keys
+        const float mn = fmaxf(m, mx);
+        const float a = fast_exp2(m - mn);
+        l *= a;
+#pragma unroll
+        for (int e = 0; e < EPL; ++e) o[e] *= a;
+#pragma unroll
+        for (int u = 0; u < DEC_UNROLL; ++u) {
+            const float pj = dot[u] > NEG ? fast_exp2(dot[u] - mn) : 0.f;
+            float vf[EPL];
+            Vec16<T>::widen(vraw[u], vf);
+            l += pj;
+#pragma unroll
+            for (int e = 0; e < EPL; ++e) o[e] = fmaf(pj, vf[e], o[e]);
+        }
+        m = mn;
+    }
+    if (own_lanes) {
+        float kf[EPL], vf[EPL];
+        Vec16<T>::widen(k_own, kf);
+        Vec16<T>::widen(v_own, vf);
+        float d = 0.f;
+#pragma unroll
+        for (int e = 0; e < EPL; ++e) d = fmaf(qf[e], kf[e], d);
+#pragma unroll
+        for (int off = 1; off < LPK; off <<= 1) d += __shfl_xor(d, off, MLLM_WAVE);
+        const float mn = fmaxf(m, d);
+        const float a = fast_exp2(m - mn), pj = fast_exp2(d - mn);
+        l = l * a + pj;
+#pragma unroll
+        for (int e = 0; e < EPL; ++e) o[e] = o[e] * a + pj * vf[e];
+        m = mn;
     }
     // Merges the states of all lane groups and wavefronts; the result is valid in lane group 0
     // of wavefront 0.
@@ -211,7 +241,7 @@ decode_attention_kernel(const T* __restrict__ q, int q_stride, int q_col,
     __threadfence();
     // Last workgroup of this (token, head): lane group G takes split G (all loads in flight at
     // once), then the same merge as above.
-    m = -INFINITY; l = 0.f;
+    m = NEG; l = 0.f;
 #pragma unroll
     for (int e = 0; e < EPL; ++e) o[e] = 0.f;
     for (int s0 = 0; s0 < nsplit; s0 += n_waves * KPW) {
@@ -265,7 +295,7 @@ long mllm_decode_attention_ws_floats(int n_q, int n_heads, int head_dim, int nsp
 }
 
 // Returns 0, a HIP error code, or -1 for sizes the kernel refuses: head_dim * element size / 16
-// must be a power of two in [2, 64]. `counters` holds n_q*n_heads ints that are zero before the
+// must be a power of two in [2, 64], page_size a power of two, and max_blocks at most 4096. `counters` holds n_q*n_heads ints that are zero before the
 // first launch (the kernel leaves them zero). With `slots` (n_q rows of the page pools, < 0: none) the
 // tokens' own keys/values are taken from columns k_col/v_col of q and written to the pages by this
 // kernel; without, they must be in the pages already.
@@ -280,6 +310,7 @@ int mllm_decode_attention(const void* q, int q_stride, int q_col, const void* k_
     const int lpk = head_dim * esz / 16;
     if (head_dim * esz % 16 != 0 || n_heads % n_kv_heads != 0 || nsplit < 1 || nsplit > 65535 ||
         waves < 1 || waves > DEC_MAX_WAVES) return -1;
+    if (page_size < 1 || (page_size & (page_size - 1)) != 0 || max_blocks > DEC_TABLE_LDS) return -1;
     dim3 grid(n_q * n_heads, nsplit);
     float* ws_o = ws;
     float* ws_ml = ws + static_cast<size_t>(n_q) * n_heads * nsplit * head_dim;

@@ -33,8 +33,10 @@ union Frag8 {
     uint16_t h[8];
 };
 
+// (At most 2 wavefronts per SIMD: the compiler may then use 256 registers, and keeps both
+// prefetched tiles in registers instead of private memory.)
 template <int DH>
-__global__ void __launch_bounds__(256)
+__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, DH >= 128 ? 1 : 2)))
 prefill_attention_kernel(const bf16_t* __restrict__ q, int q_stride, int q_col,
                          const bf16_t* __restrict__ k_pages, const bf16_t* __restrict__ v_pages, int kv_dim,
                          const int* __restrict__ block_tables, int max_blocks,
@@ -86,12 +88,9 @@ prefill_attention_kernel(const bf16_t* __restrict__ q, int q_stride, int q_col,
 
     Frag8 qf[KS];
 #pragma unroll
-    for (int ks = 0; ks < KS; ++ks) {
-        qf[ks].q = make_uint4(0, 0, 0, 0);
-        if (q_ok)
-            qf[ks].q = *reinterpret_cast<const uint4*>(q + static_cast<size_t>(q_begin + qi) * q_stride + q_col +
-                                                       h * DH + 32 * ks + 8 * G);
-    }
+    for (int ks = 0; ks < KS; ++ks)      // a lane beyond the last query takes that query again; its scores are masked
+        qf[ks].q = *reinterpret_cast<const uint4*>(q + static_cast<size_t>(q_begin + min(qi, q_len - 1)) * q_stride +
+                                                   q_col + h * DH + 32 * ks + 8 * G);
 
     float m = -INFINITY, l = 0.f;
     f32x4 o[DT];
@@ -99,72 +98,54 @@ prefill_attention_kernel(const bf16_t* __restrict__ q, int q_stride, int q_col,
     for (int dt = 0; dt < DT; ++dt) o[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
     const size_t kv_col = static_cast<size_t>(hk) * DH;
 
-    // Tiles are fetched into registers one tile ahead, so the gather of the next keys and values
-    // is in flight while the matrix cores work on the current ones.
-    constexpr int K_ITEMS = (PF_BN * (DH / 8) + 255) / 256;          // 16-byte key chunks per thread
-    constexpr int V_ITEMS = ((PF_BN / 2) * (DH / 8) + 255) / 256;    // (key pair, 8 dims) items per thread
-    struct TileRegs {
-        uint4 rk[K_ITEMS], rv0[V_ITEMS], rv1[V_ITEMS];
-    };
-    TileRegs regs_a, regs_b;
-    auto fetch = [&](TileRegs& t, int kt) {
-        uint4 (&rk)[K_ITEMS] = t.rk;
-        uint4 (&rv0)[V_ITEMS] = t.rv0;
-        uint4 (&rv1)[V_ITEMS] = t.rv1;
+    // Tiles are fetched into registers ahead of their use, so the gather of the next keys and
+    // values is in flight while the matrix cores work on the current ones. Every load of a fetch
+    // is issued unconditionally, from a key clamped into [k_lo, p_last] (always a held page): a
+    // load under a condition would make the compiler wait for all loads in flight. Keys outside
+    // that range are masked in the scores, so what was loaded in their place never counts.
+    constexpr int K_ITEMS = PF_BN * (DH / 8) / 256;          // 16-byte key chunks per thread
+    constexpr int V_ITEMS = (PF_BN / 2) * (DH / 8) / 256;    // (key pair, 8 dims) items per thread
+    static_assert(K_ITEMS * 256 == PF_BN * (DH / 8) && V_ITEMS * 256 == (PF_BN / 2) * (DH / 8), "whole items per thread");
+    typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+    u32x4 ak[K_ITEMS], av0[V_ITEMS], av1[V_ITEMS];      // register set a
+    u32x4 bk[K_ITEMS], bv0[V_ITEMS], bv1[V_ITEMS];      // register set b
+    auto fetch = [&](u32x4 (&rk)[K_ITEMS], u32x4 (&rv0)[V_ITEMS], u32x4 (&rv1)[V_ITEMS], int kt) {
         const int j_base = kt * PF_BN;
 #pragma unroll
         for (int u = 0; u < K_ITEMS; ++u) {
             const int it = tid + u * 256;
             const int row = it / (DH / 8), ch = it % (DH / 8);
-            const int j = j_base + row;
-            // always a held page (clamped); what lies outside [k_lo, p_last] becomes zero afterwards
-            const int jc = min(max(j, k_lo), p_last);
-            rk[u] = make_uint4(0, 0, 0, 0);
-            if (K_ITEMS * 256 == PF_BN * (DH / 8) || it < PF_BN * (DH / 8)) {
-                const uint4 v = *reinterpret_cast<const uint4*>(k_pages + page_row(jc) * kv_dim + kv_col + 8 * ch);
-                if (j == jc) rk[u] = v;
-            }
+            const int jc = min(max(j_base + row, k_lo), p_last);
+            rk[u] = *reinterpret_cast<const u32x4*>(k_pages + page_row(jc) * kv_dim + kv_col + 8 * ch);
         }
 #pragma unroll
         for (int u = 0; u < V_ITEMS; ++u) {
             const int it = tid + u * 256;
             const int jp = it / (DH / 8), ch = it % (DH / 8);
             const int j0 = j_base + 2 * jp;
-            rv0[u] = make_uint4(0, 0, 0, 0);
-            rv1[u] = make_uint4(0, 0, 0, 0);
-            if (V_ITEMS * 256 == (PF_BN / 2) * (DH / 8) || it < (PF_BN / 2) * (DH / 8)) {
-                const int jc0 = min(max(j0, k_lo), p_last), jc1 = min(max(j0 + 1, k_lo), p_last);
-                const uint4 a = *reinterpret_cast<const uint4*>(v_pages + page_row(jc0) * kv_dim + kv_col + 8 * ch);
-                const uint4 c = *reinterpret_cast<const uint4*>(v_pages + page_row(jc1) * kv_dim + kv_col + 8 * ch);
-                if (j0 == jc0) rv0[u] = a;
-                if (j0 + 1 == jc1) rv1[u] = c;
-            }
+            const int jc0 = min(max(j0, k_lo), p_last), jc1 = min(max(j0 + 1, k_lo), p_last);
+            rv0[u] = *reinterpret_cast<const u32x4*>(v_pages + page_row(jc0) * kv_dim + kv_col + 8 * ch);
+            rv1[u] = *reinterpret_cast<const u32x4*>(v_pages + page_row(jc1) * kv_dim + kv_col + 8 * ch);
         }
     };
-    auto stage = [&](const TileRegs& t) {
+    auto stage = [&](const u32x4 (&rk)[K_ITEMS], const u32x4 (&rv0)[V_ITEMS], const u32x4 (&rv1)[V_ITEMS]) {
         // keys row-major; values transposed: 8 dims of two neighbouring keys become 8 words
-        const uint4 (&rk)[K_ITEMS] = t.rk;
-        const uint4 (&rv0)[V_ITEMS] = t.rv0;
-        const uint4 (&rv1)[V_ITEMS] = t.rv1;
 #pragma unroll
         for (int u = 0; u < K_ITEMS; ++u) {
             const int it = tid + u * 256;
-            if (it < PF_BN * (DH / 8))
-                *reinterpret_cast<uint4*>(Ks + (it / (DH / 8)) * KSTRIDE + 8 * (it % (DH / 8))) = rk[u];
+            *reinterpret_cast<u32x4*>(Ks + (it / (DH / 8)) * KSTRIDE + 8 * (it % (DH / 8))) = rk[u];
         }
 #pragma unroll
         for (int u = 0; u < V_ITEMS; ++u) {
             const int it = tid + u * 256;
-            if (it < (PF_BN / 2) * (DH / 8)) {
-                const int jp = it / (DH / 8), ch = it % (DH / 8);
-                Frag8 v0, v1;
-                v0.q = rv0[u];
-                v1.q = rv1[u];
+            const int jp = it / (DH / 8), ch = it % (DH / 8);
+            Frag8 v0, v1;
+            v0.v = __builtin_bit_cast(bf16x8, rv0[u]);
+            v1.v = __builtin_bit_cast(bf16x8, rv1[u]);
 #pragma unroll
-                for (int i = 0; i < 8; ++i)
-                    *reinterpret_cast<uint32_t*>(Vt + (8 * ch + i) * PF_VT_STRIDE + 2 * jp) =
-                        static_cast<uint32_t>(v0.h[i]) | (static_cast<uint32_t>(v1.h[i]) << 16);
-            }
+            for (int i = 0; i < 8; ++i)
+                *reinterpret_cast<uint32_t*>(Vt + (8 * ch + i) * PF_VT_STRIDE + 2 * jp) =
+                    static_cast<uint32_t>(v0.h[i]) | (static_cast<uint32_t>(v1.h[i]) << 16);
         }
     };
 
@@ -245,22 +226,23 @@ prefill_attention_kernel(const bf16_t* __restrict__ q, int q_stride, int q_col,
         if (full) compute(kt, std::false_type{}); else compute(kt, std::true_type{});
     };
 
-    // Two register sets, each fetched two tiles ahead of its use.
+    // Two register sets, each fetched two tiles ahead of its use. The loop body has no branch
+    // around a load; past the last tile the fetches repeat clamped keys and nothing is computed.
     const int kt_first = k_lo / PF_BN, kt_last = p_last / PF_BN;
-    fetch(regs_a, kt_first);
-    if (kt_first + 1 <= kt_last) fetch(regs_b, kt_first + 1);
+    fetch(ak, av0, av1, kt_first);
+    __builtin_amdgcn_sched_barrier(0);     // set a's loads stay the older ones, as on every later iteration
+    fetch(bk, bv0, bv1, kt_first + 1);
     for (int kt = kt_first; kt <= kt_last; kt += 2) {
         lds_barrier();                     // the previous tile's readers are done
-        stage(regs_a);
+        stage(ak, av0, av1);
         lds_barrier();
-        if (kt + 2 <= kt_last) fetch(regs_a, kt + 2);
+        fetch(ak, av0, av1, kt + 2);
         run_tile(kt);
-        if (kt + 1 > kt_last) break;
         lds_barrier();
-        stage(regs_b);
+        stage(bk, bv0, bv1);
         lds_barrier();
-        if (kt + 3 <= kt_last) fetch(regs_b, kt + 3);
-        run_tile(kt + 1);
+        fetch(bk, bv0, bv1, kt + 3);
+        if (kt + 1 <= kt_last) run_tile(kt + 1);
     }
     l += __shfl_xor(l, 16, MLLM_WAVE);
     l += __shfl_xor(l, 32, MLLM_WAVE);

@@ -10,6 +10,8 @@
 // Requires K % 8 == 0 and 16-byte aligned rows; any M and N.
 #include "common.h"
 
+#include <algorithm>
+
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 
@@ -253,18 +255,19 @@ static void launch_tiled(const bf16_t* a, int lda, const bf16_t* w, int ldw, con
 // v_mfma_f32_16x16x32_bf16; a workgroup owns 16 rows of the output (more rows: more workgroups
 // per column range, placed on the same XCD so that the weights they share come from its L2).
 //   SPLIT_K:  one workgroup per 16-column tile, its wavefronts split K (wavefront w takes the
-//             32-wide k steps w, w+NW, ...) and their partial sums are added in LDS in a fixed
+//             64-element k blocks w, w+NW, ...) and their partial sums are added in LDS in a fixed
 //             order: for the narrow products, where tiles alone are too few to fill the chip.
 //   !SPLIT_K: one wavefront per tile over the whole of K (wide products such as the logits head).
-// The activations (a few KB, shared by all workgroups) are read from L2, or, with LN_FUSED,
-// normalised from the fp32 stream into LDS first: LayerNorm
+// The activations come from global memory (A_GLOBAL: a few KB, shared by all workgroups, read
+// from L2), are copied into LDS once per workgroup (A_STAGED: wide products), or are normalised
+// from the fp32 stream into LDS first (A_NORMED): LayerNorm
 // (/root/reference/src/kernels/layernorm.cu:32-49) fused into the product that follows it.
 // ---------------------------------------------------------------------------------------------
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 
 enum { A_GLOBAL = 0, A_NORMED = 1, A_STAGED = 2 };
 
-template <int MT, int ASRC, bool SPLIT_K>
+template <int MT, int ASRC, bool SPLIT_K, int U>
 __global__ void __launch_bounds__(ASRC == A_NORMED ? 512 : 1024)
 gemm_bf16_skinny(const void* __restrict__ Ain, int lda, const bf16_t* __restrict__ W, int ldw,
                  const float* __restrict__ bias, void* __restrict__ C, int ldc, int M, int N, int K, int mode,
@@ -283,8 +286,12 @@ gemm_bf16_skinny(const void* __restrict__ Ain, int lda, const bf16_t* __restrict
     if (cb >= col_blocks) return;
     const int m_base = rb * 16 * MT;
     const int n0 = (SPLIT_K ? cb : cb * nw + wave) * 16;
-    const int k_first = SPLIT_K ? wave * 32 : 0;      // first k step of this wavefront
-    const int k_step = SPLIT_K ? nw * 32 : 32;
+    // K is dealt out in blocks of 64 elements, one 128-byte line of a weight row: lane group kq
+    // takes elements 16*kq .. 16*kq+15 of a block, the first 8 in one MFMA and the rest in the
+    // next (the k index of an MFMA may be permuted as long as both operands agree), so that a
+    // wavefront uses every line it touches whole.
+    const int k_first = SPLIT_K ? wave * 64 : 0;      // first k block of this wavefront
+    const int k_stride = SPLIT_K ? nw * 64 : 64;      // distance between its k blocks
     const size_t red_bytes = SPLIT_K ? static_cast<size_t>(nw) * MT * 256 * sizeof(float) : 0;
     float* red = reinterpret_cast<float*>(smem_raw);                       // [nw][MT][256]
     bf16_t* a_s = reinterpret_cast<bf16_t*>(smem_raw + red_bytes);         // [16*MT][K+8]
@@ -314,116 +321,182 @@ gemm_bf16_skinny(const void* __restrict__ Ain, int lda, const bf16_t* __restrict
         }
     }
 
-    // The first weight fragments of this wavefront are requested before the norm, so that their
-    // latency overlaps it.
-    constexpr int PRE = 6;
-    bf16x8 bpre[PRE];
-    if (IN_LDS) {
+    // A wavefront takes its k blocks in chunks of H = U/2. All loads of a chunk are issued
+    // together and without a condition inside (a load under a condition makes the compiler wait
+    // for every load in flight); the conditions that decide whether a chunk is loaded at all are
+    // uniform over the wavefront. No load goes to a line that another load may still have in
+    // flight: loads that hit such a line queue up behind it in the vector cache. Two chunks
+    // alternate so that one is in flight while the other is multiplied; the first is requested
+    // before the norm or the copy of A, so that its latency overlaps them. Blocks left over
+    // (fewer than H) follow one by one. Only the last block of K can be short: its lanes beyond K
+    // load the row's last 16 bytes and their weight fragment is zeroed.
+    constexpr int H = U / 2;
+    static_assert(U % 2 == 0, "whole k blocks per chunk");
+    const bf16_t* A = static_cast<const bf16_t*>(Ain);
+    const bf16_t* arow = A;       // A_GLOBAL: this lane's row of A (rows beyond M: the last one, never stored)
+    if (ASRC == A_GLOBAL) arow = A + static_cast<size_t>(min(m_base + row16, M - 1)) * lda;
+    const int n_blocks = k_first < K ? (K - k_first + k_stride - 1) / k_stride : 0;   // of this wavefront
+    const int n_chunks = n_blocks / H;
+    struct Chunk {
+        bf16x8 b[U];
+        bf16x8 a[ASRC == A_GLOBAL ? U : 1];
+    };
+    auto load_steps = [&](Chunk& c, int u0, int k0) {      // the two steps of the k block at k0 into slots u0, u0+1
 #pragma unroll
-        for (int u = 0; u < PRE; ++u) {
-            const int k = k_first + u * k_step + 8 * kq;
-            bpre[u] = (k < K && n_ok) ? *reinterpret_cast<const bf16x8*>(wrow + k) : zero;
+        for (int half = 0; half < 2; ++half) {
+            const int k = min(k0 + 16 * kq + 8 * half, K - 8);
+            c.b[u0 + half] = *reinterpret_cast<const bf16x8*>(wrow + k);
+            if (ASRC == A_GLOBAL) c.a[u0 + half] = *reinterpret_cast<const bf16x8*>(arow + k);
+        }
+    };
+    auto mma_steps = [&](const Chunk& c, int u0, int k0) {
+#pragma unroll
+        for (int half = 0; half < 2; ++half) {
+            const int k = k0 + 16 * kq + 8 * half;
+            const bf16x8 b = k < K ? c.b[u0 + half] : zero;
+            const int kc = min(k, K - 8);
+#pragma unroll
+            for (int i = 0; i < MT; ++i) {
+                bf16x8 a;
+                if (IN_LDS) a = *reinterpret_cast<const bf16x8*>(a_s + static_cast<size_t>(i * 16 + row16) * a_stride + kc);
+                else a = c.a[u0 + half];
+                acc[i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, acc[i], 0, 0, 0);
+            }
+        }
+    };
+    auto load_chunk = [&](Chunk& c, int chunk) {            // chunk index within this wavefront's blocks
+#pragma unroll
+        for (int h = 0; h < H; ++h) load_steps(c, 2 * h, k_first + (chunk * H + h) * k_stride);
+        // the instruction scheduler must not sink these loads towards their uses: they are issued
+        // here to be in flight together
+        __builtin_amdgcn_sched_barrier(0);
+    };
+    auto mma_chunk = [&](const Chunk& c, int chunk) {
+#pragma unroll
+        for (int h = 0; h < H; ++h) mma_steps(c, 2 * h, k_first + (chunk * H + h) * k_stride);
+    };
+    // rows of the fp32 stream that this wavefront normalises (read before the weights are
+    // requested: loads complete in order, and the row addresses depend on these)
+    int src_row[2] = {0, 0};
+    if (LN_FUSED) {
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            const int m = min(m_base + wave + 8 * j, M - 1);      // 8 wavefronts, rows wave and wave + 8
+            src_row[j] = rows ? rows[m] : m;
         }
     }
+    Chunk c0, c1;
+    auto load_left = [&]() {                                // the blocks after the last whole chunk
+        const int first = n_chunks * H, left = n_blocks - first;
+#pragma unroll
+        for (int h = 0; h < H - 1; ++h)
+            if (h < left) load_steps(c1, 2 * h, k_first + (first + h) * k_stride);
+        __builtin_amdgcn_sched_barrier(0);
+    };
+    auto first_loads = [&]() {
+        if (n_chunks > 0) load_chunk(c0, 0);
+        else load_left();                                   // a wavefront without a whole chunk starts with these
+    };
+    first_loads();
     if (ASRC == A_STAGED) {
         // the workgroup's rows of A, copied once into LDS for all its wavefronts
-        const bf16_t* A = static_cast<const bf16_t*>(Ain);
-        const int kv = K / 8;
-        for (int idx = tid; idx < 16 * MT * kv; idx += blockDim.x) {
-            const int m = idx / kv, c = idx % kv;
-            const bf16x8 v = (m_base + m < M)
-                                 ? *reinterpret_cast<const bf16x8*>(A + static_cast<size_t>(m_base + m) * lda + 8 * c)
-                                 : zero;
-            *reinterpret_cast<bf16x8*>(a_s + static_cast<size_t>(m) * a_stride + 8 * c) = v;
+        // (four 16-byte pieces per thread requested together, then written)
+        const int kv = K / 8, total = 16 * MT * kv;
+        for (int base = tid; base < total; base += 4 * blockDim.x) {
+            bf16x8 v[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const int idx = min(base + j * static_cast<int>(blockDim.x), total - 1);
+                const int m = idx / kv, c = idx - m * kv;
+                v[j] = *reinterpret_cast<const bf16x8*>(A + static_cast<size_t>(min(m_base + m, M - 1)) * lda + 8 * c);
+            }
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const int idx = base + j * static_cast<int>(blockDim.x);
+                const int m = idx / kv, c = idx - m * kv;
+                if (idx < total)
+                    *reinterpret_cast<bf16x8*>(a_s + static_cast<size_t>(m) * a_stride + 8 * c) =
+                        (m_base + m < M) ? v[j] : zero;
+            }
         }
         __syncthreads();
     }
     if (LN_FUSED) {
-        // one wavefront per row: the row lives in registers (K <= 2048, K % 4 == 0), mean, then
-        // variance of the centred values, all in fp32
+        // 8 wavefronts, two rows each; a row lives in registers (K <= 2048, K % 4 == 0): mean,
+        // then variance of the centred values, all in fp32. Both rows and the scale and shift
+        // vectors are requested together, before anything is waited for.
         const float* x = static_cast<const float*>(Ain);
-        const int nq = K / 4;
+        const int nq = K / 4, n_u = (nq + 63) / 64;       // float4 per row; per lane (uniform)
         const float4* g4 = reinterpret_cast<const float4*>(gamma);
         const float4* b4 = reinterpret_cast<const float4*>(beta);
-        for (int m = wave; m < 16 * MT; m += nw) {
+        float4 gg[8], bb[8], v[2][8];
+        // whether this wavefront's two rows exist is uniform over it: rows beyond M are not read
+        const bool row_ok[2] = {m_base + wave < M, m_base + wave + 8 < M};
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            if (u < n_u) {
+                const int i = min(lane + 64 * u, nq - 1);
+                gg[u] = g4[i];
+                bb[u] = beta ? b4[i] : make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+                for (int j = 0; j < 2; ++j)
+                    if (row_ok[j]) v[j][u] = reinterpret_cast<const float4*>(x + static_cast<size_t>(src_row[j]) * lda)[i];
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            const int m = wave + 8 * j;
             bf16_t* dst = a_s + static_cast<size_t>(m) * a_stride;
-            if (m_base + m < M) {
-                const float4* xr = reinterpret_cast<const float4*>(
-                    x + static_cast<size_t>(rows ? rows[m_base + m] : m_base + m) * lda);
-                float4 v[8], gg[8], bb[8];
-                float s = 0.f;
+            if (!row_ok[j]) {
+                for (int i = lane; i < nq; i += 64) *reinterpret_cast<uint2*>(dst + 4 * i) = make_uint2(0, 0);
+                continue;
+            }
+            float s = 0.f;
 #pragma unroll
-                for (int u = 0; u < 8; ++u) {
-                    const int i = lane + 64 * u;
-                    const bool in = i < nq;
-                    v[u] = in ? xr[i] : make_float4(0.f, 0.f, 0.f, 0.f);
-                    gg[u] = in ? g4[i] : make_float4(0.f, 0.f, 0.f, 0.f);
-                    bb[u] = (in && beta) ? b4[i] : make_float4(0.f, 0.f, 0.f, 0.f);
-                    s += (v[u].x + v[u].y) + (v[u].z + v[u].w);
-                }
-                const float mean = wave_sum(s) / static_cast<float>(K);
-                float q = 0.f;
+            for (int u = 0; u < 8; ++u)
+                if (u < n_u && lane + 64 * u < nq) s += (v[j][u].x + v[j][u].y) + (v[j][u].z + v[j][u].w);
+            const float mean = wave_sum(s) / static_cast<float>(K);
+            float q = 0.f;
 #pragma unroll
-                for (int u = 0; u < 8; ++u) {
-                    if (lane + 64 * u < nq) {
-                        const float a = v[u].x - mean, b = v[u].y - mean, c = v[u].z - mean, d = v[u].w - mean;
-                        q += (a * a + b * b) + (c * c + d * d);
-                    }
+            for (int u = 0; u < 8; ++u) {
+                if (u < n_u && lane + 64 * u < nq) {
+                    const float a = v[j][u].x - mean, b = v[j][u].y - mean, c = v[j][u].z - mean, d = v[j][u].w - mean;
+                    q += (a * a + b * b) + (c * c + d * d);
                 }
-                const float inv = 1.0f / sqrtf(wave_sum(q) / static_cast<float>(K) + eps);
+            }
+            const float inv = 1.0f / sqrtf(wave_sum(q) / static_cast<float>(K) + eps);
 #pragma unroll
-                for (int u = 0; u < 8; ++u) {
-                    const int i = lane + 64 * u;
-                    if (i < nq) {
-                        bf16_t r0 = float_to_bf16((v[u].x - mean) * inv * gg[u].x + bb[u].x);
-                        bf16_t r1 = float_to_bf16((v[u].y - mean) * inv * gg[u].y + bb[u].y);
-                        bf16_t r2 = float_to_bf16((v[u].z - mean) * inv * gg[u].z + bb[u].z);
-                        bf16_t r3 = float_to_bf16((v[u].w - mean) * inv * gg[u].w + bb[u].w);
-                        uint2 pk;
-                        pk.x = static_cast<uint32_t>(r0.bits) | (static_cast<uint32_t>(r1.bits) << 16);
-                        pk.y = static_cast<uint32_t>(r2.bits) | (static_cast<uint32_t>(r3.bits) << 16);
-                        *reinterpret_cast<uint2*>(dst + 4 * i) = pk;
-                    }
+            for (int u = 0; u < 8; ++u) {
+                const int i = lane + 64 * u;
+                if (u < n_u && i < nq) {
+                    uint2 pk;
+                    pk.x = pack_bf16x2((v[j][u].x - mean) * inv * gg[u].x + bb[u].x, (v[j][u].y - mean) * inv * gg[u].y + bb[u].y);
+                    pk.y = pack_bf16x2((v[j][u].z - mean) * inv * gg[u].z + bb[u].z, (v[j][u].w - mean) * inv * gg[u].w + bb[u].w);
+                    *reinterpret_cast<uint2*>(dst + 4 * i) = pk;
                 }
-            } else {
-                for (int k = lane; k < K; k += 64) dst[k].bits = 0;
             }
         }
         __syncthreads();
     }
 
-    const bf16_t* A = static_cast<const bf16_t*>(Ain);
-    int k_start = k_first;
-    if (IN_LDS) {
-#pragma unroll
-        for (int u = 0; u < PRE; ++u) {
-            const int kb = k_first + u * k_step;
-            if (kb < K) {
-                const int k = kb + 8 * kq;
-                const bool kin = k < K;
-#pragma unroll
-                for (int i = 0; i < MT; ++i) {
-                    const int m = i * 16 + row16;
-                    bf16x8 a = kin ? *reinterpret_cast<const bf16x8*>(a_s + static_cast<size_t>(m) * a_stride + k) : zero;
-                    acc[i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, bpre[u], acc[i], 0, 0, 0);
-                }
-            }
+    if (n_chunks == 1) {
+        mma_chunk(c0, 0);
+    } else if (n_chunks > 1) {
+        // past the last chunk the prefetch takes chunk 0 again (long since arrived, never used)
+        for (int ci = 0; ci < n_chunks; ci += 2) {
+            load_chunk(c1, ci + 1 < n_chunks ? ci + 1 : 0);
+            mma_chunk(c0, ci);
+            load_chunk(c0, ci + 2 < n_chunks ? ci + 2 : 0);
+            if (ci + 1 < n_chunks) mma_chunk(c1, ci + 1);
         }
-        k_start = k_first + PRE * k_step;
     }
-#pragma unroll 8
-    for (int k0 = k_start; k0 < K; k0 += k_step) {
-        const int k = k0 + 8 * kq;
-        const bool kin = k < K;
-        bf16x8 b = (kin && n_ok) ? *reinterpret_cast<const bf16x8*>(wrow + k) : zero;
+    {
+        // blocks left over: fewer than H, loaded together
+        const int first = n_chunks * H, left = n_blocks - first;
+        if (n_chunks > 0) load_left();
 #pragma unroll
-        for (int i = 0; i < MT; ++i) {
-            const int m = i * 16 + row16;
-            bf16x8 a;
-            if (IN_LDS) a = kin ? *reinterpret_cast<const bf16x8*>(a_s + static_cast<size_t>(m) * a_stride + k) : zero;
-            else a = (kin && m_base + m < M) ? *reinterpret_cast<const bf16x8*>(A + static_cast<size_t>(m_base + m) * lda + k) : zero;
-            acc[i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, acc[i], 0, 0, 0);
-        }
+        for (int h = 0; h < H - 1; ++h)
+            if (h < left) mma_steps(c1, 2 * h, k_first + (first + h) * k_stride);
     }
     // accumulator layout of the 16x16 tile: register r of lane l holds row 4*(l/16) + r, column l%16
     if (!SPLIT_K) {
@@ -470,7 +543,7 @@ template <bool LN_FUSED>
 static int launch_skinny(const void* A, int lda, const bf16_t* W, int ldw, const float* bias, void* C, int ldc,
                          int M, int N, int K, int mode, const float* gamma, const float* beta, float eps,
                          const int* rows, hipStream_t stream) {
-    const int tiles = (N + 15) / 16, steps = (K + 31) / 32;
+    const int tiles = (N + 15) / 16;
     const bool split_k = tiles < 1024;
     // Narrow products: 16 rows per workgroup and one workgroup per 16 rows (more workgroups, each
     // reading only its rows). Wide products: every wavefront keeps all rows of its tile in
@@ -492,15 +565,19 @@ static int launch_skinny(const void* A, int lda, const bf16_t* W, int ldw, const
         staged_bytes = row16_bytes * mt;
     }
     int nw;
+    const int k_blocks = (K + 63) / 64;
     if (split_k) {
-        nw = LN_FUSED ? 8 : 16;
-        while (nw > 4 && nw * 3 > steps) nw >>= 1;      // at least 256 threads: one per output of the tile
+        // the wavefront count (at least 4: one thread per output of the tile) that leaves every
+        // wavefront the fewest k blocks; among equals the smallest, which has the least to add up
+        // (the fused norm is written for 8 wavefronts, two rows each)
+        nw = 4;
+        for (int cand = 5; cand <= 16; ++cand)
+            if ((k_blocks + cand - 1) / cand < (k_blocks + nw - 1) / nw) nw = cand;
+        if (LN_FUSED) nw = 8;
     } else {
         // one round of workgroups over the 256 compute units, each wavefront one tile
-        // (the fused norm holds a row in registers: at most 8 wavefronts)
-        const int nw_max = LN_FUSED ? 8 : 16;
         nw = (tiles * row_blocks + 255) / 256;
-        nw = nw < 4 ? 4 : (nw > nw_max ? nw_max : nw);
+        nw = nw < 4 ? 4 : (nw > 16 ? 16 : nw);
     }
     const int col_blocks = split_k ? tiles : (tiles + nw - 1) / nw;
     const dim3 grid((col_blocks + N_XCD - 1) / N_XCD * N_XCD * row_blocks), block(nw * 64);
@@ -508,7 +585,7 @@ static int launch_skinny(const void* A, int lda, const bf16_t* W, int ldw, const
     if (staged) {
 #define SKINNY_STAGED(MTV)                                                                             \
     case MTV: {                                                                                        \
-        auto kernel = gemm_bf16_skinny<MTV, A_STAGED, false>;                                          \
+        auto kernel = gemm_bf16_skinny<MTV, A_STAGED, false, 4>;                                        \
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),                      \
                                            hipFuncAttributeMaxDynamicSharedMemorySize,                 \
                                            static_cast<int>(staged_bytes));                            \
@@ -531,21 +608,24 @@ static int launch_skinny(const void* A, int lda, const bf16_t* W, int ldw, const
             return -2;
     }
     if (smem > 64 * 1024) return -2;
-#define SKINNY_WIDE(MTV)                                                                              \
-    case MTV:                                                                                         \
-        gemm_bf16_skinny<MTV, LN_FUSED ? A_NORMED : A_GLOBAL, false><<<grid, block, smem, stream>>>(                        \
-            A, lda, W, ldw, bias, C, ldc, M, N, K, mode, gamma, beta, eps, rows, col_blocks, row_blocks); \
-        break;
+    constexpr int ASRC = LN_FUSED ? A_NORMED : A_GLOBAL;
+#define SKINNY_LAUNCH(SPLIT, UV)                                                                       \
+    gemm_bf16_skinny<1, ASRC, SPLIT, UV><<<grid, block, smem, stream>>>(                               \
+        A, lda, W, ldw, bias, C, ldc, M, N, K, mode, gamma, beta, eps, rows, col_blocks, row_blocks)
     if (split_k) {
-        gemm_bf16_skinny<1, LN_FUSED ? A_NORMED : A_GLOBAL, true><<<grid, block, smem, stream>>>(
-            A, lda, W, ldw, bias, C, ldc, M, N, K, mode, gamma, beta, eps, rows, col_blocks, row_blocks);
-    } else {
-        switch (mt) {
-            SKINNY_WIDE(1) SKINNY_WIDE(2) SKINNY_WIDE(3) SKINNY_WIDE(4)
-            default: return -2;
+        // a chunk holds all k blocks of a wavefront when they are at most 3 (two chunks of
+        // fragments must fit the 128 registers of a 16-wavefront workgroup)
+        switch (std::min((k_blocks + nw - 1) / nw, 3)) {
+            case 1: SKINNY_LAUNCH(true, 2); break;
+            case 2: SKINNY_LAUNCH(true, 4); break;
+            default: SKINNY_LAUNCH(true, 6); break;
         }
+    } else {
+        // wide products (the logits head): normalising the rows once in a kernel of its own and
+        // staging them in LDS is faster than every workgroup normalising them again
+        return -2;
     }
-#undef SKINNY_WIDE
+#undef SKINNY_LAUNCH
     return 0;
 }
 
@@ -589,14 +669,14 @@ int mllm_gemm_bf16(const void* A, int lda, const void* W, int ldw, const float* 
 
 // LayerNorm of the fp32 rows x[M,K] (row m taken from x[rows[m]] when `rows` is given) fused into the
 // product with W[N,K]: C = epilogue(LN(x) W^T + bias).
-// M <= 16. Returns 0, a HIP error code, -1 for misaligned operands, or -2 when M or K is too large for the
-// fused kernel (the caller then runs the norm and the product separately).
+// M <= 64, N < 16384. Returns 0, a HIP error code, -1 for misaligned operands, or -2 when M, N or K is too
+// large for the fused kernel (the caller then runs the norm and the product separately).
 int mllm_ln_gemm_bf16(const float* x, int ldx, const int* rows, const float* gamma, const float* beta, float eps,
                       const void* W, int ldw, const float* bias, void* C, int ldc, int M, int N, int K, int mode,
                       hipStream_t stream) {
     if (M <= 0 || N <= 0) return 0;
     if (K % 8 != 0 || ldw % 8 != 0 || (reinterpret_cast<uintptr_t>(W) & 15)) return -1;
-    if (M > 16) return -2;
+    if (M > 64) return -2;
     int rc = launch_skinny<true>(x, ldx, static_cast<const bf16_t*>(W), ldw, bias, C, ldc, M, N, K, mode, gamma,
                                  beta, eps, rows, stream);
     if (rc != 0) return rc;

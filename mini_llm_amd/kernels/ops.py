@@ -158,13 +158,17 @@ def linear(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], out: 
     return out
 
 
+LN_FUSE_MAX_ROWS = 16      # above this many rows the norm is faster as a kernel of its own (measured)
+
+
 def ln_linear(x: torch.Tensor, gamma: torch.Tensor, beta: Optional[torch.Tensor], eps: float,
               w: torch.Tensor, bias: Optional[torch.Tensor], out: torch.Tensor, epilogue: str = "store",
               rows: Optional[torch.Tensor] = None) -> torch.Tensor:
     """out = epilogue(LayerNorm(x) @ w.T + bias) with x the fp32 stream [*,K] and w [N,K]; with
     ``rows`` (int32 [M]) row m of the input is x[rows[m]].
 
-    For bfloat16 weights and at most 16 rows the norm is fused into the product (one kernel);
+    For bfloat16 weights, at most 16 rows and fewer than 16384 columns the norm is fused into the
+    product (one kernel);
     otherwise the norm and the product run one after the other. Same numerics either way:
     statistics in fp32, the normalised rows rounded to w's dtype before the product.
     """
@@ -174,7 +178,7 @@ def ln_linear(x: torch.Tensor, gamma: torch.Tensor, beta: Optional[torch.Tensor]
     N = w.shape[0]
     if rows is not None:
         _i32(rows, "rows")
-    if (w.dtype == torch.bfloat16 and M <= 16 and x.dtype == torch.float32 and x.is_contiguous()
+    if (w.dtype == torch.bfloat16 and M <= LN_FUSE_MAX_ROWS and x.dtype == torch.float32 and x.is_contiguous()
             and gamma.data_ptr() % 16 == 0 and (beta is None or beta.data_ptr() % 16 == 0)):
         _rows2d(w, "w")
         _rows2d(out, "out")
@@ -263,7 +267,8 @@ def paged_attention(q: torch.Tensor, q_col: int, n_heads: int, n_kv_heads: int, 
     if (q.stride(0) * esz) % 16 or (q_col * esz) % 16 or (head_dim * esz) % 16 or q.data_ptr() % 16:
         raise KernelError("query rows and heads must be 16-byte aligned")
     lpk = head_dim * esz // 16
-    decode = max_q_len == 1 and lpk >= 2 and (lpk & (lpk - 1)) == 0
+    decode = (max_q_len == 1 and lpk >= 2 and (lpk & (lpk - 1)) == 0
+              and page_size & (page_size - 1) == 0 and block_tables.shape[1] <= 4096)
     k_col = v_col = 0
     slots = None
     if append is not None:
