@@ -55,6 +55,7 @@ def _rt():
         "mllm_sched_commit": (None, [vp]),
         "mllm_sched_on_token": (i, [vp, i64, i]),
         "mllm_sched_abort": (i, [vp, i64]),
+        "mllm_sched_stop": (i, [vp, i64]),
         "mllm_sched_has_work": (i, [vp]),
         "mllm_sched_state": (i, [vp, i64]),
         "mllm_sched_generated": (i, [vp, i64]),

@@ -21,6 +21,19 @@ __global__ void embed_kernel(const int* __restrict__ ids, const int* __restrict_
 }
 
 // ---------------------------------------------------------------------------
+// Token ids fed back on the device: ids[i] = prev[src[i]] where src[i] >= 0 (the request's
+// newest token is the one an earlier step sampled into prev and the host has not read yet);
+// other ids stay as the host wrote them.
+// ---------------------------------------------------------------------------
+__global__ void select_tokens_kernel(int* __restrict__ ids, const int* __restrict__ src,
+                                     const int* __restrict__ prev, int n, int n_prev) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    const int s = src[i];
+    if (s >= 0 && s < n_prev) ids[i] = prev[s];
+}
+
+// ---------------------------------------------------------------------------
 // LayerNorm over the last dimension, statistics in fp32, two passes:
 // mean, then biased variance of (x - mean); y = (x - mean) * rsqrt(var + eps) * g + b.
 // /root/reference/src/kernels/layernorm.cu:32-49. `rows` (optional) selects input rows.
@@ -159,6 +172,13 @@ int mllm_embed(const int* ids, const int* pos, const void* wte, const void* wpe,
         embed_kernel<float><<<T, 256, 0, stream>>>(ids, pos, (const float*)wte, (const float*)wpe, x, D);
     else
         embed_kernel<bf16_t><<<T, 256, 0, stream>>>(ids, pos, (const bf16_t*)wte, (const bf16_t*)wpe, x, D);
+    MLLM_LAUNCH_CHECK();
+    return 0;
+}
+
+int mllm_select_tokens(int* ids, const int* src, const int* prev, int n, int n_prev, hipStream_t stream) {
+    if (n <= 0) return 0;
+    select_tokens_kernel<<<(n + 255) / 256, 256, 0, stream>>>(ids, src, prev, n, n_prev);
     MLLM_LAUNCH_CHECK();
     return 0;
 }

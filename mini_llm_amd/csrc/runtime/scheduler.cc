@@ -223,6 +223,17 @@ int Scheduler::abort(int64_t id) {
     return 0;
 }
 
+int Scheduler::stop(int64_t id) {
+    auto it = reqs_.find(id);
+    if (it == reqs_.end()) return -2;
+    Req& r = it->second;
+    if (r.state == RequestState::Finished || r.state == RequestState::Failed) return 0;
+    plan_.erase(std::remove_if(plan_.begin(), plan_.end(),
+                               [id](const PlanEntry& e) { return e.id == id; }), plan_.end());
+    finish(r, RequestState::Finished);
+    return 0;
+}
+
 bool Scheduler::has_work() const {
     return !(waiting_.empty() && deferred_prefill_.empty() && prefill_.empty() && decode_.empty() &&
              deferred_decode_.empty());

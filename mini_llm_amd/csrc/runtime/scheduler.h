@@ -74,6 +74,10 @@ public:
     int on_token(int64_t id, bool is_eos);
     // Ends a request wherever it is; its pages are given back. 0 or -2.
     int abort(int64_t id);
+    // The request is complete as of a token sampled earlier (the caller saw the end of sequence
+    // only after the next step had been planned or run): it leaves the plan and the queues as
+    // finished, not failed, and its pages are given back. 0 or -2.
+    int stop(int64_t id);
 
     bool has_work() const;
     RequestState state(int64_t id) const;

@@ -5,6 +5,12 @@ portions under the token budget), the model runner runs it, the sampler chooses 
 for every request whose newest token was in the batch, finished requests give their
 pages back. The reference's loop: /root/reference/src/runtime/scheduler.cpp:322-356;
 its offline use of the model: /root/reference/benchmarks/gpt2/bench_batch_vs_single_wall.cu:157-171.
+
+Steps that hold only decoded tokens run one ahead of the host: a step is launched with its
+input tokens taken on the device from the step before, and only then are that earlier step's
+tokens read. The GPU so never waits for the host between decode steps. What the host learns
+late is only whether a token was the end of sequence; such a request has then run one step
+too many, whose token is dropped.
 """
 from __future__ import annotations
 
@@ -26,6 +32,7 @@ class EngineOptions:
     max_batch_num: int = 16             # sequences in one step (reference: MAX_BATCH_NUM, constants.h:20)
     max_tokens_per_step: int = 2048     # token budget of one step
     prefill_chunk: int = 512            # longest prompt portion
+    overlap_decode: bool = True         # launch a decode step before the previous one's tokens are read
 
 
 @dataclass
@@ -43,6 +50,8 @@ class _Request:
     params: SamplingParams
     finished: bool = False
     failed: Optional[str] = None
+    n_launched: int = 0                 # output tokens whose sampling has been launched
+    ended_early: bool = False           # an end-of-sequence token was read after later steps were planned
 
     @property
     def output(self) -> List[int]:
@@ -61,6 +70,7 @@ class Engine:
         self.eos_token_id = model.config.eos_token_id
         self.requests: Dict[int, _Request] = {}
         self._next_id = 0
+        self._pending = None            # (PendingTokens, [(request id, finished by that token)]) of the step in flight
 
     @classmethod
     def from_pretrained(cls, model_dir: str, dtype="bfloat16", device="cuda:0",
@@ -88,47 +98,94 @@ class Engine:
         r.finished, r.failed = True, "aborted"
 
     def has_unfinished(self) -> bool:
-        return self.scheduler.has_work()
+        return self.scheduler.has_work() or self._pending is not None
 
     # -- one iteration -------------------------------------------------------------------
+    def _is_eos(self, r: _Request, tok: int) -> bool:
+        return (not r.params.ignore_eos) and self.eos_token_id is not None and tok == self.eos_token_id
+
+    def _collect(self) -> List[RequestOutput]:
+        """Reads the tokens of the decode step in flight, if any. A request that an earlier token
+        already ended (seen late) or that was aborted drops its token."""
+        if self._pending is None:
+            return []
+        (handle, rows), self._pending = self._pending, None
+        outputs = []
+        for (rid, done), tok in zip(rows, handle.result()):
+            r = self.requests.get(rid)
+            if r is None or r.failed or r.ended_early:
+                continue
+            r.tokens.append(tok)
+            if not done and self._is_eos(r, tok):
+                # the scheduler has planned on without knowing: take the request out now
+                self.scheduler.stop(rid)
+                r.ended_early = done = True
+            r.finished = done
+            outputs.append(RequestOutput(rid, tok, done))
+        return outputs
+
     def step(self) -> List[RequestOutput]:
         plan = self.scheduler.schedule()
         outputs: List[RequestOutput] = []
         for rid, kind in self.scheduler.pop_events():
             if kind == "failed":
                 r = self.requests[rid]
+                if r.failed:                   # aborted by the caller, who knows
+                    continue
                 r.finished, r.failed = True, "the page pool cannot hold this request"
                 outputs.append(RequestOutput(rid, -1, True))
         if not plan:
-            return outputs
+            return outputs + self._collect()
         sampled = [e for e in plan if e.want_last]
+        fast = (self.runner.fast_decode and len(sampled) == len(plan) and all(e.n_tokens == 1 for e in plan))
+        if not (fast and self.options.overlap_decode):
+            # the host must know every token it feeds: read what is in flight first
+            outputs += self._collect()
+            live = [e for e in plan if not self.requests[e.request_id].finished]
+            if len(live) != len(plan):        # ended by a token just read; the scheduler dropped them too
+                plan, sampled = live, [e for e in live if e.want_last]
+                if not plan:
+                    return outputs
         temps, us = [], []
         for e in sampled:
             r = self.requests[e.request_id]
             temps.append(r.params.temperature)
-            us.append(uniform01(r.params.seed, len(r.tokens) - r.prompt_len) if r.params.temperature > 0 else 0.0)
-        if self.runner.use_graphs and len(sampled) == len(plan) and all(e.n_tokens == 1 for e in plan):
-            # every entry is one decoded token: the whole step replays as a HIP graph
-            tokens = self.runner.decode_step([e.request_id for e in plan],
-                                             [self.requests[e.request_id].tokens[e.start] for e in plan],
-                                             temps, us)
-            self.scheduler.commit()
-        else:
-            entries = []
+            us.append(uniform01(r.params.seed, r.n_launched) if r.params.temperature > 0 else 0.0)
+            r.n_launched += 1
+        if fast:
+            # every entry is one decoded token: the whole step runs from static buffers (a HIP graph)
+            in_flight = {rid: i for i, (rid, _) in enumerate(self._pending[1])} if self._pending else {}
+            toks, src = [], []
             for e in plan:
                 r = self.requests[e.request_id]
-                entries.append(StepEntry(e.request_id, r.tokens[e.start:e.start + e.n_tokens],
-                                         [e.n_tokens - 1] if e.want_last else []))
-            logits = self.runner.step(entries, manage_cache=False)
+                if e.start < len(r.tokens):
+                    toks.append(r.tokens[e.start])
+                    src.append(-1)
+                else:                          # sampled by the step in flight, not read yet
+                    toks.append(0)
+                    src.append(in_flight[e.request_id])
+            handle = self.runner.launch_decode([e.request_id for e in plan], toks, src, temps, us)
             self.scheduler.commit()
-            tokens = self.sampler.sample(logits, temps, us) if sampled else []
-        if sampled:
-            for e, tok in zip(sampled, tokens):
-                r = self.requests[e.request_id]
-                r.tokens.append(tok)
-                is_eos = (not r.params.ignore_eos) and self.eos_token_id is not None and tok == self.eos_token_id
-                r.finished = self.scheduler.on_token(e.request_id, is_eos)
-                outputs.append(RequestOutput(e.request_id, tok, r.finished))
+            # the scheduler moves on as if no token were the end of sequence; `_collect` corrects it
+            rows = [(e.request_id, self.scheduler.on_token(e.request_id, False)) for e in plan]
+            outputs += self._collect()
+            self._pending = (handle, rows)
+            if not self.options.overlap_decode:
+                outputs += self._collect()
+            return outputs
+        entries = []
+        for e in plan:
+            r = self.requests[e.request_id]
+            entries.append(StepEntry(e.request_id, r.tokens[e.start:e.start + e.n_tokens],
+                                     [e.n_tokens - 1] if e.want_last else []))
+        logits = self.runner.step(entries, manage_cache=False)
+        self.scheduler.commit()
+        tokens = self.sampler.sample(logits, temps, us) if sampled else []
+        for e, tok in zip(sampled, tokens):
+            r = self.requests[e.request_id]
+            r.tokens.append(tok)
+            r.finished = self.scheduler.on_token(e.request_id, self._is_eos(r, tok))
+            outputs.append(RequestOutput(e.request_id, tok, r.finished))
         return outputs
 
     # -- offline generation --------------------------------------------------------------

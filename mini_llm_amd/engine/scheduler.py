@@ -75,6 +75,11 @@ class Scheduler:
         if self._lib.mllm_sched_abort(self._h, rid) != 0:
             raise KeyError(f"request {rid} is unknown")
 
+    def stop(self, rid: int) -> None:
+        """The request ended with a token sampled earlier: finished (not failed), pages freed."""
+        if self._lib.mllm_sched_stop(self._h, rid) != 0:
+            raise KeyError(f"request {rid} is unknown")
+
     def has_work(self) -> bool:
         return bool(self._lib.mllm_sched_has_work(self._h))
 

@@ -114,7 +114,11 @@ class ModelRunner:
         self.n_pages = n_pages
         self._staging = _Staging(self.device)
         self._graphs: Dict[tuple, "DecodeGraph"] = {}
-        self.use_graphs = self.device.type == "cuda" and getattr(model, "graph_safe", True)
+        self._tok_out: Optional[torch.Tensor] = None      # sampled tokens of the last launched decode step
+        # Pure-decode batches may run from static buffers (`launch_decode`) unless a part of the model
+        # plans on the host; on the GPU those steps are captured and replayed as HIP graphs.
+        self.fast_decode = bool(getattr(model, "graph_safe", True))
+        self.use_graphs = self.device.type == "cuda" and self.fast_decode
 
     # -- cache bookkeeping for callers without a scheduler ---------------------------
     def ensure_request(self, rid: int) -> None:
@@ -225,26 +229,57 @@ class ModelRunner:
         return logits
 
     # -- decode steps through a captured HIP graph ------------------------------------------
-    def decode_step(self, request_ids: Sequence[int], tokens: Sequence[int],
-                    temperatures: Optional[Sequence[float]] = None,
-                    uniforms: Optional[Sequence[float]] = None) -> List[int]:
-        """One decoded token for each request (pages already reserved, lengths committed by the
-        caller afterwards): runs the model and the sampler as one HIP graph and returns the sampled
-        token of each request. The graph for a batch size is captured at its first use."""
+    def launch_decode(self, request_ids: Sequence[int], tokens: Sequence[int], src_rows: Sequence[int],
+                      temperatures: Optional[Sequence[float]] = None,
+                      uniforms: Optional[Sequence[float]] = None) -> "PendingTokens":
+        """Starts one decode step for the given requests (pages already reserved; the caller commits
+        the lengths) and returns at once. Row i's input token is ``tokens[i]``, or, where
+        ``src_rows[i] >= 0``, the token that the previous launch sampled in that row (the host need
+        not have read it). The model and the sampler run from static buffers, on the GPU as one HIP
+        graph captured at a batch size's first use. ``PendingTokens.result()`` waits for the
+        sampled tokens."""
         B = len(request_ids)
         greedy = temperatures is None or all(t <= 0 for t in temperatures)
         bucket = B if B <= 8 else -(-B // 8) * 8
+        if self._tok_out is None or self._tok_out.numel() < bucket:
+            if self._graphs:
+                # captured graphs hold the old buffer's address
+                self._graphs.clear()
+            n = max(bucket, -(-self.manager.n_state_slots // 8) * 8, 8)
+            self._tok_out = torch.zeros(n, dtype=torch.int32, device=self.device)
         key = (bucket, greedy)
         g = self._graphs.get(key)
         if g is None:
             g = self._graphs[key] = DecodeGraph(self, bucket, greedy)
-        return g.run(request_ids, tokens, temperatures, uniforms)
+        return g.launch(request_ids, tokens, src_rows, temperatures, uniforms)
+
+    def decode_step(self, request_ids: Sequence[int], tokens: Sequence[int],
+                    temperatures: Optional[Sequence[float]] = None,
+                    uniforms: Optional[Sequence[float]] = None) -> List[int]:
+        """One decoded token for each request, waited for: ``launch_decode`` with every input token
+        known to the host."""
+        return self.launch_decode(request_ids, tokens, [-1] * len(request_ids), temperatures, uniforms).result()
+
+
+class PendingTokens:
+    """The sampled tokens of a launched decode step; ``result()`` waits until they have reached
+    the host."""
+
+    def __init__(self, host: torch.Tensor, n: int, event):
+        self._host, self._n, self._event = host, n, event
+
+    def result(self) -> List[int]:
+        if self._event is not None:
+            self._event.synchronize()
+        return self._host[:self._n].tolist()
 
 
 class DecodeGraph:
-    """A decode step of fixed batch size captured as a HIP graph: embedding, every layer, the
-    head and the sampler replay from static buffers; per step the host only refreshes the index
-    arrays (one copy) and reads the sampled tokens back.
+    """A decode step of fixed batch size on static buffers: embedding, every layer, the head and
+    the sampler; on the GPU captured once and replayed as a HIP graph. Per step the host only
+    refreshes the index arrays (one copy) and later reads the sampled tokens, which every graph
+    of a runner leaves in the same device buffer, so that the next step can take its input
+    tokens from there before the host has seen them.
 
     Rows beyond the live batch repeat row 0 without writing to the cache, so one graph serves
     every batch size up to its own.
@@ -255,37 +290,44 @@ class DecodeGraph:
         self.runner, self.batch, self.greedy = runner, batch, greedy
         model, cache = runner.model, runner.cache
         dev = runner.device
+        on_gpu = dev.type == "cuda"
         max_pos = model.max_positions
         cap_blocks = runner.n_pages if max_pos is None else min(runner.n_pages, -(-max_pos // runner.page_size))
         self.max_blocks = [max(1, cap_blocks)] * cache.n_groups
         B = batch
         self.offs = _layout(B, B, B, self.max_blocks)
-        self.n_ints = self.offs[-1]
+        self.n_ctx_ints = self.offs[-1]
+        self.n_ints = self.n_ctx_ints + B                  # then: the row of the last launch each token comes from
         self.dev_ints = torch.zeros(self.n_ints, dtype=torch.int32, device=dev)
+        self.src_rows = self.dev_ints[self.n_ctx_ints:]
         self.ctx = runner._context(self.dev_ints, self.offs, B, B, B, self.max_blocks, 1,
                                    self.max_blocks[0] * runner.page_size if self.max_blocks else 1)
-        self.h_float = torch.zeros((2, B), dtype=torch.float32, pin_memory=True)
+        self.h_float = torch.zeros((2, B), dtype=torch.float32, pin_memory=on_gpu)
         self.d_float = torch.zeros((2, B), dtype=torch.float32, device=dev)
-        self.out = torch.zeros(B, dtype=torch.int32, device=dev)
-        self.h_out = torch.zeros(B, dtype=torch.int32, pin_memory=True)
-        self.graph: Optional[torch.cuda.CUDAGraph] = None
+        self.out = runner._tok_out[:B]
+        # two host buffers in turn: one may still be unread when the next step's copy is queued
+        self.h_out = [torch.zeros(B, dtype=torch.int32, pin_memory=on_gpu) for _ in range(2)]
+        self._turn = 0
+        self.capture = runner.use_graphs
+        self.graph: Optional["torch.cuda.CUDAGraph"] = None
         self._ops = ops
 
     def _forward(self) -> None:
+        self._ops.select_tokens(self.ctx.token_ids, self.src_rows, self.runner._tok_out)
         logits = self.runner.model.forward(self.ctx, self.runner.cache)
         if self.greedy:
             self._ops.argmax(logits, self.out)
         else:
             self._ops.sample(logits, self.d_float[0], self.d_float[1], self.out)
 
-    def _fill(self, request_ids, tokens) -> None:
+    def _fill(self, request_ids, tokens, src_rows) -> None:
         r, B, n = self.runner, self.batch, len(request_ids)
         ids = np.empty(B, dtype=np.int64)
         ids[:n] = request_ids
         ids[n:] = request_ids[0]
         n_tok = np.ones(B, dtype=np.int32)
         host, buf = r._staging.take(self.n_ints)
-        seg = r._fill(host, self.offs, ids, n_tok, self.max_blocks)
+        seg = r._fill(host[:self.n_ctx_ints], self.offs, ids, n_tok, self.max_blocks)
         tok = seg[0]
         tok[:n] = tokens
         tok[n:] = tokens[0]
@@ -294,27 +336,41 @@ class DecodeGraph:
         seg[7][:] = np.arange(B, dtype=np.int32)
         for g in range(len(self.max_blocks)):
             seg[9 + 2 * g][n:] = -1              # padding rows write nothing to the cache
+        src = host[self.n_ctx_ints:self.n_ints]
+        src[:n] = src_rows
+        src[n:] = src_rows[0]
         self.h_cu_q, self.h_starts, self.h_state_slots = seg[3], seg[5], seg[6]
         _Staging.upload(buf, self.n_ints, self.dev_ints)
 
-    def run(self, request_ids, tokens, temperatures, uniforms) -> List[int]:
+    def launch(self, request_ids, tokens, src_rows, temperatures, uniforms) -> PendingTokens:
         n = len(request_ids)
-        self._fill(request_ids, tokens)
+        self._fill(request_ids, tokens, src_rows)
         if not self.greedy:
             h = self.h_float.numpy()
             h[0, :n] = temperatures
             h[1, :n] = uniforms
             h[0, n:] = 0.0
             self.d_float.copy_(self.h_float, non_blocking=True)
-        if self.graph is None:
-            # First use: run once eagerly (loads the kernels, sizes their scratch), then capture.
-            # Running the same step twice is harmless: it writes the same keys and values.
+        if not self.capture:
             self._forward()
-            torch.cuda.synchronize()
-            self.graph = torch.cuda.CUDAGraph()
-            with torch.cuda.graph(self.graph):
+        else:
+            if self.graph is None:
+                # First use: run once eagerly (loads the kernels, sizes their scratch), then capture.
+                # The eager run's effects are the step's own (same keys and values written, same
+                # tokens sampled); the fed-back tokens are set aside, since it overwrites them.
+                fed = self.runner._tok_out.clone()
                 self._forward()
-        self.graph.replay()
-        self.h_out.copy_(self.out, non_blocking=True)
-        torch.cuda.current_stream().synchronize()
-        return self.h_out[:n].tolist()
+                torch.cuda.synchronize()
+                self.runner._tok_out.copy_(fed)
+                self.graph = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(self.graph):
+                    self._forward()
+            self.graph.replay()
+        self._turn ^= 1
+        host = self.h_out[self._turn]
+        host.copy_(self.out, non_blocking=True)
+        event = None
+        if self.capture:
+            event = torch.cuda.Event()
+            event.record()
+        return PendingTokens(host, n, event)

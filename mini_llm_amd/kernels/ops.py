@@ -95,6 +95,19 @@ def embed(ids: torch.Tensor, positions: Optional[torch.Tensor], wte: torch.Tenso
     return out
 
 
+def select_tokens(ids: torch.Tensor, src: torch.Tensor, prev: torch.Tensor) -> torch.Tensor:
+    """ids[i] = prev[src[i]] where src[i] >= 0, in place: token ids that an earlier step sampled
+    on the device and the host has not read yet."""
+    _gpu(ids, src, prev)
+    n = ids.numel()
+    _i32(ids, "ids")
+    _i32(src, "src", n)
+    _i32(prev, "prev")
+    lib = load_library("elementwise")
+    _check(lib.mllm_select_tokens(_p(ids), _p(src), _p(prev), n, prev.numel(), _stream()), "select_tokens")
+    return ids
+
+
 def layernorm(x: torch.Tensor, gamma: torch.Tensor, beta: Optional[torch.Tensor], eps: float,
               out: torch.Tensor, rows: Optional[torch.Tensor] = None) -> torch.Tensor:
     """out[i,:] = LayerNorm(x[rows[i] if rows else i,:]); statistics in fp32."""

@@ -23,6 +23,13 @@ def embed(ids, positions, wte, wpe, out):
     return out
 
 
+def select_tokens(ids, src, prev):
+    for i in range(ids.numel()):
+        if int(src[i]) >= 0:
+            ids[i] = prev[int(src[i])]
+    return ids
+
+
 def layernorm(x, gamma, beta, eps, out, rows=None):
     src = x if rows is None else x[rows.long()]
     s = src.to(PRECISE)
@@ -118,7 +125,7 @@ def sample(logits, temperature, u, out):
     return out
 
 
-_NAMES = ("embed", "layernorm", "linear", "ln_linear", "kv_append", "paged_attention", "argmax", "sample")
+_NAMES = ("embed", "select_tokens", "layernorm", "linear", "ln_linear", "kv_append", "paged_attention", "argmax", "sample")
 
 
 def install(monkeypatch):

@@ -75,23 +75,31 @@ def test_temperature_sampling_does_not_depend_on_batching(tiny_model_dirs, dtype
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_graph_decode_matches_eager_steps(tiny_model_dirs, dtype):
-    """Decode steps replay as HIP graphs (padded to a bucket of 16 for 11 requests); the tokens
-    equal those of the same engine stepping eagerly, replay after replay."""
+    """Decode steps replay as HIP graphs (padded to a bucket of 16 for 11 requests), each launched
+    before the previous one's tokens are read; the tokens equal those of the same engine waiting
+    for every step, running the static buffers without a graph, and stepping through the general
+    step function, replay after replay."""
     from mini_llm_amd import Engine, EngineOptions, SamplingParams
     prompts = _prompts("a", (3, 5, 8, 13, 21, 34, 4, 9, 16, 25, 1), 7)
     params = [SamplingParams(temperature=0.0 if i % 2 else 0.7, seed=i, max_new_tokens=20, ignore_eos=True)
               for i in range(len(prompts))]
     outs = {}
-    for graphs in (True, False):
+    for mode in ("graph", "graph, waited for", "static buffers", "general steps"):
         e = Engine.from_pretrained(tiny_model_dirs["a"], dtype=dtype,
-                                   options=EngineOptions(kv_block_size=4, total_kv_blocks=256, max_batch_num=16))
-        assert e.runner.use_graphs
-        e.runner.use_graphs = graphs
-        outs[graphs] = e.generate(prompts, params)
-        assert (len(e.runner._graphs) > 0) == graphs
-        assert e.stats()["free_pages"] == 256
-    assert outs[True] == outs[False]
-    assert all(len(o) == 20 for o in outs[True])
+                                   options=EngineOptions(kv_block_size=4, total_kv_blocks=256, max_batch_num=16,
+                                                         overlap_decode=(mode != "graph, waited for")))
+        assert e.runner.use_graphs and e.runner.fast_decode
+        if mode == "static buffers":
+            e.runner.use_graphs = False
+        if mode == "general steps":
+            e.runner.fast_decode = False
+        outs[mode] = e.generate(prompts, params)
+        graphs = list(e.runner._graphs.values())
+        assert (len(graphs) > 0) == (mode != "general steps")
+        assert all((g.graph is not None) == mode.startswith("graph") for g in graphs)
+        assert e.stats()["free_pages"] == 256 and not e.has_unfinished()
+    assert all(o == outs["graph"] for o in outs.values())
+    assert all(len(o) == 20 for o in outs["graph"])
 
 
 def test_command_line(tiny_model_dirs, tmp_path):

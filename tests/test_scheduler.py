@@ -215,3 +215,67 @@ def test_greedy_generation_matches_plain_and_stops_at_eos(cpu_ops, tiny_model_di
     e2.eos_token_id = outs[0][0]
     assert e2.generate([prompts[0]], SamplingParams(max_new_tokens=16)) == [[outs[0][0]]]
     assert e2.generate([prompts[0]], SamplingParams(max_new_tokens=3, ignore_eos=True)) == [outs[0][:3]]
+
+
+def test_overlapped_decode_gives_the_same_tokens(cpu_ops, tiny_model_dirs):
+    """Decode steps launched before the previous step's tokens are read (tokens fed on the
+    device) produce what step-by-step decoding produces, also when pages run out on the way."""
+    from mini_llm_amd import SamplingParams
+    g = torch.Generator().manual_seed(11)
+    prompts = [torch.randint(0, 1000, (n,), generator=g).tolist() for n in (3, 20, 41, 64)]
+    params = [SamplingParams(temperature=0.7 if i % 2 else 0.0, seed=10 + i, max_new_tokens=12 + 5 * i,
+                             ignore_eos=True) for i in range(4)]
+    for pages in (64, 24):
+        outs = []
+        for overlap in (False, True):
+            e = _engine(tiny_model_dirs["b"], kv_block_size=8, total_kv_blocks=pages, max_batch_num=4,
+                        max_tokens_per_step=32, prefill_chunk=16, overlap_decode=overlap)
+            outs.append(e.generate(prompts, params))
+            assert e.stats()["free_pages"] == pages and e.runner.manager.check() == ""
+        assert outs[0] == outs[1]
+        assert [len(o) for o in outs[0]] == [12, 17, 22, 27]
+
+
+def test_end_of_sequence_seen_one_step_late(cpu_ops, tiny_model_dirs):
+    """A decoded token that is the end of sequence is read only after the next step has been
+    launched: the request still ends with that token, the extra step's token is dropped and every
+    page comes back, while the other requests go on undisturbed."""
+    from mini_llm_amd import SamplingParams
+    g = torch.Generator().manual_seed(5)
+    prompts = [torch.randint(0, 511, (n,), generator=g).tolist() for n in (7, 19, 30)]
+    free = _engine(tiny_model_dirs["a"], kv_block_size=4, total_kv_blocks=60, max_batch_num=4)
+    sp = [SamplingParams(temperature=1.5, seed=3 + i, max_new_tokens=14, ignore_eos=True) for i in range(3)]
+    full = free.generate(prompts, sp)
+    # a token that request 0 decodes (not its first, which the prompt step samples), where it first occurs
+    j = next(j for j in range(2, 14) if full[0][j] not in full[0][:j])
+    eos = full[0][j]
+    expect = [o[:o.index(eos) + 1] if eos in o else o for o in full]
+    assert len(expect[0]) == j + 1
+    for overlap in (True, False):
+        e = _engine(tiny_model_dirs["a"], kv_block_size=4, total_kv_blocks=60, max_batch_num=4,
+                    overlap_decode=overlap)
+        e.eos_token_id = eos
+        stop = [SamplingParams(temperature=1.5, seed=3 + i, max_new_tokens=14) for i in range(3)]
+        assert e.generate(prompts, stop) == expect
+        assert e.stats()["free_pages"] == 60 and e.runner.manager.check() == ""
+        assert not e.has_unfinished()
+
+
+def test_outputs_of_steps_arrive_in_order_and_abort_in_flight(cpu_ops, tiny_model_dirs):
+    from mini_llm_amd import SamplingParams
+    e = _engine(tiny_model_dirs["a"], kv_block_size=4, total_kv_blocks=60, max_batch_num=4)
+    a = e.add_request([5, 6, 7, 8], SamplingParams(max_new_tokens=6, ignore_eos=True))
+    b = e.add_request([9, 10, 11], SamplingParams(max_new_tokens=9, ignore_eos=True))
+    seen = {a: [], b: []}
+    steps = 0
+    while e.has_unfinished():
+        for out in e.step():
+            seen[out.request_id].append((out.token, out.finished))
+        steps += 1
+        if steps == 4:
+            e.abort(b)               # b has a token in flight; it is dropped
+    assert [t for t, _ in seen[a]] == e.requests[a].output and len(seen[a]) == 6
+    assert [f for _, f in seen[a]] == [False] * 5 + [True]
+    assert e.requests[b].failed == "aborted" and len(seen[b]) < 9
+    assert [t for t, _ in seen[b]] == e.requests[b].output
+    assert e.stats()["free_pages"] == 60 and e.runner.manager.check() == ""
