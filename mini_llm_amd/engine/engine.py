@@ -79,6 +79,34 @@ class Engine:
             options = EngineOptions(**{**(options.__dict__ if options else {}), **kw})
         return cls(load_model(model_dir, dtype, device), options)
 
+    @classmethod
+    def from_random(cls, preset: Union[str, dict], seed: int = 0, dtype="bfloat16", device="cuda:0",
+                    options: Optional[EngineOptions] = None, **kw) -> "Engine":
+        """An engine over random weights: ``preset`` names a size under config/presets (or is a
+        config.json dictionary); the model folder is written to a temporary place and loaded as
+        any other."""
+        import json
+        import os
+        import tempfile
+        from ..weights.random_init import write_random_model
+        if isinstance(preset, str):
+            d = os.path.join(os.path.dirname(os.path.abspath(__file__)), "..", "config", "presets")
+            path = os.path.join(d, preset + ".json")
+            if not os.path.isfile(path):
+                names = sorted(f[:-5] for f in os.listdir(d) if f.endswith(".json"))
+                raise ValueError(f"unknown preset '{preset}'; known: {names}")
+            with open(path) as f:
+                preset = json.load(f)
+        with tempfile.TemporaryDirectory() as tmp:
+            write_random_model(dict(preset), tmp, seed, "float32" if dtype == "float32" else "bfloat16")
+            return cls.from_pretrained(tmp, dtype=dtype, device=device, options=options, **kw)
+
+    def step_logits(self, entries: Sequence[StepEntry]) -> Optional[torch.Tensor]:
+        """The step function itself, for callers that bring their own tokens (tests, replay):
+        runs the entries through the model and the cache and returns fp32 logits at the wanted
+        places. Requests stepped this way are not known to the scheduler."""
+        return self.runner.step(entries, manage_cache=True)
+
     # -- requests ------------------------------------------------------------------------
     def add_request(self, prompt_ids: Sequence[int], params: Optional[SamplingParams] = None,
                     request_id: Optional[int] = None) -> int:

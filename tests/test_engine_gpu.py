@@ -128,3 +128,34 @@ def test_command_line(tiny_model_dirs, tmp_path):
     assert r.returncode == 0, r.stderr
     s = r.stdout.strip().splitlines()
     assert len(s) == 3 and s[-1].endswith("[DONE]") and all(l.startswith("0 ") for l in s)
+
+
+def test_random_preset_entry_points(tmp_path):
+    """`--preset` on the command line and `Engine.from_random` generate with the same random
+    weights as a folder written by `make-model` with that seed; `step_logits` is the step function."""
+    from mini_llm_amd import Engine, EngineOptions, SamplingParams
+    from mini_llm_amd.engine.step import StepEntry
+    cli = os.path.join(ROOT, "bin", "mini-llm")
+    made = str(tmp_path / "made")
+    mk = subprocess.run([sys.executable, cli, "make-model", "--preset", "tiny-b", "--seed", "5", "--out", made],
+                        capture_output=True, text=True, timeout=120)
+    assert mk.returncode == 0, mk.stderr
+    common = ["--prompt-ids", "4 5 6 7", "--max-new-tokens", "5", "--ignore-eos", "--kv-block-size", "8",
+              "--total-kv-blocks", "16", "--max-batch-num", "2"]
+    a = subprocess.run([sys.executable, cli, "generate", "--model", made] + common,
+                       capture_output=True, text=True, timeout=300)
+    b = subprocess.run([sys.executable, cli, "generate", "--preset", "tiny-b", "--weights-seed", "5"] + common,
+                       capture_output=True, text=True, timeout=300)
+    assert a.returncode == 0 and b.returncode == 0, (a.stderr, b.stderr)
+    assert a.stdout == b.stdout and a.stdout.strip().endswith("[DONE]")
+    e = Engine.from_random("tiny-b", 5, options=EngineOptions(kv_block_size=8, total_kv_blocks=16, max_batch_num=2))
+    out = e.generate([[4, 5, 6, 7]], SamplingParams(max_new_tokens=5, ignore_eos=True))[0]
+    assert " ".join(map(str, out)) + " [DONE]" == a.stdout.strip()
+    logits = e.step_logits([StepEntry(77, [4, 5, 6, 7], [3])])
+    assert logits.shape == (1, e.model.vocab_size) and int(logits[0].argmax()) == out[0]
+    e.runner.end_request(77)
+    with pytest.raises(ValueError, match="unknown preset"):
+        Engine.from_random("no-such-size")
+    bad = subprocess.run([sys.executable, cli, "generate", "--preset", "no-such-size", "--prompt-ids", "1"],
+                         capture_output=True, text=True, timeout=120)
+    assert bad.returncode == 1 and "unknown preset" in bad.stderr
