@@ -25,6 +25,17 @@ typedef float f32x16 __attribute__((ext_vector_type(16)));
 // accumulator registers hold 4 consecutive columns of one output row: the epilogue stores them
 // as one 8- or 16-byte access.
 // ---------------------------------------------------------------------------------------------
+// Optional second destination of a plain bf16 store: columns [q_cols, q_cols + kv_dim) of output row
+// m also go to row slots[m] of the key pages and the next kv_dim columns to the value pages (the
+// fused QKV product writes a step's keys and values where attention reads them;
+// /root/reference/src/kernels/prefill/append_kv.cu:28-46 is a kernel of its own). slots == nullptr: off.
+struct KvScatter {
+    const int* slots;
+    bf16_t* k_pages;
+    bf16_t* v_pages;
+    int q_cols, kv_dim;
+};
+
 template <int MODE>
 __device__ __forceinline__ void store4(void* C, size_t idx, const float (&v)[4], bool vec, int n_left) {
     // v: 4 consecutive columns of one row, bias already added; n_left: columns that exist (1..4)
@@ -61,7 +72,7 @@ template <int WM, int WN, int TM, int TN, int BKP, int DEPTH, bool EDGE, int MOD
 __global__ void __launch_bounds__(WM * WN * 64)
 gemm_bf16_mfma(const bf16_t* __restrict__ A, int lda, const bf16_t* __restrict__ W, int ldw,
                const float* __restrict__ bias, void* __restrict__ C, int ldc, int M, int N, int K,
-               int tiles_m, int tiles_n, int xm, int xn) {
+               int tiles_m, int tiles_n, int xm, int xn, KvScatter kv) {
     constexpr int NT = WM * WN * 64;
     constexpr int BM = WM * TM * 32, BN = WN * TN * 32;
     constexpr int STRIDE = BKP + 8;
@@ -207,6 +218,7 @@ gemm_bf16_mfma(const bf16_t* __restrict__ A, int lda, const bf16_t* __restrict__
     for (int i = 0; i < TM; ++i) {
         const int m = m0 + (wm * TM + i) * 32 + lane % 32;
         if (EDGE && m >= M) continue;
+        const int slot = (MODE == EPI_STORE && kv.slots != nullptr) ? kv.slots[m] : -1;
 #pragma unroll
         for (int j = 0; j < TN; ++j) {
 #pragma unroll
@@ -218,6 +230,20 @@ gemm_bf16_mfma(const bf16_t* __restrict__ A, int lda, const bf16_t* __restrict__
 #pragma unroll
                 for (int e = 0; e < 4; ++e) v[e] = acc[i][j][4 * g + e] + ((bias && e < n_left) ? bias[n + e] : 0.f);
                 store4<MODE>(C, static_cast<size_t>(m) * ldc + n, v, vec, n_left);
+                if (MODE == EPI_STORE && slot >= 0 && n >= kv.q_cols) {
+                    // q_cols and kv_dim are multiples of 4: the four columns lie in one of the two parts
+                    const int c = n - kv.q_cols;
+                    bf16_t* dst = (c < kv.kv_dim ? kv.k_pages + c : kv.v_pages + (c - kv.kv_dim)) +
+                                  static_cast<size_t>(slot) * kv.kv_dim;
+                    if (n_left >= 4) {
+                        uint2 pk;
+                        pk.x = pack_bf16x2(v[0], v[1]);
+                        pk.y = pack_bf16x2(v[2], v[3]);
+                        *reinterpret_cast<uint2*>(dst) = pk;
+                    } else {
+                        for (int e = 0; e < n_left; ++e) dst[e] = float_to_bf16(v[e]);
+                    }
+                }
             }
         }
     }
@@ -225,7 +251,7 @@ gemm_bf16_mfma(const bf16_t* __restrict__ A, int lda, const bf16_t* __restrict__
 
 template <int WM, int WN, int TM, int TN, int BKP, int DEPTH>
 static void launch_tiled(const bf16_t* a, int lda, const bf16_t* w, int ldw, const float* bias, void* C, int ldc,
-                         int M, int N, int K, int mode, hipStream_t stream) {
+                         int M, int N, int K, int mode, hipStream_t stream, KvScatter kv = KvScatter{}) {
     constexpr int BM = WM * TM * 32, BN = WN * TN * 32;
     const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
     // split of the output among the XCDs (xm x xn = 8) that keeps the A rows plus W rows of one XCD smallest
@@ -239,7 +265,7 @@ static void launch_tiled(const bf16_t* a, int lda, const bf16_t* w, int ldw, con
     const int per_xcd = ((tiles_m + xm - 1) / xm) * ((tiles_n + xn - 1) / xn);
     const dim3 grid(per_xcd * N_XCD), block(WM * WN * 64);
     const bool edge = !(M % BM == 0 && N % BN == 0 && K % BKP == 0);
-#define TILED(E, MD) gemm_bf16_mfma<WM, WN, TM, TN, BKP, DEPTH, E, MD><<<grid, block, 0, stream>>>(a, lda, w, ldw, bias, C, ldc, M, N, K, tiles_m, tiles_n, xm, xn)
+#define TILED(E, MD) gemm_bf16_mfma<WM, WN, TM, TN, BKP, DEPTH, E, MD><<<grid, block, 0, stream>>>(a, lda, w, ldw, bias, C, ldc, M, N, K, tiles_m, tiles_n, xm, xn, kv)
 #define TILED_MODE(MD) case MD: if (edge) TILED(true, MD); else TILED(false, MD); break;
     switch (mode) {
         TILED_MODE(EPI_STORE) TILED_MODE(EPI_GELU_TANH) TILED_MODE(EPI_GELU_ERF) TILED_MODE(EPI_ADD_RESIDUAL)
@@ -630,23 +656,19 @@ static int launch_skinny(const void* A, int lda, const bf16_t* W, int ldw, const
 }
 
 
-extern "C" {
-
-
-// Returns 0, a HIP error code, or -1 when K or the row strides are not multiples of 8
-// elements or a base pointer is not 16-byte aligned.
-int mllm_gemm_bf16(const void* A, int lda, const void* W, int ldw, const float* bias, void* C, int ldc,
-                   int M, int N, int K, int mode, hipStream_t stream) {
+static int gemm_bf16_dispatch(const void* A, int lda, const void* W, int ldw, const float* bias, void* C, int ldc,
+                              int M, int N, int K, int mode, hipStream_t stream, KvScatter kv) {
     if (M <= 0 || N <= 0) return 0;
     if (K % 8 != 0 || lda % 8 != 0 || ldw % 8 != 0) return -1;
     if ((reinterpret_cast<uintptr_t>(A) & 15) || (reinterpret_cast<uintptr_t>(W) & 15)) return -1;
     const bf16_t* a = static_cast<const bf16_t*>(A);
     const bf16_t* w = static_cast<const bf16_t*>(W);
-    if (M <= 64 && launch_skinny<false>(A, lda, w, ldw, bias, C, ldc, M, N, K, mode, nullptr, nullptr, 0.f,
-                                        nullptr, stream) == 0) {
+    const bool scatter = kv.slots != nullptr;       // only the many-row kernel scatters
+    if (!scatter && M <= 64 && launch_skinny<false>(A, lda, w, ldw, bias, C, ldc, M, N, K, mode, nullptr, nullptr,
+                                                    0.f, nullptr, stream) == 0) {
         // few rows: weight-streaming kernel
     } else if (M <= 32) {
-        launch_tiled<1, 4, 1, 1, 64, 3>(a, lda, w, ldw, bias, C, ldc, M, N, K, mode, stream);
+        launch_tiled<1, 4, 1, 1, 64, 3>(a, lda, w, ldw, bias, C, ldc, M, N, K, mode, stream, kv);
     } else {
         // Tile choice, measured at 2048 rows on GPT-2 shapes: a large tile moves fewer bytes per
         // flop, but pays only when its workgroups fill the 256 compute units in one round (or in
@@ -654,17 +676,40 @@ int mllm_gemm_bf16(const void* A, int lda, const void* W, int ldw, const float* 
         auto blocks = [&](int bm, int bn) { return static_cast<long>((M + bm - 1) / bm) * ((N + bn - 1) / bn); };
         auto one_round = [](long n) { return n >= 192 && n <= 256; };
         if (one_round(blocks(128, 192))) {
-            launch_tiled<4, 2, 1, 3, 32, 4>(a, lda, w, ldw, bias, C, ldc, M, N, K, mode, stream);     // 128x192
+            launch_tiled<4, 2, 1, 3, 32, 4>(a, lda, w, ldw, bias, C, ldc, M, N, K, mode, stream, kv);     // 128x192
         } else if (blocks(128, 128) >= 512 || one_round(blocks(128, 128))) {
-            launch_tiled<2, 2, 2, 2, 32, 6>(a, lda, w, ldw, bias, C, ldc, M, N, K, mode, stream);     // 128x128
+            launch_tiled<2, 2, 2, 2, 32, 6>(a, lda, w, ldw, bias, C, ldc, M, N, K, mode, stream, kv);     // 128x128
         } else if (one_round(blocks(64, 96))) {
-            launch_tiled<2, 3, 1, 1, 64, 3>(a, lda, w, ldw, bias, C, ldc, M, N, K, mode, stream);     // 64x96
+            launch_tiled<2, 3, 1, 1, 64, 3>(a, lda, w, ldw, bias, C, ldc, M, N, K, mode, stream, kv);     // 64x96
         } else {
-            launch_tiled<2, 2, 1, 1, 64, 4>(a, lda, w, ldw, bias, C, ldc, M, N, K, mode, stream);     // 64x64
+            launch_tiled<2, 2, 1, 1, 64, 4>(a, lda, w, ldw, bias, C, ldc, M, N, K, mode, stream, kv);     // 64x64
         }
     }
     MLLM_LAUNCH_CHECK();
     return 0;
+}
+
+extern "C" {
+
+// Returns 0, a HIP error code, or -1 when K or the row strides are not multiples of 8
+// elements or a base pointer is not 16-byte aligned.
+int mllm_gemm_bf16(const void* A, int lda, const void* W, int ldw, const float* bias, void* C, int ldc,
+                   int M, int N, int K, int mode, hipStream_t stream) {
+    return gemm_bf16_dispatch(A, lda, W, ldw, bias, C, ldc, M, N, K, mode, stream, KvScatter{});
+}
+
+// The plain bf16 store (mode 0) with the key/value scatter of KvScatter fused: C = A W^T + bias, and
+// columns [q_cols, q_cols + kv_dim) / [q_cols + kv_dim, q_cols + 2 kv_dim) of row m also go to row
+// slots[m] (>= 0) of k_pages / v_pages ([rows, kv_dim] bf16). q_cols and kv_dim must be multiples
+// of 4 and N == q_cols + 2 kv_dim; -1 otherwise or as mllm_gemm_bf16.
+int mllm_gemm_bf16_kv(const void* A, int lda, const void* W, int ldw, const float* bias, void* C, int ldc,
+                      int M, int N, int K, const int* slots, void* k_pages, void* v_pages, int q_cols, int kv_dim,
+                      hipStream_t stream) {
+    if (slots == nullptr || q_cols < 0 || kv_dim <= 0 || q_cols % 4 != 0 || kv_dim % 4 != 0 ||
+        N != q_cols + 2 * kv_dim)
+        return -1;
+    KvScatter kv{slots, static_cast<bf16_t*>(k_pages), static_cast<bf16_t*>(v_pages), q_cols, kv_dim};
+    return gemm_bf16_dispatch(A, lda, W, ldw, bias, C, ldc, M, N, K, EPI_STORE, stream, kv);
 }
 
 // LayerNorm of the fp32 rows x[M,K] (row m taken from x[rows[m]] when `rows` is given) fused into the

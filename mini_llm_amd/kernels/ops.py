@@ -130,12 +130,22 @@ def layernorm(x: torch.Tensor, gamma: torch.Tensor, beta: Optional[torch.Tensor]
     return out
 
 
+def linear_scatters_kv(dtype: torch.dtype, rows: int) -> bool:
+    """Whether ``linear(..., kv_scatter=...)`` can write a fused QKV product's keys and values
+    to the pages itself: the many-row bf16 kernel does."""
+    return dtype == torch.bfloat16 and rows > 64
+
+
 def linear(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], out: torch.Tensor,
-           epilogue: str = "store") -> torch.Tensor:
+           epilogue: str = "store", kv_scatter: Optional[tuple] = None) -> torch.Tensor:
     """out = epilogue(a @ w.T + bias). a: [M,K], w: [N,K] (same dtype), bias: fp32 [N].
 
     epilogue: "store" | "gelu_tanh" | "gelu_erf" (out in a's dtype), "add_residual"
     (out fp32, accumulated in place), "store_f32" (out fp32).
+
+    ``kv_scatter=(slots, k_pages, v_pages, q_cols)`` (only with "store" and where
+    ``linear_scatters_kv`` says so): the columns after the first q_cols are keys, then values, of
+    kv_dim = k_pages.shape[1] columns each, and row m's also go to row slots[m] (>= 0) of the pages.
     """
     _gpu(a, w, bias, out)
     _rows2d(a, "a")
@@ -153,14 +163,32 @@ def linear(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], out: 
     if bias is not None and (bias.dtype != torch.float32 or bias.numel() != N or not bias.is_contiguous()):
         raise KernelError(f"bias must be contiguous fp32 [{N}]")
     mode = EPILOGUES[epilogue]
+    if kv_scatter is not None and a.dtype != torch.bfloat16:
+        raise KernelError("linear: the key/value scatter exists for bfloat16 only")
     if a.dtype == torch.float32:
         lib = load_library("gemm_f32")
         rc = lib.mllm_gemm_f32(_p(a), a.stride(0), _p(w), w.stride(0), _p(bias), _p(out), out.stride(0),
                                M, N, K, mode, _stream())
     elif a.dtype == torch.bfloat16:
         lib = load_library("gemm_bf16")
-        rc = lib.mllm_gemm_bf16(_p(a), a.stride(0), _p(w), w.stride(0), _p(bias), _p(out), out.stride(0),
-                                M, N, K, mode, _stream())
+        if kv_scatter is not None:
+            slots, k_pages, v_pages, q_cols = kv_scatter
+            _gpu(slots, k_pages, v_pages)
+            kv_dim = k_pages.shape[1]
+            if epilogue != "store" or not linear_scatters_kv(a.dtype, M):
+                raise KernelError("linear: the key/value scatter needs the plain store and more than 64 bf16 rows")
+            _i32(slots, "slots", M)
+            for name, pg in (("k_pages", k_pages), ("v_pages", v_pages)):
+                if pg.dim() != 2 or pg.shape[1] != kv_dim or not pg.is_contiguous() or pg.dtype != a.dtype:
+                    raise KernelError(f"{name} must be contiguous [rows, {kv_dim}] {a.dtype}")
+            if q_cols % 4 or kv_dim % 4 or N != q_cols + 2 * kv_dim:
+                raise KernelError(f"linear: {N} columns are not {q_cols} + 2 x {kv_dim} (multiples of 4)")
+            rc = lib.mllm_gemm_bf16_kv(_p(a), a.stride(0), _p(w), w.stride(0), _p(bias), _p(out), out.stride(0),
+                                       M, N, K, _p(slots), _p(k_pages), _p(v_pages), int(q_cols), int(kv_dim),
+                                       _stream())
+        else:
+            rc = lib.mllm_gemm_bf16(_p(a), a.stride(0), _p(w), w.stride(0), _p(bias), _p(out), out.stride(0),
+                                    M, N, K, mode, _stream())
         if rc == -1:
             raise KernelError(
                 f"linear(bf16): K={K} and the row strides ({a.stride(0)}, {w.stride(0)}) must be multiples "

@@ -51,15 +51,20 @@ class CausalSelfAttention(Mixer):
 
     def forward(self, h, ctx, cache_view: KVCacheView, x, write: bool = True) -> None:
         T = h.shape[0]
+        g = cache_view.group
         qkv = torch.empty((T, self.q_dim + 2 * self.kv_dim), dtype=self.dtype, device=h.device)
+        # Prompt portions: the product writes the new keys and values to the pages itself, unless a
+        # position encoding still has to turn them. (Single tokens: the attention kernel does.)
+        scatter = (write and self.position is None and ctx.max_q_len > 1
+                   and ops.linear_scatters_kv(self.dtype, T))
+        opts = {"kv_scatter": (ctx.slots[g], cache_view.k_pages, cache_view.v_pages, self.q_dim)} if scatter else {}
         if isinstance(h, NormedInput):
-            h.linear(self.qkv, qkv, "store")
+            h.linear(self.qkv, qkv, "store", **opts)
         else:
-            self.qkv(h, qkv, "store")
+            self.qkv(h, qkv, "store", **opts)
         if self.position is not None:
             self.position.in_mixer(qkv, self, ctx)
-        g = cache_view.group
-        append = (self.q_dim, self.q_dim + self.kv_dim, ctx.slots[g]) if write else None
+        append = (self.q_dim, self.q_dim + self.kv_dim, ctx.slots[g]) if write and not scatter else None
         attn = torch.empty((T, self.q_dim), dtype=self.dtype, device=h.device)
         ops.paged_attention(qkv, 0, self.n_heads, self.n_kv_heads, self.head_dim,
                             cache_view.k_pages, cache_view.v_pages, cache_view.page_size,

@@ -75,7 +75,11 @@ class NormedInput:
             self._h = self.norm.forward(self.x)
         return self._h
 
-    def linear(self, lin, out: torch.Tensor, epilogue: str = "store") -> torch.Tensor:
+    def linear(self, lin, out: torch.Tensor, epilogue: str = "store", **linear_options) -> torch.Tensor:
+        """``lin`` applied to the normalised input. Options of the linear map itself (such as a
+        key/value scatter) are its own business: with them the norm runs first, unfused."""
+        if linear_options:
+            return lin(self.tensor(), out, epilogue, **linear_options)
         if self._h is not None:
             return lin(self._h, out, epilogue)
         return self.norm.linear(self.x, lin, out, epilogue)

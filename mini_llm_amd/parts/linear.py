@@ -45,5 +45,8 @@ class Linear:
     def _set_bias(self, t: torch.Tensor) -> None:
         self.bias = t
 
-    def __call__(self, a: torch.Tensor, out: torch.Tensor, epilogue: str = "store") -> torch.Tensor:
+    def __call__(self, a: torch.Tensor, out: torch.Tensor, epilogue: str = "store",
+                 kv_scatter: Optional[tuple] = None) -> torch.Tensor:
+        if kv_scatter is not None:
+            return ops.linear(a, self.weight, self.bias, out, epilogue, kv_scatter=kv_scatter)
         return ops.linear(a, self.weight, self.bias, out, epilogue)

@@ -50,7 +50,11 @@ def _gelu_erf(v):
     return 0.5 * v * (1.0 + torch.erf(v / math.sqrt(2.0)))
 
 
-def linear(a, w, bias, out, epilogue="store"):
+def linear_scatters_kv(dtype, rows):
+    return False
+
+
+def linear(a, w, bias, out, epilogue="store", kv_scatter=None):
     y = a.to(PRECISE) @ w.to(PRECISE).T
     if bias is not None:
         y = y + bias.to(PRECISE)
@@ -62,6 +66,9 @@ def linear(a, w, bias, out, epilogue="store"):
         out.add_(y.to(out.dtype))
     else:
         out.copy_(y.to(out.dtype))
+    if kv_scatter is not None:
+        slots, k_pages, v_pages, q_cols = kv_scatter
+        kv_append(out, q_cols, q_cols + k_pages.shape[1], k_pages.shape[1], k_pages, v_pages, slots)
     return out
 
 
@@ -125,7 +132,7 @@ def sample(logits, temperature, u, out):
     return out
 
 
-_NAMES = ("embed", "select_tokens", "layernorm", "linear", "ln_linear", "kv_append", "paged_attention", "argmax", "sample")
+_NAMES = ("embed", "select_tokens", "layernorm", "linear", "linear_scatters_kv", "ln_linear", "kv_append", "paged_attention", "argmax", "sample")
 
 
 def install(monkeypatch):

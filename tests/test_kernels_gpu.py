@@ -138,6 +138,40 @@ def test_linear_bf16_tile_choices(ops, M, N, K, epi):
     assert err <= (2e-5 + 2e-5 * math.sqrt(K) if f32_out else 4e-2), err
 
 
+@pytest.mark.parametrize("M,H,Hkv,dh,K", [(2048, 12, 12, 64, 768),      # 128x192 tiles
+                                          (300, 6, 2, 16, 96),         # 64x64 tiles, ragged, grouped heads
+                                          (70, 3, 3, 48, 144),         # just above the few-row kernel
+                                          (1000, 16, 4, 32, 520)])
+def test_linear_bf16_scatters_keys_and_values(ops, M, H, Hkv, dh, K):
+    """The fused QKV product with the page write in its epilogue: output as without, and the key
+    and value columns of every row with a slot arrive in that row of the pages, nothing else."""
+    g = torch.Generator().manual_seed(M + K)
+    q_cols, kv_dim = H * dh, Hkv * dh
+    N = q_cols + 2 * kv_dim
+    a = _rand((M, K), torch.bfloat16, g)
+    w = _rand((N, K), torch.bfloat16, g, std=1.0 / math.sqrt(K))
+    bias = 0.5 * _rand((N,), torch.float32, g)
+    rows = M + 37
+    perm = torch.randperm(rows, generator=g)[:M].to(torch.int32)
+    perm[::7] = -1                                   # rows that write nothing
+    k0 = _rand((rows, kv_dim), torch.bfloat16, g)
+    v0 = _rand((rows, kv_dim), torch.bfloat16, g)
+    kp, vp = k0.clone().to(DEV), v0.clone().to(DEV)
+    out = torch.empty((M, N), dtype=torch.bfloat16, device=DEV)
+    assert ops.linear_scatters_kv(torch.bfloat16, M)
+    ops.linear(a.to(DEV), w.to(DEV), bias.to(DEV), out, "store", kv_scatter=(perm.to(DEV), kp, vp, q_cols))
+    plain = torch.empty((M, N), dtype=torch.bfloat16, device=DEV)
+    ops.linear(a.to(DEV), w.to(DEV), bias.to(DEV), plain, "store")
+    assert torch.equal(out, plain)
+    ref = plain_ops.linear(a, w, bias, torch.empty((M, N), dtype=torch.float64))
+    assert (out.cpu().double() - ref).abs().max().item() <= 4e-2
+    kr, vr = k0.clone(), v0.clone()
+    plain_ops.kv_append(out.cpu(), q_cols, q_cols + kv_dim, kv_dim, kr, vr, perm)
+    assert torch.equal(kp.cpu(), kr) and torch.equal(vp.cpu(), vr)
+    with pytest.raises(ops.KernelError, match="scatter"):
+        ops.linear(a[:8].to(DEV), w.to(DEV), None, out[:8], "store", kv_scatter=(perm[:8].to(DEV), kp, vp, q_cols))
+
+
 @pytest.mark.parametrize("M", [1, 8, 16, 17, 48, 64])
 @pytest.mark.parametrize("N,K", [(2304, 768), (768, 3072), (1000, 96), (50257, 768), (72, 1600), (4800, 1600),
                                  (1600, 6400), (1024, 4096)])
