@@ -24,7 +24,8 @@ typedef float f32x4 __attribute__((ext_vector_type(4)));
 #define PF_BM 64
 #define PF_BN 128
 #define PF_TABLE_LDS 2048   // block-table entries staged in LDS (longer tables are read from memory)
-#define PF_VT_STRIDE (PF_BN + 2)   // elements per transposed value row: an odd number of words, so staging writes spread over banks
+#define PF_VT_STRIDE (PF_BN + 2)   // elements per transposed value row: an odd number of words, so that the staging
+                                   // writes of rows 8 apart and the fragment reads of neighbouring rows spread over banks
 
 union Frag8 {
     bf16x8 v;
@@ -103,49 +104,44 @@ prefill_attention_kernel(const bf16_t* __restrict__ q, int q_stride, int q_col,
     // is issued unconditionally, from a key clamped into [k_lo, p_last] (always a held page): a
     // load under a condition would make the compiler wait for all loads in flight. Keys outside
     // that range are masked in the scores, so what was loaded in their place never counts.
-    constexpr int K_ITEMS = PF_BN * (DH / 8) / 256;          // 16-byte key chunks per thread
-    constexpr int V_ITEMS = (PF_BN / 2) * (DH / 8) / 256;    // (key pair, 8 dims) items per thread
-    static_assert(K_ITEMS * 256 == PF_BN * (DH / 8) && V_ITEMS * 256 == (PF_BN / 2) * (DH / 8), "whole items per thread");
+    // A thread takes KPT neighbouring keys (one group, inside one page) and 8 dims of them, keys
+    // and values alike: one block-table lookup and one address per tile, the rest are constant
+    // steps from it.
+    constexpr int CH = DH / 8;                               // 16-byte chunks per row
+    constexpr int KPT = PF_BN * CH / 256;                    // keys per thread: 2, 4, 8 for head sizes 32, 64, 128
+    static_assert(KPT * 256 == PF_BN * CH && (KPT & (KPT - 1)) == 0, "whole key groups per thread");
     typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
-    u32x4 ak[K_ITEMS], av0[V_ITEMS], av1[V_ITEMS];      // register set a
-    u32x4 bk[K_ITEMS], bv0[V_ITEMS], bv1[V_ITEMS];      // register set b
-    auto fetch = [&](u32x4 (&rk)[K_ITEMS], u32x4 (&rv0)[V_ITEMS], u32x4 (&rv1)[V_ITEMS], int kt) {
-        const int j_base = kt * PF_BN;
+    u32x4 ak[KPT], av[KPT];      // register set a
+    u32x4 bk[KPT], bv[KPT];      // register set b
+    const int ch = tid % CH, grp = tid / CH;
+    const int g_lo = k_lo & ~(KPT - 1), g_hi = p_last & ~(KPT - 1);      // first keys of the groups that hold k_lo and p_last
+    auto fetch = [&](u32x4 (&rk)[KPT], u32x4 (&rv)[KPT], int kt) {
+        const int g0 = min(max(kt * PF_BN + grp * KPT, g_lo), g_hi);
+        const size_t base = page_row(g0) * kv_dim + kv_col + 8 * ch;
 #pragma unroll
-        for (int u = 0; u < K_ITEMS; ++u) {
-            const int it = tid + u * 256;
-            const int row = it / (DH / 8), ch = it % (DH / 8);
-            const int jc = min(max(j_base + row, k_lo), p_last);
-            rk[u] = *reinterpret_cast<const u32x4*>(k_pages + page_row(jc) * kv_dim + kv_col + 8 * ch);
-        }
-#pragma unroll
-        for (int u = 0; u < V_ITEMS; ++u) {
-            const int it = tid + u * 256;
-            const int jp = it / (DH / 8), ch = it % (DH / 8);
-            const int j0 = j_base + 2 * jp;
-            const int jc0 = min(max(j0, k_lo), p_last), jc1 = min(max(j0 + 1, k_lo), p_last);
-            rv0[u] = *reinterpret_cast<const u32x4*>(v_pages + page_row(jc0) * kv_dim + kv_col + 8 * ch);
-            rv1[u] = *reinterpret_cast<const u32x4*>(v_pages + page_row(jc1) * kv_dim + kv_col + 8 * ch);
+        for (int u = 0; u < KPT; ++u) {
+            const int off = (min(max(g0 + u, k_lo), p_last) - g0) * kv_dim;     // stays inside the group
+            rk[u] = *reinterpret_cast<const u32x4*>(k_pages + base + off);
+            rv[u] = *reinterpret_cast<const u32x4*>(v_pages + base + off);
         }
     };
-    auto stage = [&](const u32x4 (&rk)[K_ITEMS], const u32x4 (&rv0)[V_ITEMS], const u32x4 (&rv1)[V_ITEMS]) {
-        // keys row-major; values transposed: 8 dims of two neighbouring keys become 8 words
+    auto stage = [&](const u32x4 (&rk)[KPT], const u32x4 (&rv)[KPT]) {
+        // keys row-major; values transposed: dim i of the thread's KPT keys becomes KPT/2 neighbouring words
 #pragma unroll
-        for (int u = 0; u < K_ITEMS; ++u) {
-            const int it = tid + u * 256;
-            *reinterpret_cast<u32x4*>(Ks + (it / (DH / 8)) * KSTRIDE + 8 * (it % (DH / 8))) = rk[u];
-        }
+        for (int u = 0; u < KPT; ++u)
+            *reinterpret_cast<u32x4*>(Ks + (grp * KPT + u) * KSTRIDE + 8 * ch) = rk[u];
+        Frag8 v[KPT];
 #pragma unroll
-        for (int u = 0; u < V_ITEMS; ++u) {
-            const int it = tid + u * 256;
-            const int jp = it / (DH / 8), ch = it % (DH / 8);
-            Frag8 v0, v1;
-            v0.v = __builtin_bit_cast(bf16x8, rv0[u]);
-            v1.v = __builtin_bit_cast(bf16x8, rv1[u]);
+        for (int u = 0; u < KPT; ++u) v[u].v = __builtin_bit_cast(bf16x8, rv[u]);
 #pragma unroll
-            for (int i = 0; i < 8; ++i)
-                *reinterpret_cast<uint32_t*>(Vt + (8 * ch + i) * PF_VT_STRIDE + 2 * jp) =
-                    static_cast<uint32_t>(v0.h[i]) | (static_cast<uint32_t>(v1.h[i]) << 16);
+        for (int i = 0; i < 8; ++i) {
+            uint32_t w[KPT / 2];
+#pragma unroll
+            for (int u = 0; u < KPT; u += 2)
+                w[u / 2] = static_cast<uint32_t>(v[u].h[i]) | (static_cast<uint32_t>(v[u + 1].h[i]) << 16);
+            uint32_t* dst = reinterpret_cast<uint32_t*>(Vt + (8 * ch + i) * PF_VT_STRIDE + grp * KPT);
+#pragma unroll
+            for (int u = 0; u < KPT / 2; ++u) dst[u] = w[u];
         }
     };
 
@@ -168,7 +164,7 @@ prefill_attention_kernel(const bf16_t* __restrict__ q, int q_stride, int q_col,
             }
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
-                s[nt][r] = acc[r] * scale_log2e;
+                s[nt][r] = acc[r];                   // raw dot product; the scale is applied with the exponent
                 if (MASKED) {
                     const int j = j_base + 16 * nt + 4 * G + r;
                     const bool seen = q_ok && j <= p && (window <= 0 || j > p - window);
@@ -180,7 +176,7 @@ prefill_attention_kernel(const bf16_t* __restrict__ q, int q_stride, int q_col,
         // the four lane groups of a query agree on the maximum
         tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 16, MLLM_WAVE));
         tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 32, MLLM_WAVE));
-        const float m_new = fmaxf(m, tile_max);
+        const float m_new = fmaxf(m, tile_max * scale_log2e);        // the scale is positive
         const float m_use = (m_new == -INFINITY) ? 0.f : m_new;      // nothing seen yet: all weights are 0
         const float alpha = fast_exp2(m - m_use);
         m = m_new;
@@ -189,7 +185,7 @@ prefill_attention_kernel(const bf16_t* __restrict__ q, int q_stride, int q_col,
         for (int nt = 0; nt < PF_BN / 16; ++nt)
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
-                s[nt][r] = fast_exp2(s[nt][r] - m_use);
+                s[nt][r] = fast_exp2(fmaf(s[nt][r], scale_log2e, -m_use));
                 psum += s[nt][r];
             }
         l = l * alpha + psum;                 // this lane's share of the sum; merged over groups at the end
@@ -229,19 +225,19 @@ prefill_attention_kernel(const bf16_t* __restrict__ q, int q_stride, int q_col,
     // Two register sets, each fetched two tiles ahead of its use. The loop body has no branch
     // around a load; past the last tile the fetches repeat clamped keys and nothing is computed.
     const int kt_first = k_lo / PF_BN, kt_last = p_last / PF_BN;
-    fetch(ak, av0, av1, kt_first);
+    fetch(ak, av, kt_first);
     __builtin_amdgcn_sched_barrier(0);     // set a's loads stay the older ones, as on every later iteration
-    fetch(bk, bv0, bv1, kt_first + 1);
+    fetch(bk, bv, kt_first + 1);
     for (int kt = kt_first; kt <= kt_last; kt += 2) {
         lds_barrier();                     // the previous tile's readers are done
-        stage(ak, av0, av1);
+        stage(ak, av);
         lds_barrier();
-        fetch(ak, av0, av1, kt + 2);
+        fetch(ak, av, kt + 2);
         run_tile(kt);
         lds_barrier();
-        stage(bk, bv0, bv1);
+        stage(bk, bv);
         lds_barrier();
-        fetch(bk, bv0, bv1, kt + 3);
+        fetch(bk, bv, kt + 3);
         if (kt + 1 <= kt_last) run_tile(kt + 1);
     }
     l += __shfl_xor(l, 16, MLLM_WAVE);
@@ -264,7 +260,8 @@ extern "C" {
 // n_tiles_upper: an upper bound of the number of 64-query tiles, sum over sequences of
 // ceil(q_len / 64) (e.g. n_tokens / 64 + n_seqs); surplus workgroups leave at once.
 // Returns 0, a HIP error code, or -1 when the head size is not 32, 64 or 128, the page size is no
-// power of two, or a block table has more than PF_TABLE_LDS entries.
+// power of two or smaller than head_dim / 16 (a thread's group of keys must lie in one page), or a
+// block table has more than PF_TABLE_LDS entries.
 int mllm_prefill_attention_bf16(const void* q, int q_stride, int q_col, const void* k_pages, const void* v_pages,
                                 int kv_dim, const int* block_tables, int max_blocks, const int* cu_q,
                                 const int* ctx_len, int n_seqs, int n_tiles_upper, int n_heads, int n_kv_heads,
@@ -272,7 +269,7 @@ int mllm_prefill_attention_bf16(const void* q, int q_stride, int q_col, const vo
                                 hipStream_t stream) {
     if (n_seqs <= 0 || n_tiles_upper <= 0) return 0;
     if (n_heads % n_kv_heads != 0 || n_tiles_upper > 65535) return -1;
-    if ((page_size & (page_size - 1)) != 0 || max_blocks > PF_TABLE_LDS) return -1;
+    if ((page_size & (page_size - 1)) != 0 || page_size < head_dim / 16 || max_blocks > PF_TABLE_LDS) return -1;
     const dim3 grid(n_heads, n_tiles_upper);
     const float sl2 = scale * 1.44269504088896340736f;
 #define PF_CASE(D)                                                                                          \

@@ -336,7 +336,8 @@ def paged_attention(q: torch.Tensor, q_col: int, n_heads: int, n_kv_heads: int, 
         return out
     if (q.dtype == torch.bfloat16 and head_dim in (32, 64, 128) and max_q_len > 1
             and cu_q is not None and ctx_len is not None
-            and page_size & (page_size - 1) == 0 and block_tables.shape[1] <= 2048):
+            and page_size & (page_size - 1) == 0 and page_size >= head_dim // 16
+            and block_tables.shape[1] <= 2048):
         # prompt portions: tiles of 64 queries on the matrix cores
         B = block_tables.shape[0]
         _i32(cu_q, "cu_q", B + 1)
