@@ -110,6 +110,76 @@ def prefill_run(model_dir, dtype, cfg, n_req=2, n_tok=1024, reps=5):
     return T / dt, dt, flops
 
 
+def serving_run(model_dir, dtype, cfg, n_req, prompt_lo, prompt_hi, new_tokens, max_batch, chunk, pages, seed):
+    """Continuous batching from a full queue: n_req requests with prompt lengths uniform in
+    [prompt_lo, prompt_hi] and new_tokens generated each, prompts fed in portions of `chunk`, at most
+    max_batch requests a step, `pages` pages of 16 tokens in the pool. Returns a dictionary of
+    totals, times and the scheduler's counters."""
+    import torch
+    from mini_llm_amd import Engine, EngineOptions, SamplingParams
+    engine = Engine.from_pretrained(model_dir, dtype=dtype, device="cuda:0",
+                                    options=EngineOptions(kv_block_size=16, total_kv_blocks=pages,
+                                                          max_batch_num=max_batch,
+                                                          max_tokens_per_step=max(2048, max_batch + chunk),
+                                                          prefill_chunk=chunk))
+    g = torch.Generator().manual_seed(seed)
+    lens = torch.randint(prompt_lo, prompt_hi + 1, (n_req,), generator=g).tolist()
+    params = SamplingParams(max_new_tokens=new_tokens, ignore_eos=True)
+    for n in lens:
+        engine.add_request(torch.randint(0, cfg["vocab_size"], (n,), generator=g).tolist(), params)
+    # untimed: one short request through prefill and decode loads the kernels and captures nothing that
+    # the timed run would not capture itself
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    n_out = n_steps = 0
+    first = None
+    while engine.has_unfinished():
+        outs = engine.step()
+        n_steps += 1
+        if outs and first is None:
+            torch.cuda.synchronize()
+            first = time.perf_counter() - t0
+        n_out += sum(1 for o in outs if o.token >= 0)
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    st = engine.stats()
+    failed = sum(1 for r in engine.requests.values() if r.failed)
+    assert n_out == (n_req - failed) * new_tokens, (n_out, n_req, failed, new_tokens)
+    assert st["free_pages"] == pages and engine.runner.manager.check() == ""
+    return {"seconds": dt, "generated": n_out, "prompt_tokens": sum(lens), "steps": n_steps,
+            "first_token_s": first, "failed": failed, "counters": st}
+
+
+def serving_main(args, cfg, model_dir):
+    """--workload continuous: BASELINE.json configs[3] (made for GPT-2 medium sizes); --workload
+    kv-pressure: the second workload of configs[4] (GPT-2 XL sizes), the pool capped at 60 % of what
+    the 64 requests of a full batch hold at their end, so that requests are deferred and preempted."""
+    if args.workload == "continuous":
+        n_req, lo, hi, new, max_batch, chunk = 64, 64, 768, 256, 64, 256
+        pages = n_req * ((hi + new + 15) // 16) + 16
+    else:
+        n_req, lo, hi, new, max_batch, chunk = 256, 512, 512, 512, 64, 512
+        pages = int(0.6 * max_batch * ((hi + new + 15) // 16))
+    r = serving_run(model_dir, args.dtype, cfg, n_req, lo, hi, new, max_batch, chunk, pages, seed=7)
+    c = r["counters"]
+    rec = {"metric": f"generated tok/s, {args.workload} workload ({args.size} sizes)",
+           "value": round(r["generated"] / r["seconds"], 1), "unit": "tok/s", "n_gpus": 1,
+           "steps": r["steps"], "warmup": 0, "ms_per_step": round(1e3 * r["seconds"] / r["steps"], 4),
+           "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+           "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
+           "data": "synthetic (random weights seed 2, uniform random token ids and prompt lengths, seed 7)",
+           "config": {"model": args.size + "-sizes", "n_layer": cfg["n_layer"], "n_layer_full": SIZES[args.size][0],
+                      "requests": n_req, "prompt_min": lo, "prompt_max": hi, "new_tokens": new,
+                      "max_batch_num": max_batch, "prefill_chunk": chunk, "kv_blocks": pages, "kv_block_size": 16,
+                      "prompt_tokens": r["prompt_tokens"], "generated_tokens": r["generated"],
+                      "total_tok_per_s": round((r["generated"] + r["prompt_tokens"]) / r["seconds"], 1),
+                      "seconds": round(r["seconds"], 3), "first_token_ms": round(1e3 * (r["first_token_s"] or 0), 2),
+                      "preemptions": c["preemptions"], "deferred_decodes": c["deferred_decodes"],
+                      "deferred_prefills": c["deferred_prefills"], "failed": r["failed"]}}
+    print(json.dumps(rec))
+    return 0
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -122,6 +192,9 @@ def main():
     ap.add_argument("--prompt-len", type=int, default=512)
     ap.add_argument("--no-points", action="store_true", help="skip the batch-1/64 and prefill measurements")
     ap.add_argument("--prefill-only", action="store_true", help="measure only the 2,048-token prefill (profiling)")
+    ap.add_argument("--workload", default="decode", choices=["decode", "continuous", "kv-pressure"],
+                    help="decode: the headline measurement; continuous / kv-pressure: a queue of requests "
+                         "through the scheduler (BASELINE.json configs[3] and configs[4])")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
@@ -134,26 +207,33 @@ def main():
     steps = min(args.steps, cfg["n_positions"] - args.prompt_len - args.warmup - 2 - 64)
     with tempfile.TemporaryDirectory() as d:
         write_random_model(dict(cfg), d, seed=2)
+        if args.workload != "decode":
+            return serving_main(args, cfg, d)
         if args.prefill_only:
             ptps, pdt, flops = prefill_run(d, args.dtype, cfg)
             print(json.dumps({"metric": "prefill tok/s at 2,048 tokens", "value": round(ptps, 1), "unit": "tok/s",
                               "ms": round(pdt * 1e3, 4), "frac": round(flops / pdt / MFMA_PEAK[args.dtype], 5)}))
             return 0
         tps, step_s, mean_ctx = decode_run(d, args.dtype, args.batch, args.prompt_len, steps, args.warmup, cfg)
+        # The reference's own decode numbers at this workload (GPT-2 small, 512-token prompts; fp32 on a
+        # TITAN V: /root/reference benchmark gpt2_decode_batch_sweep_512.csv:2-5), where it has one.
+        reference_tps = {1: 116.9, 2: 223.1, 4: 438.6, 8: 854.4}.get(args.batch) \
+            if (args.size == "gpt2-small" and args.prompt_len == 512 and cfg["n_layer"] == SIZES[args.size][0]) else None
         bytes_step = weight_bytes(cfg, esz) + args.batch * mean_ctx * kv_bytes_per_token(cfg, esz)
         achieved = bytes_step / step_s
         rec = {
             "metric": f"decode tok/s at batch {args.batch} ({args.size} sizes, {args.prompt_len}-token prompts)",
             "value": round(tps, 1), "unit": "tok/s", "n_gpus": 1, "steps": steps, "warmup": args.warmup,
             "ms_per_step": round(step_s * 1e3, 4), "higher_is_better": True, "scaling": "weak",
-            "vs_baseline": None, "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
+            "vs_baseline": round(tps / reference_tps, 2) if reference_tps else None, "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
             "data": "synthetic (random weights seed 2, uniform random token ids)",
             "config": {"model": args.size + "-sizes", "n_layer": cfg["n_layer"], "n_layer_full": SIZES[args.size][0],
                        "n_embd": cfg["n_embd"], "n_head": cfg["n_head"], "head_dim": cfg["n_embd"] // cfg["n_head"],
                        "n_inner": cfg["n_inner"], "vocab_size": cfg["vocab_size"],
                        "n_positions": cfg["n_positions"], "global_batch": args.batch,
                        "prompt_len": args.prompt_len, "seq_len": cfg["n_positions"],
-                       "mean_context": round(mean_ctx, 1), "kv_block_size": 16, "parallelism": "single-gpu"},
+                       "mean_context": round(mean_ctx, 1), "kv_block_size": 16, "parallelism": "single-gpu",
+                       "baseline": (f"{reference_tps} tok/s: the reference, fp32, TITAN V" if reference_tps else "none")},
             "roofline": {"bound": "hbm", "achieved": round(achieved / 1e9, 2), "peak": HBM_PEAK / 1e9,
                          "unit": "GB/s", "frac": round(achieved / HBM_PEAK, 5)},
         }
