@@ -242,11 +242,13 @@ class ModelRunner:
         greedy = temperatures is None or all(t <= 0 for t in temperatures)
         bucket = B if B <= 8 else -(-B // 8) * 8
         if self._tok_out is None or self._tok_out.numel() < bucket:
-            if self._graphs:
-                # captured graphs hold the old buffer's address
-                self._graphs.clear()
+            # (sized for the most requests the cache manager admits, so this happens once)
             n = max(bucket, -(-self.manager.n_state_slots // 8) * 8, 8)
-            self._tok_out = torch.zeros(n, dtype=torch.int32, device=self.device)
+            grown = torch.zeros(n, dtype=torch.int32, device=self.device)
+            if self._tok_out is not None:
+                grown[:self._tok_out.numel()].copy_(self._tok_out)     # tokens a later launch may still take
+                self._graphs.clear()                                   # captured graphs hold the old address
+            self._tok_out = grown
         key = (bucket, greedy)
         g = self._graphs.get(key)
         if g is None:

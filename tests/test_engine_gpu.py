@@ -159,3 +159,29 @@ def test_random_preset_entry_points(tmp_path):
     bad = subprocess.run([sys.executable, cli, "generate", "--preset", "no-such-size", "--prompt-ids", "1"],
                          capture_output=True, text=True, timeout=120)
     assert bad.returncode == 1 and "unknown preset" in bad.stderr
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_end_of_sequence_under_overlapped_graph_decode(tiny_model_dirs, dtype):
+    """A decoded end-of-sequence token is read one step late while HIP graphs replay: generation
+    still ends with that token for that request only, under page pressure too, and all pages return."""
+    from mini_llm_amd import Engine, EngineOptions, SamplingParams
+    prompts = _prompts("b", (7, 19, 30, 52), 3)
+
+    def run(eos, pages, overlap, **sp):
+        e = Engine.from_pretrained(tiny_model_dirs["b"], dtype=dtype,
+                                   options=EngineOptions(kv_block_size=8, total_kv_blocks=pages, max_batch_num=4,
+                                                         overlap_decode=overlap))
+        e.eos_token_id = eos
+        out = e.generate(prompts, [SamplingParams(temperature=1.3, seed=20 + i, max_new_tokens=18, **sp)
+                                   for i in range(len(prompts))])
+        assert e.stats()["free_pages"] == pages and e.runner.manager.check() == "" and not e.has_unfinished()
+        return out
+
+    full = run(None, 64, True, ignore_eos=True)
+    j = next(j for j in range(2, 18) if full[1][j] not in full[1][:j])
+    eos = full[1][j]
+    expect = [o[:o.index(eos) + 1] if eos in o else o for o in full]
+    assert len(expect[1]) == j + 1
+    for pages, overlap in ((64, True), (64, False), (22, True)):
+        assert run(eos, pages, overlap) == expect
