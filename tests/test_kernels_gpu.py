@@ -194,7 +194,9 @@ def test_linear_bf16_few_rows(ops, M, N, K):
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("M,N,K", [(1, 2304, 768), (8, 3072, 768), (16, 320, 96), (5, 200, 1600), (17, 96, 64),
                                    (3, 64, 4096), (16, 6400, 1600), (9, 50257, 1024), (16, 3072, 1024), (33, 2304, 768),
-                                   (64, 50257, 768), (64, 104, 1600), (65, 96, 64)])
+                                   (64, 50257, 768), (64, 104, 1600), (65, 96, 64),
+                                   # more than 16 rows: the norm runs as a kernel of its own
+                                   (64, 3072, 768), (48, 4096, 1024), (17, 40, 72), (31, 1000, 2048), (50, 136, 200)])
 @pytest.mark.parametrize("epi", ["store", "gelu_tanh", "gelu_erf", "store_f32"])
 def test_ln_linear(ops, dtype, M, N, K, epi):
     """LayerNorm fused into the product (bf16, few rows) and its unfused form give the plain result."""
