@@ -39,7 +39,14 @@ def _gpu(*tensors: Optional[torch.Tensor]) -> None:
                 f"(device={t.device}, shape={tuple(t.shape)})")
 
 
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
 def _stream() -> ctypes.c_void_p:
+    """The current HIP stream of the current device (the raw handle: building a Stream object
+    for every launch costs more than many of the launches)."""
+    if _raw_stream is not None:
+        return ctypes.c_void_p(_raw_stream(torch.cuda.current_device()))
     return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
 
 
