@@ -20,6 +20,9 @@ class Linear:
                  dtype: torch.dtype, device, init_std: float = 0.02, bias_std: float = 0.02):
         if weight_layout not in ("in_out", "out_in"):
             raise ValueError(f"weight_layout must be 'in_out' or 'out_in', got {weight_layout!r}")
+        if dtype == torch.bfloat16 and in_features % 8 != 0:
+            raise ValueError(f"a bfloat16 linear map needs an input width that is a multiple of 8, got "
+                             f"{in_features} (its kernels load 16 bytes at a time); use float32 for this size")
         self.in_features, self.out_features = in_features, out_features
         self.has_bias = bias
         self.weight_layout = weight_layout

@@ -170,3 +170,22 @@ def test_loader_lists_every_mismatch(tmp_path):
     os.remove(os.path.join(d, "model.safetensors"))
     with pytest.raises(WeightsError, match="neither model.safetensors"):
         load_model(d, "float32", "cpu")
+
+
+def test_sizes_the_kernels_cannot_take_are_refused_when_the_model_is_built(tmp_path):
+    """A feed-forward width that is no multiple of 8 has no bfloat16 kernel: building the model says
+    so (float32 takes it); a head size that is no multiple of 16 is refused for every dtype."""
+    from mini_llm_amd import load_model, write_random_model
+    cfg = dict(json.load(open(os.path.join(os.path.dirname(__file__), "..", "mini_llm_amd", "config", "presets",
+                                          "tiny-a.json"))))
+    cfg["n_inner"] = 100
+    d = str(tmp_path / "odd")
+    write_random_model(cfg, d, seed=0)
+    with pytest.raises(ValueError, match="multiple of 8"):
+        load_model(d, "bfloat16", "cpu")
+    assert load_model(d, "float32", "cpu") is not None
+    cfg2 = dict(cfg, n_inner=256, n_embd=40, n_head=4)     # head size 10
+    d2 = str(tmp_path / "odd2")
+    with pytest.raises(ValueError, match="head"):
+        write_random_model(cfg2, d2, seed=0)
+        load_model(d2, "float32", "cpu")
