@@ -12,7 +12,7 @@ dtype):
   in place; ``cache_spec()`` says what cache it needs (or None).
 * ``FeedForward.forward(h, ctx, x)``: adds its output into ``x`` in place.
 * ``PositionEncoding.at_embedding(x, ctx)`` / ``.table``: acts where tokens are
-  embedded; ``.in_mixer(q, k, ctx)``: acts on queries/keys inside a mixer.
+  embedded; ``.in_mixer(qkv, mixer, ctx)``: turns queries/keys in place inside a mixer.
 * ``Block.forward(x, ctx, cache_view, write)``: runs one layer on the stream.
 """
 from __future__ import annotations
@@ -107,13 +107,20 @@ class FeedForward(Part):
 
 
 class PositionEncoding(Part):
+    """How positions enter the model. Three places, any of which an encoding may use: a learned
+    table added where tokens are embedded (``table``, fused into the embedding kernel),
+    ``at_embedding`` (anything else done to the embedded stream), and ``in_mixer`` (queries and
+    keys turned by position inside every mixer that takes positions: set ``applies_in_mixer``)."""
+
     table: Optional[torch.Tensor] = None     # learned absolute table, if the encoding is one
+    applies_in_mixer = False                 # True: mixers call in_mixer() before keys are written
 
     def at_embedding(self, x, ctx) -> None:
         pass
 
-    def in_mixer(self, q, k, ctx):
-        return q, k
+    def in_mixer(self, qkv: torch.Tensor, mixer, ctx) -> None:
+        """Changes, in place, the query and key columns of ``qkv`` ([T, q | k | v], the mixer says
+        where: mixer.q_dim, mixer.kv_dim, mixer.head_dim) for the positions ``ctx.positions``."""
 
 
 class Block(Part):

@@ -298,3 +298,207 @@ def test_toy_architecture_with_a_stateful_mixer(tmp_path, dtype):
     runner.end_request(3)
     out = runner.step([StepEntry(4, seqs[3], list(range(9)))]).float().cpu()
     assert (out.double() - _toy_plain(w, cfg, seqs[3])).abs().max() <= tol
+
+
+# ---------------------------------------------------------------------------------------------
+# A second toy architecture: a position encoding that turns queries and keys inside the mixer
+# (no table at the embedding), a feed-forward that routes every token to one of several experts
+# in the first layer and a dense one in the second, grouped heads, a window in the second layer.
+# The toy parts compute with torch; the framework's own parts around them run their kernels.
+# ---------------------------------------------------------------------------------------------
+
+def _define_routed_toy():
+    from mini_llm_amd.config.base import LayerCall, LayerSpec, ModelConfig, PartSpec
+    from mini_llm_amd.config.registry import register_architecture
+    from mini_llm_amd.models.decoder import DecoderModel, build_layers
+    from mini_llm_amd.parts.base import (FeedForward, ParamSpec, PositionEncoding, register_feed_forward,
+                                         register_position)
+    from mini_llm_amd.parts.embedding import TiedHead, TokenEmbedding
+    from mini_llm_amd.parts.norms import LayerNorm
+
+    @register_position("toy_half_turn", replace=True)
+    class HalfTurn(PositionEncoding):
+        """Per head, the pair (v[i], v[i + dh/2]) is turned by the angle pos * base^(-i / (dh/2))."""
+        applies_in_mixer = True
+        max_positions = None
+
+        def __init__(self, base, dtype, device):
+            super().__init__(dtype, device)
+            self.base = base
+
+        def in_mixer(self, qkv, mixer, ctx):
+            dh, half = mixer.head_dim, mixer.head_dim // 2
+            rate = self.base ** (-torch.arange(half, device=qkv.device, dtype=torch.float32) / half)
+            angle = ctx.positions[:qkv.shape[0]].float()[:, None, None] * rate
+            cos, sin = angle.cos(), angle.sin()
+            qk = qkv[:, :mixer.q_dim + mixer.kv_dim].view(qkv.shape[0], -1, dh)
+            a, b = qk[..., :half].float(), qk[..., half:].float()
+            turned = torch.cat([a * cos - b * sin, b * cos + a * sin], dim=-1)   # before qk is written
+            qk.copy_(turned)
+
+    @register_feed_forward("toy_one_of_n", replace=True)
+    class OneOfN(FeedForward):
+        """p = softmax(h R^T) in fp32; the token goes to expert e = argmax p and
+        x += p_e * W2_e gelu(W1_e h)."""
+
+        def __init__(self, size, inner, n_experts, dtype, device):
+            super().__init__(dtype, device)
+            self.size, self.inner, self.n = size, inner, n_experts
+            self.router, self.up, self.down = None, [None] * n_experts, [None] * n_experts
+
+        def param_specs(self, prefix):
+            def put(lst, e):
+                return lambda t: lst.__setitem__(e, t)
+            specs = [ParamSpec(prefix + "router", (self.n, self.size), "vector",
+                               lambda t: setattr(self, "router", t), (0.0, 1.0))]
+            for e in range(self.n):
+                specs.append(ParamSpec(f"{prefix}expert.{e}.up", (self.inner, self.size), "matrix", put(self.up, e)))
+                specs.append(ParamSpec(f"{prefix}expert.{e}.down", (self.size, self.inner), "matrix", put(self.down, e)))
+            return specs
+
+        def forward(self, h, ctx, x):
+            p = torch.softmax(h.float() @ self.router.t(), dim=-1)
+            gate, chosen = p.max(dim=-1)
+            for e in range(self.n):
+                y = torch.nn.functional.gelu(h @ self.up[e].t()) @ self.down[e].t()
+                x += (gate * (chosen == e))[:, None] * y.float()
+
+    @dataclasses.dataclass(frozen=True)
+    class RoutedConfig(ModelConfig):
+        vocab: int
+        width: int
+        heads: int
+        groups: int
+        experts: int
+        window: int
+        base: float
+        eps: float
+        architecture = "ToyRoutedLM"
+
+        @property
+        def vocab_size(self):
+            return self.vocab
+
+        @property
+        def hidden_size(self):
+            return self.width
+
+        @classmethod
+        def from_dict(cls, d):
+            return cls(*(d[k] for k in ("vocab", "width", "heads", "groups", "experts", "window", "base", "eps")))
+
+        def to_dict(self):
+            return dict(dataclasses.asdict(self), architectures=["ToyRoutedLM"])
+
+        def layer_specs(self):
+            dh = self.width // self.heads
+            norm = PartSpec("layernorm", {"size": self.width, "eps": self.eps})
+            dense = PartSpec("dense_mlp", dict(hidden_size=self.width, inner_size=3 * self.width, activation="gelu_tanh",
+                                               bias=True, weight_layout="out_in", names={"up": "up", "down": "down"}))
+            routed = PartSpec("toy_one_of_n", dict(size=self.width, inner=2 * self.width, n_experts=self.experts))
+            att = lambda window: PartSpec("causal_attention", dict(
+                hidden_size=self.width, n_heads=self.heads, n_kv_heads=self.groups, head_dim=dh,
+                scale=1.0 / math.sqrt(dh), window=window, bias=True, weight_layout="out_in",
+                names={"qkv": "qkv", "out": "o"}))
+            return [LayerSpec("pre_norm", att(None), routed, norm, "l0.", ("n1", "n2")),
+                    LayerSpec("pre_norm", att(self.window), dense, norm, "l1.", ("n1", "n2"))]
+
+        def layer_order(self):
+            return [LayerCall(0, 0), LayerCall(1, 1)]
+
+    def build(config, dtype, device):
+        emb = TokenEmbedding(config.vocab, config.width, "emb", dtype, device)
+        turn = HalfTurn(config.base, dtype, device)
+        layers, prefixes = build_layers(config.layer_specs(), dtype, device, position=turn)
+        final = LayerNorm(size=config.width, eps=config.eps, dtype=dtype, device=device)
+        return DecoderModel(config, emb, turn, layers, prefixes, config.layer_order(),
+                            final, "final", TiedHead(emb, dtype, device), dtype, device)
+
+    register_architecture("ToyRoutedLM", RoutedConfig, build, replace=True)
+
+
+def _routed_plain(w, cfg, ids):
+    """Whole sequence, no cache, float64. Returns the logits and the smallest gap between the
+    two largest router logits of any token (a tie there would make the comparison meaningless)
+    and the set of experts that were chosen."""
+    D, H, G = cfg["width"], cfg["heads"], cfg["groups"]
+    dh, n = D // H, len(ids)
+    x = w["emb.weight"][torch.tensor(ids)]
+    ln = lambda x, p: P.layer_norm(x, w[p + ".weight"], w[p + ".bias"], cfg["eps"])
+    pos = torch.arange(n, dtype=torch.float64)
+    turn_by = torch.polar(torch.ones(n, dh // 2, dtype=torch.float64),
+                          pos[:, None] * cfg["base"] ** (-torch.arange(dh // 2, dtype=torch.float64) / (dh // 2)))
+
+    def turn(t, heads):
+        t = t.view(n, heads, dh)
+        z = torch.complex(t[..., :dh // 2], t[..., dh // 2:]) * turn_by[:, None, :]
+        return torch.cat([z.real, z.imag], dim=-1)
+
+    gap, used = float("inf"), set()
+    for layer in (0, 1):
+        p = f"l{layer}."
+        qkv = ln(x, p + "n1") @ w[p + "qkv.weight"].T + w[p + "qkv.bias"]
+        q = turn(qkv[:, :D], H).reshape(n, D)
+        k = turn(qkv[:, D:D + G * dh], G)
+        v = qkv[:, D + G * dh:].view(n, G, dh)
+        wide = lambda t: t[:, :, None, :].expand(n, G, H // G, dh).reshape(n, D)
+        a = P.causal_attention(q, wide(k), wide(v), H, window=cfg["window"] if layer == 1 else None)
+        x = x + a @ w[p + "o.weight"].T + w[p + "o.bias"]
+        h = ln(x, p + "n2")
+        if layer == 0:
+            scores = h @ w[p + "router"].T
+            top = scores.topk(2, dim=-1).values
+            gap = min(gap, float((top[:, 0] - top[:, 1]).min()))
+            prob = torch.softmax(scores, dim=-1)
+            rows = []
+            for t in range(n):
+                e = int(prob[t].argmax())
+                used.add(e)
+                rows.append(prob[t, e] * (P.gelu_erf(h[t] @ w[f"{p}expert.{e}.up"].T) @ w[f"{p}expert.{e}.down"].T))
+            x = x + torch.stack(rows)
+        else:
+            x = x + P.gelu_tanh(h @ w[p + "up.weight"].T + w[p + "up.bias"]) @ w[p + "down.weight"].T + w[p + "down.bias"]
+    return ln(x, "final") @ w["emb.weight"].T, gap, used
+
+
+ROUTED_CFG = dict(architectures=["ToyRoutedLM"], vocab=157, width=64, heads=4, groups=2, experts=3, window=6,
+                  base=50.0, eps=1e-5)
+ROUTED_SEED = 30
+
+
+def _routed_sequences():
+    g = torch.Generator().manual_seed(ROUTED_SEED)
+    return {1: torch.randint(0, 157, (26,), generator=g).tolist(), 2: torch.randint(0, 157, (15,), generator=g).tolist()}
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_toy_architecture_with_turned_keys_and_routed_experts(tmp_path, dtype):
+    from safetensors import safe_open
+    from mini_llm_amd import write_random_model
+    from mini_llm_amd.engine.step import ModelRunner, StepEntry
+    from mini_llm_amd.models import load_model
+    _define_routed_toy()
+    d = write_random_model(ROUTED_CFG, str(tmp_path / "routed"), seed=ROUTED_SEED)
+    model = load_model(d, dtype, DEV)
+    assert all(layer.mixer.position is model.position for layer in model.layers)
+    runner = ModelRunner(model, page_size=4, n_pages=14, max_num_seqs=2)
+    runner.cache.poison()
+    with safe_open(d + "/model.safetensors", framework="pt") as f:
+        w = {k: f.get_tensor(k).double() for k in f.keys()}
+    seqs = _routed_sequences()
+    got, fed = {r: [] for r in seqs}, {r: 0 for r in seqs}
+    plan = [{1: 9, 2: 2}, {1: 1, 2: 6}, {1: 1}, {1: 13, 2: 1}, {1: 2, 2: 6}]
+    for step in plan:
+        entries = [StepEntry(r, seqs[r][fed[r]:fed[r] + n], list(range(n))) for r, n in step.items()]
+        logits = runner.step(entries).float().cpu()
+        i = 0
+        for r, n in step.items():
+            got[r].append(logits[i:i + n])
+            i += n
+            fed[r] += n
+    tol = 3e-5 if dtype == "float32" else 4e-2
+    for r, ids in seqs.items():
+        assert fed[r] == len(ids)
+        ref, gap, used = _routed_plain(w, ROUTED_CFG, ids)
+        assert gap > 0.3 and len(used) >= 2, "the seed gives a near tie between experts, or one expert only"
+        assert (torch.cat(got[r]).double() - ref).abs().max() <= tol, r
