@@ -283,6 +283,11 @@ static void launch_tiled(const bf16_t* a, int lda, const bf16_t* w, int ldw, con
 //   SPLIT_K:  one workgroup per 16-column tile, its wavefronts split K (wavefront w takes the
 //             64-element k blocks w, w+NW, ...) and their partial sums are added in LDS in a fixed
 //             order: for the narrow products, where tiles alone are too few to fill the chip.
+//             With k_parts > 1 several workgroups share a tile as well (blockIdx.y is the part):
+//             each writes its sum to a workspace, and the last one to arrive, found through a
+//             counter per tile, adds the parts in the order of their index and runs the
+//             epilogue. For products whose tiles alone use a fraction of the compute units and
+//             whose K is long (the second product of the feed-forward).
 //   !SPLIT_K: one wavefront per tile over the whole of K (wide products such as the logits head).
 // The activations come from global memory (A_GLOBAL: a few KB, shared by all workgroups, read
 // from L2), are copied into LDS once per workgroup (A_STAGED: wide products), or are normalised
@@ -298,8 +303,10 @@ __global__ void __launch_bounds__(ASRC == A_NORMED ? 512 : 1024)
 gemm_bf16_skinny(const void* __restrict__ Ain, int lda, const bf16_t* __restrict__ W, int ldw,
                  const float* __restrict__ bias, void* __restrict__ C, int ldc, int M, int N, int K, int mode,
                  const float* __restrict__ gamma, const float* __restrict__ beta, float eps,
-                 const int* __restrict__ rows, int col_blocks, int row_blocks) {
+                 const int* __restrict__ rows, int col_blocks, int row_blocks, int k_parts,
+                 float* __restrict__ part_sums, int* __restrict__ part_counters) {
     extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
+    __shared__ int sm_last;
     constexpr bool LN_FUSED = ASRC == A_NORMED;
     constexpr bool IN_LDS = ASRC != A_GLOBAL;
     const int tid = threadIdx.x, wave = tid / 64, lane = tid % 64;
@@ -316,8 +323,10 @@ gemm_bf16_skinny(const void* __restrict__ Ain, int lda, const bf16_t* __restrict
     // takes elements 16*kq .. 16*kq+15 of a block, the first 8 in one MFMA and the rest in the
     // next (the k index of an MFMA may be permuted as long as both operands agree), so that a
     // wavefront uses every line it touches whole.
-    const int k_first = SPLIT_K ? wave * 64 : 0;      // first k block of this wavefront
-    const int k_stride = SPLIT_K ? nw * 64 : 64;      // distance between its k blocks
+    // (with k_parts workgroups on the tile, over all their wavefronts alike)
+    const int part = SPLIT_K ? blockIdx.y : 0;
+    const int k_first = SPLIT_K ? (part * nw + wave) * 64 : 0;      // first k block of this wavefront
+    const int k_stride = SPLIT_K ? nw * k_parts * 64 : 64;         // distance between its k blocks
     const size_t red_bytes = SPLIT_K ? static_cast<size_t>(nw) * MT * 256 * sizeof(float) : 0;
     float* red = reinterpret_cast<float*>(smem_raw);                       // [nw][MT][256]
     bf16_t* a_s = reinterpret_cast<bf16_t*>(smem_raw + red_bytes);         // [16*MT][K+8]
@@ -545,9 +554,36 @@ gemm_bf16_skinny(const void* __restrict__ Ain, int lda, const bf16_t* __restrict
     if (MT == 1) {
         // one output per thread (the first 256); its bias and old residual value were requested
         // before the MFMA loop
-        if (ep_ok) {
-            float v = 0.f;
+        float v = 0.f;
+        if (tid < 256)
             for (int w = 0; w < nw; ++w) v += red[static_cast<size_t>(w) * 256 + tid];
+        if (k_parts > 1) {
+            // The parts of a tile meet in the workspace. Stores and loads of it are at device scope
+            // (workgroups of one tile may run on different XCDs, whose L2 caches do not see each
+            // other's lines); one thread's fences order them around the counter (a fence in every
+            // thread costs tens of microseconds here, one about 1.5). The last workgroup leaves the
+            // counter at zero for the next launch.
+            const int tile = cb * row_blocks + rb;
+            float* sums = part_sums + static_cast<size_t>(tile) * k_parts * 256;
+            if (tid < 256) __hip_atomic_store(&sums[part * 256 + tid], v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __syncthreads();
+            if (tid == 0) {
+                __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");      // after the barrier: covers every thread's stores
+                const int arrived = __hip_atomic_fetch_add(&part_counters[tile], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                sm_last = (arrived == k_parts - 1) ? 1 : 0;
+                if (sm_last) {
+                    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+                    __hip_atomic_store(&part_counters[tile], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                }
+            }
+            __syncthreads();
+            if (!sm_last) return;
+            v = 0.f;
+            if (tid < 256)
+                for (int p = 0; p < k_parts; ++p)
+                    v += __hip_atomic_load(&sums[p * 256 + tid], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+        if (ep_ok) {
             v += ep_bias;
             if (mode == EPI_ADD_RESIDUAL) static_cast<float*>(C)[ep_idx] = ep_old + v;
             else epilogue<bf16_t>(mode, v, 0.f, C, ep_idx);
@@ -565,10 +601,15 @@ gemm_bf16_skinny(const void* __restrict__ Ain, int lda, const bf16_t* __restrict
     }
 }
 
+constexpr int SPLIT_COUNTERS = 4096;      // tiles that may be shared by several workgroups
+constexpr int SPLIT_MAX_PARTS = 8;
+constexpr int SPLIT_MIN_K_BLOCKS = 12;    // k blocks of 64 elements that every part keeps at least
+constexpr int SPLIT_FROM_K_BLOCKS = 80;   // shorter K: the fences cost more than the parallelism gains (measured)
+
 template <bool LN_FUSED>
 static int launch_skinny(const void* A, int lda, const bf16_t* W, int ldw, const float* bias, void* C, int ldc,
                          int M, int N, int K, int mode, const float* gamma, const float* beta, float eps,
-                         const int* rows, hipStream_t stream) {
+                         const int* rows, hipStream_t stream, void* workspace = nullptr, size_t workspace_bytes = 0) {
     const int tiles = (N + 15) / 16;
     const bool split_k = tiles < 1024;
     // Narrow products: 16 rows per workgroup and one workgroup per 16 rows (more workgroups, each
@@ -591,7 +632,22 @@ static int launch_skinny(const void* A, int lda, const bf16_t* W, int ldw, const
         staged_bytes = row16_bytes * mt;
     }
     int nw;
-    const int k_blocks = (K + 63) / 64;
+    int k_blocks = (K + 63) / 64;
+    // Narrow products with a long K (from SPLIT_FROM_K_BLOCKS blocks): k_parts workgroups per tile,
+    // as many as fit one round over the 256 compute units while each keeps at least
+    // SPLIT_MIN_K_BLOCKS k blocks. Needs the workspace: SPLIT_COUNTERS counters, then 256 floats
+    // per tile and part.
+    int k_parts = 1;
+    if (split_k && !LN_FUSED && workspace != nullptr && k_blocks >= SPLIT_FROM_K_BLOCKS) {
+        const int wgs = tiles * row_blocks;
+        k_parts = std::min(std::min(256 / std::max(wgs, 1), k_blocks / SPLIT_MIN_K_BLOCKS), SPLIT_MAX_PARTS);
+        if (k_parts < 2 || wgs > SPLIT_COUNTERS ||
+            workspace_bytes < SPLIT_COUNTERS * sizeof(int) + static_cast<size_t>(wgs) * k_parts * 256 * sizeof(float))
+            k_parts = 1;
+        k_blocks = (k_blocks + k_parts - 1) / k_parts;      // per workgroup from here on
+    }
+    int* part_counters = static_cast<int*>(workspace);
+    float* part_sums = reinterpret_cast<float*>(static_cast<char*>(workspace) + SPLIT_COUNTERS * sizeof(int));
     if (split_k) {
         // the wavefront count (at least 4: one thread per output of the tile) that leaves every
         // wavefront the fewest k blocks; among equals the smallest, which has the least to add up
@@ -606,7 +662,7 @@ static int launch_skinny(const void* A, int lda, const bf16_t* W, int ldw, const
         nw = nw < 4 ? 4 : (nw > 16 ? 16 : nw);
     }
     const int col_blocks = split_k ? tiles : (tiles + nw - 1) / nw;
-    const dim3 grid((col_blocks + N_XCD - 1) / N_XCD * N_XCD * row_blocks), block(nw * 64);
+    const dim3 grid((col_blocks + N_XCD - 1) / N_XCD * N_XCD * row_blocks, k_parts), block(nw * 64);
     size_t smem = split_k ? static_cast<size_t>(nw) * mt * 256 * sizeof(float) : 0;
     if (staged) {
 #define SKINNY_STAGED(MTV)                                                                             \
@@ -617,7 +673,7 @@ static int launch_skinny(const void* A, int lda, const bf16_t* W, int ldw, const
                                            static_cast<int>(staged_bytes));                            \
         if (e != hipSuccess) return static_cast<int>(e);                                               \
         kernel<<<grid, block, staged_bytes, stream>>>(A, lda, W, ldw, bias, C, ldc, M, N, K, mode, gamma, beta, \
-                                                      eps, rows, col_blocks, row_blocks);              \
+                                                      eps, rows, col_blocks, row_blocks, 1, nullptr, nullptr); \
         break;                                                                                         \
     }
         switch (mt) {
@@ -637,7 +693,8 @@ static int launch_skinny(const void* A, int lda, const bf16_t* W, int ldw, const
     constexpr int ASRC = LN_FUSED ? A_NORMED : A_GLOBAL;
 #define SKINNY_LAUNCH(SPLIT, UV)                                                                       \
     gemm_bf16_skinny<1, ASRC, SPLIT, UV><<<grid, block, smem, stream>>>(                               \
-        A, lda, W, ldw, bias, C, ldc, M, N, K, mode, gamma, beta, eps, rows, col_blocks, row_blocks)
+        A, lda, W, ldw, bias, C, ldc, M, N, K, mode, gamma, beta, eps, rows, col_blocks, row_blocks, k_parts,    \
+        part_sums, part_counters)
     if (split_k) {
         // a chunk holds all k blocks of a wavefront when they are at most 3 (two chunks of
         // fragments must fit the 128 registers of a 16-wavefront workgroup)
@@ -657,7 +714,8 @@ static int launch_skinny(const void* A, int lda, const bf16_t* W, int ldw, const
 
 
 static int gemm_bf16_dispatch(const void* A, int lda, const void* W, int ldw, const float* bias, void* C, int ldc,
-                              int M, int N, int K, int mode, hipStream_t stream, KvScatter kv) {
+                              int M, int N, int K, int mode, hipStream_t stream, KvScatter kv,
+                              void* workspace = nullptr, size_t workspace_bytes = 0) {
     if (M <= 0 || N <= 0) return 0;
     if (K % 8 != 0 || lda % 8 != 0 || ldw % 8 != 0) return -1;
     if ((reinterpret_cast<uintptr_t>(A) & 15) || (reinterpret_cast<uintptr_t>(W) & 15)) return -1;
@@ -665,7 +723,7 @@ static int gemm_bf16_dispatch(const void* A, int lda, const void* W, int ldw, co
     const bf16_t* w = static_cast<const bf16_t*>(W);
     const bool scatter = kv.slots != nullptr;       // only the many-row kernel scatters
     if (!scatter && M <= 64 && launch_skinny<false>(A, lda, w, ldw, bias, C, ldc, M, N, K, mode, nullptr, nullptr,
-                                                    0.f, nullptr, stream) == 0) {
+                                                    0.f, nullptr, stream, workspace, workspace_bytes) == 0) {
         // few rows: weight-streaming kernel
     } else if (M <= 32) {
         launch_tiled<1, 4, 1, 1, 64, 3>(a, lda, w, ldw, bias, C, ldc, M, N, K, mode, stream, kv);
@@ -693,10 +751,16 @@ extern "C" {
 
 // Returns 0, a HIP error code, or -1 when K or the row strides are not multiples of 8
 // elements or a base pointer is not 16-byte aligned.
+// `workspace` (optional; 4-byte aligned, zero when first handed over, never written by anyone else)
+// lets narrow products of few rows and a long K share a tile among several workgroups: 16 KB of
+// counters, then 1 KB per workgroup of such a launch (at most 256). Launches that use one
+// workspace must not overlap.
 int mllm_gemm_bf16(const void* A, int lda, const void* W, int ldw, const float* bias, void* C, int ldc,
-                   int M, int N, int K, int mode, hipStream_t stream) {
-    return gemm_bf16_dispatch(A, lda, W, ldw, bias, C, ldc, M, N, K, mode, stream, KvScatter{});
+                   int M, int N, int K, int mode, void* workspace, size_t workspace_bytes, hipStream_t stream) {
+    return gemm_bf16_dispatch(A, lda, W, ldw, bias, C, ldc, M, N, K, mode, stream, KvScatter{}, workspace,
+                              workspace_bytes);
 }
+
 
 // The plain bf16 store (mode 0) with the key/value scatter of KvScatter fused: C = A W^T + bias, and
 // columns [q_cols, q_cols + kv_dim) / [q_cols + kv_dim, q_cols + 2 kv_dim) of row m also go to row

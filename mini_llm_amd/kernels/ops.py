@@ -194,8 +194,10 @@ def linear(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], out: 
                                        M, N, K, _p(slots), _p(k_pages), _p(v_pages), int(q_cols), int(kv_dim),
                                        _stream())
         else:
+            ws = _gemm_workspace(a.device) if M <= 64 else None
             rc = lib.mllm_gemm_bf16(_p(a), a.stride(0), _p(w), w.stride(0), _p(bias), _p(out), out.stride(0),
-                                    M, N, K, mode, _stream())
+                                    M, N, K, mode, _p(ws), ctypes.c_size_t(GEMM_WORKSPACE_BYTES if M <= 64 else 0),
+                                    _stream())
         if rc == -1:
             raise KernelError(
                 f"linear(bf16): K={K} and the row strides ({a.stride(0)}, {w.stride(0)}) must be multiples "
@@ -204,6 +206,19 @@ def linear(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], out: 
         raise KernelError(f"linear: unsupported dtype {a.dtype}")
     _check(rc, "linear")
     return out
+
+
+GEMM_WORKSPACE_BYTES = 16 * 1024 + 256 * 1024     # counters, then 1 KB per workgroup of a shared-tile launch
+_GEMM_WS = {}
+
+
+def _gemm_workspace(device) -> torch.Tensor:
+    """Scratch of the few-row products that share a tile among workgroups: zeroed once per device
+    (the kernel leaves its counters at zero); launches on one stream use it one after the other."""
+    ws = _GEMM_WS.get(device)
+    if ws is None:
+        ws = _GEMM_WS[device] = torch.zeros(GEMM_WORKSPACE_BYTES // 4, dtype=torch.int32, device=device)
+    return ws
 
 
 LN_FUSE_MAX_ROWS = 16      # above this many rows the norm is faster as a kernel of its own (measured)

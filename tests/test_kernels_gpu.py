@@ -191,6 +191,42 @@ def test_linear_bf16_few_rows(ops, M, N, K):
         assert err <= (2e-5 + 2e-5 * math.sqrt(K) if f32_out else 4e-2), (epi, err)
 
 
+@pytest.mark.parametrize("M,N,K", [(8, 1600, 6400), (1, 1280, 5120), (16, 72, 8192), (5, 200, 5192), (32, 40, 6400),
+                                   (64, 24, 5128)])
+def test_linear_bf16_few_rows_long_k_shares_tiles(ops, M, N, K):
+    """Narrow products with a long K: several workgroups share a tile and the last to arrive adds their
+    parts. Every call gives the same bits (the parts are added in a fixed order, the counters are
+    left at zero), eagerly and in replays of a HIP graph."""
+    g = torch.Generator().manual_seed(M + N + K)
+    a = _rand((M, K), torch.bfloat16, g).to(DEV)
+    w = _rand((N, K), torch.bfloat16, g, std=1.0 / math.sqrt(K)).to(DEV)
+    bias = (0.5 * _rand((N,), torch.float32, g)).to(DEV)
+    x0 = _rand((M, N), torch.float32, g)
+    ref = plain_ops.linear(a.cpu(), w.cpu(), bias.cpu(), x0.double().clone(), "add_residual")
+    outs = []
+    for _ in range(3):
+        x = x0.clone().to(DEV)
+        ops.linear(a, w, bias, x, "add_residual")
+        outs.append(x.cpu())
+    assert (outs[0].double() - ref).abs().max().item() <= 2e-5 + 2e-5 * math.sqrt(K)
+    assert torch.equal(outs[0], outs[1]) and torch.equal(outs[0], outs[2])
+    x = x0.clone().to(DEV)
+    y = torch.empty(M, N, dtype=torch.bfloat16, device=DEV)
+    ops.linear(a, w, bias, y, "gelu_tanh")
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        ops.linear(a, w, bias, x, "add_residual")
+        ops.linear(a, w, bias, y, "gelu_tanh")
+    y_eager = y.cpu()
+    for _ in range(3):
+        x.copy_(x0)
+        y.zero_()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(x.cpu(), outs[0]) and torch.equal(y.cpu(), y_eager)
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("M,N,K", [(1, 2304, 768), (8, 3072, 768), (16, 320, 96), (5, 200, 1600), (17, 96, 64),
                                    (3, 64, 4096), (16, 6400, 1600), (9, 50257, 1024), (16, 3072, 1024), (33, 2304, 768),
