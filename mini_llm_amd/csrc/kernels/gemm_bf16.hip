@@ -276,10 +276,15 @@ static void launch_tiled(const bf16_t* a, int lda, const bf16_t* w, int ldw, con
 }
 
 // ---------------------------------------------------------------------------------------------
-// Few rows (decode): M <= 64. The product is bound by streaming W once. Each lane loads 16
-// contiguous bytes of a weight row straight from global memory into the B operand of
-// v_mfma_f32_16x16x32_bf16; a workgroup owns 16 rows of the output (more rows: more workgroups
-// per column range, placed on the same XCD so that the weights they share come from its L2).
+// Few rows (decode): M <= 64. The product is bound by streaming W once, and how fast a compute
+// unit streams depends on the shape of a wavefront's load: 8 consecutive lanes take one 128-byte
+// line (8 weight rows x 1 line per load) at up to 90 GB/s per unit, but the MFMA operand layout
+// (consecutive lanes = consecutive weight rows, 4 lines per 4 lanes) at under 40 (measured). So
+// the loads use the first shape and the 16-byte pieces change lanes through a 2 KB region of LDS
+// private to the wavefront (no barrier: LDS serves a wavefront's requests in order), swizzled so
+// that neither the writes nor the reads conflict. A workgroup owns 16 rows of the output (more
+// rows: more workgroups per column range, placed on the same XCD so that the weights they share
+// come from its L2).
 //   SPLIT_K:  one workgroup per 16-column tile, its wavefronts split K (wavefront w takes the
 //             64-element k blocks w, w+NW, ...) and their partial sums are added in LDS in a fixed
 //             order: for the narrow products, where tiles alone are too few to fill the chip.
@@ -298,8 +303,8 @@ typedef float f32x4 __attribute__((ext_vector_type(4)));
 
 enum { A_GLOBAL = 0, A_NORMED = 1, A_STAGED = 2 };
 
-template <int MT, int ASRC, bool SPLIT_K, int U>
-__global__ void __launch_bounds__(ASRC == A_NORMED ? 512 : 1024)
+template <int MT, int ASRC, bool SPLIT_K, int U, bool A_TWO = true>
+__global__ void __launch_bounds__(ASRC == A_NORMED ? 512 : (ASRC == A_GLOBAL ? 768 : 1024))
 gemm_bf16_skinny(const void* __restrict__ Ain, int lda, const bf16_t* __restrict__ W, int ldw,
                  const float* __restrict__ bias, void* __restrict__ C, int ldc, int M, int N, int K, int mode,
                  const float* __restrict__ gamma, const float* __restrict__ beta, float eps,
@@ -309,7 +314,11 @@ gemm_bf16_skinny(const void* __restrict__ Ain, int lda, const bf16_t* __restrict
     __shared__ int sm_last;
     constexpr bool LN_FUSED = ASRC == A_NORMED;
     constexpr bool IN_LDS = ASRC != A_GLOBAL;
-    const int tid = threadIdx.x, wave = tid / 64, lane = tid % 64;
+    // The wavefront's index as a scalar: what depends on it alone (its k blocks, whether it has a
+    // whole chunk, whether it owns outputs) then branches for real. Derived from threadIdx it would
+    // count as divergent, both sides of every such condition would run one after the other under
+    // masks, and loads pending from one side would be waited for on the other.
+    const int tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid / 64), lane = tid % 64;
     const int nw = blockDim.x / 64;
     const int row16 = lane % 16, kq = lane / 16;
     // workgroup id -> (column block, row block): the row blocks of one column block have ids that
@@ -319,22 +328,35 @@ gemm_bf16_skinny(const void* __restrict__ Ain, int lda, const bf16_t* __restrict
     if (cb >= col_blocks) return;
     const int m_base = rb * 16 * MT;
     const int n0 = (SPLIT_K ? cb : cb * nw + wave) * 16;
-    // K is dealt out in blocks of 64 elements, one 128-byte line of a weight row: lane group kq
-    // takes elements 16*kq .. 16*kq+15 of a block, the first 8 in one MFMA and the rest in the
-    // next (the k index of an MFMA may be permuted as long as both operands agree), so that a
-    // wavefront uses every line it touches whole.
+    // K is dealt out in blocks of 64 elements, one 128-byte line of a weight row. In the MFMAs
+    // lane group kq takes elements 16*kq .. 16*kq+15 of a block, the first 8 in one MFMA and the
+    // rest in the next (the k index of an MFMA may be permuted as long as both operands agree).
     // (with k_parts workgroups on the tile, over all their wavefronts alike)
     const int part = SPLIT_K ? blockIdx.y : 0;
     const int k_first = SPLIT_K ? (part * nw + wave) * 64 : 0;      // first k block of this wavefront
     const int k_stride = SPLIT_K ? nw * k_parts * 64 : 64;         // distance between its k blocks
     const size_t red_bytes = SPLIT_K ? static_cast<size_t>(nw) * MT * 256 * sizeof(float) : 0;
+    constexpr int STAGE_BYTES = ASRC == A_GLOBAL ? 4096 : 2048;            // per wavefront: W block (+ A block)
     float* red = reinterpret_cast<float*>(smem_raw);                       // [nw][MT][256]
-    bf16_t* a_s = reinterpret_cast<bf16_t*>(smem_raw + red_bytes);         // [16*MT][K+8]
+    bf16x8* stage_w = reinterpret_cast<bf16x8*>(smem_raw + red_bytes + static_cast<size_t>(wave) * STAGE_BYTES);
+    bf16x8* stage_a = stage_w + 128;                                       // (A_GLOBAL only)
+    bf16_t* a_s = reinterpret_cast<bf16_t*>(smem_raw + red_bytes + static_cast<size_t>(nw) * STAGE_BYTES);   // [16*MT][K+8]
     const int a_stride = K + 8;
     const int n = n0 + row16;
     const bool n_ok = n < N;
-    const bf16_t* wrow = W + static_cast<size_t>(n_ok ? n : 0) * ldw;
     const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
+    // Loads: lane -> (row lr = lane / 8 of 8, 16-byte piece lane % 8 of the row's 128-byte line);
+    // two loads cover the tile's 16 rows. The piece a lane fetches is its slot number XORed with a
+    // swizzle of the row (the row modulo 8, its lowest bit flipped for rows 8..15), so that slot s
+    // of row r, written to LDS lane-linearly, holds piece s ^ swizzle(r): then the 16 lanes of an
+    // operand read (rows 0..15, one piece number) fall on 16 different 16-byte bank groups.
+    const int lr = lane / 8;
+    const int piece[2] = {(lane % 8) ^ lr, (lane % 8) ^ lr ^ 1};
+    const bf16_t* wrow[2];
+#pragma unroll
+    for (int j = 0; j < 2; ++j) wrow[j] = W + static_cast<size_t>(min(n0 + lr + 8 * j, N - 1)) * ldw;
+    // reads: this lane's MFMA row/column is row16; for MFMA step `half` it wants piece 2*kq + half
+    const int rd_swz = row16 < 8 ? row16 : ((row16 - 8) ^ 1);
 
     f32x4 acc[MT];
 #pragma unroll
@@ -345,15 +367,13 @@ gemm_bf16_skinny(const void* __restrict__ Ain, int lda, const bf16_t* __restrict
     bool ep_ok = false;
     size_t ep_idx = 0;
     float ep_bias = 0.f, ep_old = 0.f;
-    if (SPLIT_K && MT == 1 && tid < 256) {
-        const int r = tid / 64, l = tid % 64;
-        const int m = m_base + 4 * (l / 16) + r, nn = n0 + l % 16;
+    if (SPLIT_K && MT == 1 && wave < 4) {
+        // (loads without a per-lane condition: outputs beyond M or N read the last row or column)
+        const int m = m_base + 4 * (lane / 16) + wave, nn = n0 + lane % 16;
         ep_ok = m < M && nn < N;
-        if (ep_ok) {
-            ep_idx = static_cast<size_t>(m) * ldc + nn;
-            if (bias) ep_bias = bias[nn];
-            if (mode == EPI_ADD_RESIDUAL) ep_old = static_cast<const float*>(C)[ep_idx];
-        }
+        ep_idx = static_cast<size_t>(min(m, M - 1)) * ldc + min(nn, N - 1);
+        if (bias) ep_bias = bias[min(nn, N - 1)];
+        if (mode == EPI_ADD_RESIDUAL) ep_old = static_cast<const float*>(C)[ep_idx];
     }
 
     // A wavefront takes its k blocks in chunks of H = U/2. All loads of a chunk are issued
@@ -368,33 +388,60 @@ gemm_bf16_skinny(const void* __restrict__ Ain, int lda, const bf16_t* __restrict
     constexpr int H = U / 2;
     static_assert(U % 2 == 0, "whole k blocks per chunk");
     const bf16_t* A = static_cast<const bf16_t*>(Ain);
-    const bf16_t* arow = A;       // A_GLOBAL: this lane's row of A (rows beyond M: the last one, never stored)
-    if (ASRC == A_GLOBAL) arow = A + static_cast<size_t>(min(m_base + row16, M - 1)) * lda;
+    // A_GLOBAL: the rows of A travel like the weights (rows beyond M: the last one, never stored);
+    // a workgroup with at most 8 rows needs one load per k block
+    const bf16_t* arow[2] = {A, A};
+    // (A_TWO false: the launcher knows that M <= 8, and the chunks keep half the registers for A)
+    const bool a_two = A_TWO && M - m_base > 8;
+    if (ASRC == A_GLOBAL) {
+#pragma unroll
+        for (int j = 0; j < 2; ++j) arow[j] = A + static_cast<size_t>(min(m_base + lr + 8 * j, M - 1)) * lda;
+    }
     const int n_blocks = k_first < K ? (K - k_first + k_stride - 1) / k_stride : 0;   // of this wavefront
     const int n_chunks = n_blocks / H;
     struct Chunk {
         bf16x8 b[U];
-        bf16x8 a[ASRC == A_GLOBAL ? U : 1];
+        bf16x8 a[ASRC == A_GLOBAL ? (A_TWO ? U : U / 2) : 1];
     };
-    auto load_steps = [&](Chunk& c, int u0, int k0) {      // the two steps of the k block at k0 into slots u0, u0+1
+    auto load_steps = [&](Chunk& c, int u0, int k0) {      // the k block at k0 (rows 0..7, rows 8..15) into slots u0, u0+1
 #pragma unroll
-        for (int half = 0; half < 2; ++half) {
-            const int k = min(k0 + 16 * kq + 8 * half, K - 8);
-            c.b[u0 + half] = *reinterpret_cast<const bf16x8*>(wrow + k);
-            if (ASRC == A_GLOBAL) c.a[u0 + half] = *reinterpret_cast<const bf16x8*>(arow + k);
+        for (int j = 0; j < 2; ++j) {
+            const int k = min(k0 + 8 * piece[j], K - 8);
+            c.b[u0 + j] = *reinterpret_cast<const bf16x8*>(wrow[j] + k);
+            if (ASRC == A_GLOBAL && (j == 0 || a_two)) c.a[A_TWO ? u0 + j : u0 / 2] = *reinterpret_cast<const bf16x8*>(arow[j] + k);
         }
     };
     auto mma_steps = [&](const Chunk& c, int u0, int k0) {
+        // through the wavefront's LDS region into the operand layout
+        stage_w[lane] = c.b[u0];
+        stage_w[64 + lane] = c.b[u0 + 1];
+        if (ASRC == A_GLOBAL) {
+            stage_a[lane] = c.a[A_TWO ? u0 : u0 / 2];
+            if (a_two) stage_a[64 + lane] = c.a[A_TWO ? u0 + 1 : 0];
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        bf16x8 bf[2], af[2];
+#pragma unroll
+        for (int half = 0; half < 2; ++half) {
+            const int p = 2 * kq + half;
+            bf[half] = stage_w[row16 * 8 + (p ^ rd_swz)];
+            if (ASRC == A_GLOBAL) af[half] = stage_a[row16 * 8 + (p ^ rd_swz)];
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 #pragma unroll
         for (int half = 0; half < 2; ++half) {
             const int k = k0 + 16 * kq + 8 * half;
-            const bf16x8 b = k < K ? c.b[u0 + half] : zero;
+            const bf16x8 b = k < K ? bf[half] : zero;
             const int kc = min(k, K - 8);
 #pragma unroll
             for (int i = 0; i < MT; ++i) {
                 bf16x8 a;
                 if (IN_LDS) a = *reinterpret_cast<const bf16x8*>(a_s + static_cast<size_t>(i * 16 + row16) * a_stride + kc);
-                else a = c.a[u0 + half];
+                else a = af[half];
                 acc[i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, acc[i], 0, 0, 0);
             }
         }
@@ -432,6 +479,30 @@ gemm_bf16_skinny(const void* __restrict__ Ain, int lda, const bf16_t* __restrict
         if (n_chunks > 0) load_chunk(c0, 0);
         else load_left();                                   // a wavefront without a whole chunk starts with these
     };
+    // The fused norm's operands are requested before the weights: loads return in the order of
+    // their requests, so the norm (whose rows come from L2) can be computed while the weights are
+    // still on their way from memory, which it could not if it had to wait for them first.
+    const int nq = K / 4, n_u = (nq + 63) / 64;       // float4 per row; per lane (uniform)
+    float4 gg[8], bb[8], v[2][8];
+    // whether this wavefront's two rows exist is uniform over it: rows beyond M are not read
+    const bool row_ok[2] = {m_base + wave < M, m_base + wave + 8 < M};
+    if (LN_FUSED) {
+        const float* x = static_cast<const float*>(Ain);
+        const float4* g4 = reinterpret_cast<const float4*>(gamma);
+        const float4* b4 = reinterpret_cast<const float4*>(beta);
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            if (u < n_u) {
+                const int i = min(lane + 64 * u, nq - 1);
+                gg[u] = g4[i];
+                bb[u] = beta ? b4[i] : make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+                for (int j = 0; j < 2; ++j)
+                    if (row_ok[j]) v[j][u] = reinterpret_cast<const float4*>(x + static_cast<size_t>(src_row[j]) * lda)[i];
+            }
+        }
+        __builtin_amdgcn_sched_barrier(0);
+    }
     first_loads();
     if (ASRC == A_STAGED) {
         // the workgroup's rows of A, copied once into LDS for all its wavefronts
@@ -458,26 +529,7 @@ gemm_bf16_skinny(const void* __restrict__ Ain, int lda, const bf16_t* __restrict
     }
     if (LN_FUSED) {
         // 8 wavefronts, two rows each; a row lives in registers (K <= 2048, K % 4 == 0): mean,
-        // then variance of the centred values, all in fp32. Both rows and the scale and shift
-        // vectors are requested together, before anything is waited for.
-        const float* x = static_cast<const float*>(Ain);
-        const int nq = K / 4, n_u = (nq + 63) / 64;       // float4 per row; per lane (uniform)
-        const float4* g4 = reinterpret_cast<const float4*>(gamma);
-        const float4* b4 = reinterpret_cast<const float4*>(beta);
-        float4 gg[8], bb[8], v[2][8];
-        // whether this wavefront's two rows exist is uniform over it: rows beyond M are not read
-        const bool row_ok[2] = {m_base + wave < M, m_base + wave + 8 < M};
-#pragma unroll
-        for (int u = 0; u < 8; ++u) {
-            if (u < n_u) {
-                const int i = min(lane + 64 * u, nq - 1);
-                gg[u] = g4[i];
-                bb[u] = beta ? b4[i] : make_float4(0.f, 0.f, 0.f, 0.f);
-#pragma unroll
-                for (int j = 0; j < 2; ++j)
-                    if (row_ok[j]) v[j][u] = reinterpret_cast<const float4*>(x + static_cast<size_t>(src_row[j]) * lda)[i];
-            }
-        }
+        // then variance of the centred values, all in fp32.
 #pragma unroll
         for (int j = 0; j < 2; ++j) {
             const int m = wave + 8 * j;
@@ -601,6 +653,7 @@ gemm_bf16_skinny(const void* __restrict__ Ain, int lda, const bf16_t* __restrict
     }
 }
 
+constexpr int MAX_DYNAMIC_LDS = 160 * 1024 - 1024;      // the unit's LDS less the kernel's static variables
 constexpr int SPLIT_COUNTERS = 4096;      // tiles that may be shared by several workgroups
 constexpr int SPLIT_MAX_PARTS = 8;
 constexpr int SPLIT_MIN_K_BLOCKS = 12;    // k blocks of 64 elements that every part keeps at least
@@ -624,7 +677,7 @@ static int launch_skinny(const void* A, int lda, const bf16_t* W, int ldw, const
     size_t staged_bytes = 0;
     if (staged) {
         const size_t row16_bytes = static_cast<size_t>(16) * (K + 8) * sizeof(bf16_t);
-        int fit = static_cast<int>(160 * 1024 / row16_bytes);
+        int fit = static_cast<int>((160 - 32) * 1024 / row16_bytes);      // 32 KB: the wavefronts' transposition regions
         if (fit < 1) return -2;
         if (fit > 4) fit = 4;
         row_blocks = (mt + fit - 1) / fit;
@@ -652,8 +705,10 @@ static int launch_skinny(const void* A, int lda, const bf16_t* W, int ldw, const
         // the wavefront count (at least 4: one thread per output of the tile) that leaves every
         // wavefront the fewest k blocks; among equals the smallest, which has the least to add up
         // (the fused norm is written for 8 wavefronts, two rows each)
+        // (at most 12: two chunks of loads in flight per wavefront need more than the 128 registers
+        // that 16 wavefronts would leave each)
         nw = 4;
-        for (int cand = 5; cand <= 16; ++cand)
+        for (int cand = 5; cand <= 12; ++cand)
             if ((k_blocks + cand - 1) / cand < (k_blocks + nw - 1) / nw) nw = cand;
         if (LN_FUSED) nw = 8;
     } else {
@@ -664,7 +719,9 @@ static int launch_skinny(const void* A, int lda, const bf16_t* W, int ldw, const
     const int col_blocks = split_k ? tiles : (tiles + nw - 1) / nw;
     const dim3 grid((col_blocks + N_XCD - 1) / N_XCD * N_XCD * row_blocks, k_parts), block(nw * 64);
     size_t smem = split_k ? static_cast<size_t>(nw) * mt * 256 * sizeof(float) : 0;
+    smem += static_cast<size_t>(nw) * (LN_FUSED || staged ? 2048 : 4096);     // the wavefronts' transposition regions
     if (staged) {
+        staged_bytes += smem;
 #define SKINNY_STAGED(MTV)                                                                             \
     case MTV: {                                                                                        \
         auto kernel = gemm_bf16_skinny<MTV, A_STAGED, false, 4>;                                        \
@@ -689,19 +746,45 @@ static int launch_skinny(const void* A, int lda, const bf16_t* W, int ldw, const
             (reinterpret_cast<uintptr_t>(gamma) & 15) || (reinterpret_cast<uintptr_t>(beta) & 15))
             return -2;
     }
-    if (smem > 64 * 1024) return -2;
+    if (smem > MAX_DYNAMIC_LDS) return -2;
     constexpr int ASRC = LN_FUSED ? A_NORMED : A_GLOBAL;
-#define SKINNY_LAUNCH(SPLIT, UV)                                                                       \
-    gemm_bf16_skinny<1, ASRC, SPLIT, UV><<<grid, block, smem, stream>>>(                               \
-        A, lda, W, ldw, bias, C, ldc, M, N, K, mode, gamma, beta, eps, rows, col_blocks, row_blocks, k_parts,    \
-        part_sums, part_counters)
+#define SKINNY_LAUNCH(SPLIT, UV, A2)                                                                   \
+    do {                                                                                               \
+        auto kernel = gemm_bf16_skinny<1, ASRC, SPLIT, UV, A2>;                                        \
+        static bool lds_allowed = false;      /* more than 64 KB of dynamic LDS has to be asked for once */ \
+        if (!lds_allowed) {                                                                            \
+            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),                  \
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, MAX_DYNAMIC_LDS); \
+            if (e != hipSuccess) return static_cast<int>(e);                                           \
+            lds_allowed = true;                                                                        \
+        }                                                                                              \
+        kernel<<<grid, block, smem, stream>>>(A, lda, W, ldw, bias, C, ldc, M, N, K, mode, gamma, beta, eps, rows, \
+                                              col_blocks, row_blocks, k_parts, part_sums, part_counters); \
+    } while (0)
     if (split_k) {
-        // a chunk holds all k blocks of a wavefront when they are at most 3 (two chunks of
-        // fragments must fit the 128 registers of a 16-wavefront workgroup)
-        switch (std::min((k_blocks + nw - 1) / nw, 3)) {
-            case 1: SKINNY_LAUNCH(true, 2); break;
-            case 2: SKINNY_LAUNCH(true, 4); break;
-            default: SKINNY_LAUNCH(true, 6); break;
+        // a chunk holds all k blocks of a wavefront when they are at most 3 (4 without the fused
+        // norm and with at most 8 rows; with more rows A takes two loads per block and 3 blocks
+        // are the most): two chunks of fragments must fit the registers
+        const int per_wave = (k_blocks + nw - 1) / nw;
+        if (LN_FUSED) {
+            switch (std::min(per_wave, 3)) {
+                case 1: SKINNY_LAUNCH(true, 2, false); break;
+                case 2: SKINNY_LAUNCH(true, 4, false); break;
+                default: SKINNY_LAUNCH(true, 6, false); break;
+            }
+        } else if (M <= 8) {
+            switch (std::min(per_wave, 4)) {
+                case 1: SKINNY_LAUNCH(true, 2, false); break;
+                case 2: SKINNY_LAUNCH(true, 4, false); break;
+                case 3: SKINNY_LAUNCH(true, 6, false); break;
+                default: SKINNY_LAUNCH(true, 8, false); break;
+            }
+        } else {
+            switch (std::min(per_wave, 3)) {
+                case 1: SKINNY_LAUNCH(true, 2, true); break;
+                case 2: SKINNY_LAUNCH(true, 4, true); break;
+                default: SKINNY_LAUNCH(true, 6, true); break;
+            }
         }
     } else {
         // wide products (the logits head): normalising the rows once in a kernel of its own and
