@@ -150,8 +150,7 @@ decode_attention_kernel(const T* __restrict__ q, int q_stride, int q_col,
             float d = 0.f;
 #pragma unroll
             for (int e = 0; e < EPL; ++e) d = fmaf(qf[e], kf[e], d);
-#pragma unroll
-            for (int off = 1; off < LPK; off <<= 1) d += __shfl_xor(d, off, MLLM_WAVE);
+            d = group_sum<LPK>(d);
             const bool valid = j0 + u * n_waves * KPW + g < ke_pages;
             dot[u] = valid ? d : NEG;
             mx = fmaxf(mx, dot[u]);
@@ -180,8 +179,7 @@ decode_attention_kernel(const T* __restrict__ q, int q_stride, int q_col,
         float d = 0.f;
 #pragma unroll
         for (int e = 0; e < EPL; ++e) d = fmaf(qf[e], kf[e], d);
-#pragma unroll
-        for (int off = 1; off < LPK; off <<= 1) d += __shfl_xor(d, off, MLLM_WAVE);
+        d = group_sum<LPK>(d);
         const float mn = fmaxf(m, d);
         const float a = fast_exp2(m - mn), pj = fast_exp2(d - mn);
         l = l * a + pj;

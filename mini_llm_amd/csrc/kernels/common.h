@@ -64,15 +64,48 @@ __device__ __forceinline__ void load8(const bf16_t* p, float (&v)[8]) {
     v[6] = __uint_as_float(a.w << 16); v[7] = __uint_as_float(a.w & 0xffff0000u);
 }
 
-__device__ __forceinline__ float wave_sum(float v) {
-#pragma unroll
-    for (int off = MLLM_WAVE / 2; off > 0; off >>= 1) v += __shfl_xor(v, off, MLLM_WAVE);
+// Reductions over the 64 lanes of a wavefront; every lane gets the same result. Within a row of
+// 16 lanes the values move through the DPP path of the vector ALU (lane swaps inside quads, then
+// the mirrored half row and the mirrored row: after each step all lanes of the growing group hold
+// the group's result, since the operation is commutative), the four row results are read as
+// scalars. A shuffle through LDS (__shfl_xor) has several times the latency per step.
+template <int CTRL>
+__device__ __forceinline__ float dpp_move(float v) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xF, 0xF, false));
+}
+constexpr int DPP_SWAP_1 = 0xB1;          // quad_perm:[1,0,3,2]
+constexpr int DPP_SWAP_2 = 0x4E;          // quad_perm:[2,3,0,1]
+constexpr int DPP_HALF_MIRROR = 0x141;    // lane i <-> 7 - i within 8
+constexpr int DPP_ROW_MIRROR = 0x140;     // lane i <-> 15 - i within 16
+__device__ __forceinline__ float row_lane(float v, int lane) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), lane));
+}
+// Sum over aligned groups of LANES consecutive lanes (a power of two), in every lane of the group.
+template <int LANES>
+__device__ __forceinline__ float group_sum(float v) {
+    static_assert(LANES >= 1 && LANES <= MLLM_WAVE && (LANES & (LANES - 1)) == 0, "a power of two up to the wavefront");
+    if (LANES >= 2) v += dpp_move<DPP_SWAP_1>(v);
+    if (LANES >= 4) v += dpp_move<DPP_SWAP_2>(v);
+    if (LANES >= 8) v += dpp_move<DPP_HALF_MIRROR>(v);
+    if (LANES >= 16) v += dpp_move<DPP_ROW_MIRROR>(v);
+    if (LANES >= 32) v += __shfl_xor(v, 16, MLLM_WAVE);
+    if (LANES >= 64) v += __shfl_xor(v, 32, MLLM_WAVE);
     return v;
 }
+__device__ __forceinline__ float wave_sum(float v) {
+    static_assert(MLLM_WAVE == 64, "four rows of 16 lanes");
+    v += dpp_move<DPP_SWAP_1>(v);
+    v += dpp_move<DPP_SWAP_2>(v);
+    v += dpp_move<DPP_HALF_MIRROR>(v);
+    v += dpp_move<DPP_ROW_MIRROR>(v);
+    return (row_lane(v, 0) + row_lane(v, 16)) + (row_lane(v, 32) + row_lane(v, 48));
+}
 __device__ __forceinline__ float wave_max(float v) {
-#pragma unroll
-    for (int off = MLLM_WAVE / 2; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, MLLM_WAVE));
-    return v;
+    v = fmaxf(v, dpp_move<DPP_SWAP_1>(v));
+    v = fmaxf(v, dpp_move<DPP_SWAP_2>(v));
+    v = fmaxf(v, dpp_move<DPP_HALF_MIRROR>(v));
+    v = fmaxf(v, dpp_move<DPP_ROW_MIRROR>(v));
+    return fmaxf(fmaxf(row_lane(v, 0), row_lane(v, 16)), fmaxf(row_lane(v, 32), row_lane(v, 48)));
 }
 
 // Orders LDS traffic between the lanes of ONE wavefront (which run in lockstep):

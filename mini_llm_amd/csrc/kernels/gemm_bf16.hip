@@ -490,15 +490,23 @@ gemm_bf16_skinny(const void* __restrict__ Ain, int lda, const bf16_t* __restrict
         const float* x = static_cast<const float*>(Ain);
         const float4* g4 = reinterpret_cast<const float4*>(gamma);
         const float4* b4 = reinterpret_cast<const float4*>(beta);
+        // (the rows first: they come from L2, and their mean and variance need nothing else)
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            if (u < n_u) {
+                const int i = min(lane + 64 * u, nq - 1);
+#pragma unroll
+                for (int j = 0; j < 2; ++j)
+                    if (row_ok[j]) v[j][u] = reinterpret_cast<const float4*>(x + static_cast<size_t>(src_row[j]) * lda)[i];
+            }
+        }
+        __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int u = 0; u < 8; ++u) {
             if (u < n_u) {
                 const int i = min(lane + 64 * u, nq - 1);
                 gg[u] = g4[i];
                 bb[u] = beta ? b4[i] : make_float4(0.f, 0.f, 0.f, 0.f);
-#pragma unroll
-                for (int j = 0; j < 2; ++j)
-                    if (row_ok[j]) v[j][u] = reinterpret_cast<const float4*>(x + static_cast<size_t>(src_row[j]) * lda)[i];
             }
         }
         __builtin_amdgcn_sched_barrier(0);
