@@ -303,13 +303,19 @@ typedef float f32x4 __attribute__((ext_vector_type(4)));
 
 enum { A_GLOBAL = 0, A_NORMED = 1, A_STAGED = 2 };
 
-template <int MT, int ASRC, bool SPLIT_K, int U, bool A_TWO = true>
+template <int MT, int ASRC, bool SPLIT_K, int U, bool A_TWO = true, int NT = 1>
 __global__ void __launch_bounds__(ASRC == A_NORMED ? 512 : (ASRC == A_GLOBAL ? 768 : 1024))
 gemm_bf16_skinny(const void* __restrict__ Ain, int lda, const bf16_t* __restrict__ W, int ldw,
                  const float* __restrict__ bias, void* __restrict__ C, int ldc, int M, int N, int K, int mode,
                  const float* __restrict__ gamma, const float* __restrict__ beta, float eps,
-                 const int* __restrict__ rows, int col_blocks, int row_blocks, int k_parts,
+                 const int* __restrict__ rows, int col_blocks, int row_blocks, int cols_per_wg, int k_parts,
                  float* __restrict__ part_sums, int* __restrict__ part_counters) {
+    // NT > 1 (SPLIT_K, MT == 1): the workgroup owns cols_per_wg <= 16 NT columns, NT tiles that share
+    // the rows of A, the last one possibly narrower: for products with more than 256 tiles, whose
+    // columns are dealt out evenly to 256 workgroups (one per compute unit; a kernel of this size
+    // keeps one workgroup per unit, so 400 one-tile workgroups would take two rounds).
+    static_assert(NT == 1 || (MT == 1 && SPLIT_K), "column tiles per workgroup: split-K kernels of one row tile");
+    constexpr int T = MT * NT;      // accumulators: row tiles (NT == 1) or column tiles (MT == 1)
     extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
     __shared__ int sm_last;
     constexpr bool LN_FUSED = ASRC == A_NORMED;
@@ -327,7 +333,7 @@ gemm_bf16_skinny(const void* __restrict__ Ain, int lda, const bf16_t* __restrict
     const int cb = (g / (N_XCD * row_blocks)) * N_XCD + g % N_XCD, rb = (g / N_XCD) % row_blocks;
     if (cb >= col_blocks) return;
     const int m_base = rb * 16 * MT;
-    const int n0 = (SPLIT_K ? cb : cb * nw + wave) * 16;
+    const int n0 = SPLIT_K ? cb * cols_per_wg : (cb * nw + wave) * 16;
     // K is dealt out in blocks of 64 elements, one 128-byte line of a weight row. In the MFMAs
     // lane group kq takes elements 16*kq .. 16*kq+15 of a block, the first 8 in one MFMA and the
     // rest in the next (the k index of an MFMA may be permuted as long as both operands agree).
@@ -335,9 +341,9 @@ gemm_bf16_skinny(const void* __restrict__ Ain, int lda, const bf16_t* __restrict
     const int part = SPLIT_K ? blockIdx.y : 0;
     const int k_first = SPLIT_K ? (part * nw + wave) * 64 : 0;      // first k block of this wavefront
     const int k_stride = SPLIT_K ? nw * k_parts * 64 : 64;         // distance between its k blocks
-    const size_t red_bytes = SPLIT_K ? static_cast<size_t>(nw) * MT * 256 * sizeof(float) : 0;
+    const size_t red_bytes = SPLIT_K ? static_cast<size_t>(nw) * T * 256 * sizeof(float) : 0;
     constexpr int STAGE_BYTES = ASRC == A_GLOBAL ? 4096 : 2048;            // per wavefront: W block (+ A block)
-    float* red = reinterpret_cast<float*>(smem_raw);                       // [nw][MT][256]
+    float* red = reinterpret_cast<float*>(smem_raw);                       // [nw][T][256]
     bf16x8* stage_w = reinterpret_cast<bf16x8*>(smem_raw + red_bytes + static_cast<size_t>(wave) * STAGE_BYTES);
     bf16x8* stage_a = stage_w + 128;                                       // (A_GLOBAL only)
     bf16_t* a_s = reinterpret_cast<bf16_t*>(smem_raw + red_bytes + static_cast<size_t>(nw) * STAGE_BYTES);   // [16*MT][K+8]
@@ -352,28 +358,38 @@ gemm_bf16_skinny(const void* __restrict__ Ain, int lda, const bf16_t* __restrict
     // operand read (rows 0..15, one piece number) fall on 16 different 16-byte bank groups.
     const int lr = lane / 8;
     const int piece[2] = {(lane % 8) ^ lr, (lane % 8) ^ lr ^ 1};
-    const bf16_t* wrow[2];
+    // (columns beyond the workgroup's or the matrix's: the last valid one, never stored)
+    const bf16_t* wrow[NT][2];
 #pragma unroll
-    for (int j = 0; j < 2; ++j) wrow[j] = W + static_cast<size_t>(min(n0 + lr + 8 * j, N - 1)) * ldw;
+    for (int t = 0; t < NT; ++t)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+            wrow[t][j] = W + static_cast<size_t>(min(n0 + min(16 * t + lr + 8 * j, cols_per_wg - 1), N - 1)) * ldw;
     // reads: this lane's MFMA row/column is row16; for MFMA step `half` it wants piece 2*kq + half
     const int rd_swz = row16 < 8 ? row16 : ((row16 - 8) ^ 1);
 
-    f32x4 acc[MT];
+    f32x4 acc[T];
 #pragma unroll
-    for (int i = 0; i < MT; ++i) acc[i] = f32x4{0.f, 0.f, 0.f, 0.f};
+    for (int i = 0; i < T; ++i) acc[i] = f32x4{0.f, 0.f, 0.f, 0.f};
 
     // Split-K epilogue operands (thread tid < 256 owns output element tid of the 16x16 tile, in
     // accumulator order): requested now so that their latency hides behind the product.
-    bool ep_ok = false;
-    size_t ep_idx = 0;
-    float ep_bias = 0.f, ep_old = 0.f;
+    bool ep_ok[NT];
+    size_t ep_idx[NT];
+    float ep_bias[NT], ep_old[NT];
+#pragma unroll
+    for (int t = 0; t < NT; ++t) { ep_ok[t] = false; ep_idx[t] = 0; ep_bias[t] = 0.f; ep_old[t] = 0.f; }
     if (SPLIT_K && MT == 1 && wave < 4) {
         // (loads without a per-lane condition: outputs beyond M or N read the last row or column)
-        const int m = m_base + 4 * (lane / 16) + wave, nn = n0 + lane % 16;
-        ep_ok = m < M && nn < N;
-        ep_idx = static_cast<size_t>(min(m, M - 1)) * ldc + min(nn, N - 1);
-        if (bias) ep_bias = bias[min(nn, N - 1)];
-        if (mode == EPI_ADD_RESIDUAL) ep_old = static_cast<const float*>(C)[ep_idx];
+        const int m = m_base + 4 * (lane / 16) + wave;
+#pragma unroll
+        for (int t = 0; t < NT; ++t) {
+            const int ct = 16 * t + lane % 16, nn = n0 + ct;
+            ep_ok[t] = m < M && nn < N && ct < cols_per_wg;
+            ep_idx[t] = static_cast<size_t>(min(m, M - 1)) * ldc + min(nn, N - 1);
+            if (bias) ep_bias[t] = bias[min(nn, N - 1)];
+            if (mode == EPI_ADD_RESIDUAL) ep_old[t] = static_cast<const float*>(C)[ep_idx[t]];
+        }
     }
 
     // A wavefront takes its k blocks in chunks of H = U/2. All loads of a chunk are issued
@@ -400,49 +416,54 @@ gemm_bf16_skinny(const void* __restrict__ Ain, int lda, const bf16_t* __restrict
     const int n_blocks = k_first < K ? (K - k_first + k_stride - 1) / k_stride : 0;   // of this wavefront
     const int n_chunks = n_blocks / H;
     struct Chunk {
-        bf16x8 b[U];
+        bf16x8 b[NT][U];
         bf16x8 a[ASRC == A_GLOBAL ? (A_TWO ? U : U / 2) : 1];
     };
     auto load_steps = [&](Chunk& c, int u0, int k0) {      // the k block at k0 (rows 0..7, rows 8..15) into slots u0, u0+1
 #pragma unroll
         for (int j = 0; j < 2; ++j) {
             const int k = min(k0 + 8 * piece[j], K - 8);
-            c.b[u0 + j] = *reinterpret_cast<const bf16x8*>(wrow[j] + k);
+#pragma unroll
+            for (int t = 0; t < NT; ++t) c.b[t][u0 + j] = *reinterpret_cast<const bf16x8*>(wrow[t][j] + k);
             if (ASRC == A_GLOBAL && (j == 0 || a_two)) c.a[A_TWO ? u0 + j : u0 / 2] = *reinterpret_cast<const bf16x8*>(arow[j] + k);
         }
     };
+    auto wave_lds_order = [&]() {       // orders the wavefront's own LDS writes and reads (no instruction)
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    };
     auto mma_steps = [&](const Chunk& c, int u0, int k0) {
         // through the wavefront's LDS region into the operand layout
-        stage_w[lane] = c.b[u0];
-        stage_w[64 + lane] = c.b[u0 + 1];
+        bf16x8 af[2];
         if (ASRC == A_GLOBAL) {
             stage_a[lane] = c.a[A_TWO ? u0 : u0 / 2];
             if (a_two) stage_a[64 + lane] = c.a[A_TWO ? u0 + 1 : 0];
+            wave_lds_order();
+#pragma unroll
+            for (int half = 0; half < 2; ++half) af[half] = stage_a[row16 * 8 + ((2 * kq + half) ^ rd_swz)];
         }
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-        __builtin_amdgcn_wave_barrier();
-        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-        bf16x8 bf[2], af[2];
 #pragma unroll
-        for (int half = 0; half < 2; ++half) {
-            const int p = 2 * kq + half;
-            bf[half] = stage_w[row16 * 8 + (p ^ rd_swz)];
-            if (ASRC == A_GLOBAL) af[half] = stage_a[row16 * 8 + (p ^ rd_swz)];
-        }
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-        __builtin_amdgcn_wave_barrier();
-        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        for (int t = 0; t < NT; ++t) {
+            stage_w[lane] = c.b[t][u0];
+            stage_w[64 + lane] = c.b[t][u0 + 1];
+            wave_lds_order();
+            bf16x8 bf[2];
 #pragma unroll
-        for (int half = 0; half < 2; ++half) {
-            const int k = k0 + 16 * kq + 8 * half;
-            const bf16x8 b = k < K ? bf[half] : zero;
-            const int kc = min(k, K - 8);
+            for (int half = 0; half < 2; ++half) bf[half] = stage_w[row16 * 8 + ((2 * kq + half) ^ rd_swz)];
+            wave_lds_order();
 #pragma unroll
-            for (int i = 0; i < MT; ++i) {
-                bf16x8 a;
-                if (IN_LDS) a = *reinterpret_cast<const bf16x8*>(a_s + static_cast<size_t>(i * 16 + row16) * a_stride + kc);
-                else a = af[half];
-                acc[i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, acc[i], 0, 0, 0);
+            for (int half = 0; half < 2; ++half) {
+                const int k = k0 + 16 * kq + 8 * half;
+                const bf16x8 b = k < K ? bf[half] : zero;
+                const int kc = min(k, K - 8);
+#pragma unroll
+                for (int i = 0; i < MT; ++i) {
+                    bf16x8 a;
+                    if (IN_LDS) a = *reinterpret_cast<const bf16x8*>(a_s + static_cast<size_t>(i * 16 + row16) * a_stride + kc);
+                    else a = af[half];
+                    acc[i * NT + t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, acc[i * NT + t], 0, 0, 0);
+                }
             }
         }
     };
@@ -607,17 +628,22 @@ gemm_bf16_skinny(const void* __restrict__ Ain, int lda, const bf16_t* __restrict
         return;
     }
 #pragma unroll
-    for (int i = 0; i < MT; ++i)
+    for (int i = 0; i < T; ++i)
 #pragma unroll
-        for (int r = 0; r < 4; ++r) red[(static_cast<size_t>(wave) * MT + i) * 256 + r * 64 + lane] = acc[i][r];
+        for (int r = 0; r < 4; ++r) red[(static_cast<size_t>(wave) * T + i) * 256 + r * 64 + lane] = acc[i][r];
     __syncthreads();
     if (MT == 1) {
-        // one output per thread (the first 256); its bias and old residual value were requested
-        // before the MFMA loop
-        float v = 0.f;
-        if (tid < 256)
-            for (int w = 0; w < nw; ++w) v += red[static_cast<size_t>(w) * 256 + tid];
-        if (k_parts > 1) {
+        // one output per tile and thread (the first 256); its bias and old residual value were
+        // requested before the MFMA loop
+        float vt[NT];
+#pragma unroll
+        for (int t = 0; t < NT; ++t) {
+            vt[t] = 0.f;
+            if (tid < 256)
+                for (int w = 0; w < nw; ++w) vt[t] += red[(static_cast<size_t>(w) * NT + t) * 256 + tid];
+        }
+        float& v = vt[0];
+        if (NT == 1 && k_parts > 1) {
             // The parts of a tile meet in the workspace. Stores and loads of it are at device scope
             // (workgroups of one tile may run on different XCDs, whose L2 caches do not see each
             // other's lines); one thread's fences order them around the counter (a fence in every
@@ -643,10 +669,13 @@ gemm_bf16_skinny(const void* __restrict__ Ain, int lda, const bf16_t* __restrict
                 for (int p = 0; p < k_parts; ++p)
                     v += __hip_atomic_load(&sums[p * 256 + tid], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
-        if (ep_ok) {
-            v += ep_bias;
-            if (mode == EPI_ADD_RESIDUAL) static_cast<float*>(C)[ep_idx] = ep_old + v;
-            else epilogue<bf16_t>(mode, v, 0.f, C, ep_idx);
+#pragma unroll
+        for (int t = 0; t < NT; ++t) {
+            if (ep_ok[t]) {
+                const float r = vt[t] + ep_bias[t];
+                if (mode == EPI_ADD_RESIDUAL) static_cast<float*>(C)[ep_idx[t]] = ep_old[t] + r;
+                else epilogue<bf16_t>(mode, r, 0.f, C, ep_idx[t]);
+            }
         }
         return;
     }
@@ -724,9 +753,15 @@ static int launch_skinny(const void* A, int lda, const bf16_t* W, int ldw, const
         nw = (tiles * row_blocks + 255) / 256;
         nw = nw < 4 ? 4 : (nw > 16 ? 16 : nw);
     }
-    const int col_blocks = split_k ? tiles : (tiles + nw - 1) / nw;
+    // More than 256 tiles (and one row block): two tiles per workgroup, the columns dealt out evenly
+    // to 256 workgroups.
+    int cols_per_wg = 16;
+    const bool two_tiles = split_k && row_blocks == 1 && k_parts == 1 && tiles > 256 && tiles <= 512 &&
+                           (LN_FUSED || M <= 8);
+    if (two_tiles) cols_per_wg = (N + 255) / 256;
+    const int col_blocks = split_k ? (N + cols_per_wg - 1) / cols_per_wg : (tiles + nw - 1) / nw;
     const dim3 grid((col_blocks + N_XCD - 1) / N_XCD * N_XCD * row_blocks, k_parts), block(nw * 64);
-    size_t smem = split_k ? static_cast<size_t>(nw) * mt * 256 * sizeof(float) : 0;
+    size_t smem = split_k ? static_cast<size_t>(nw) * mt * (two_tiles ? 2 : 1) * 256 * sizeof(float) : 0;
     smem += static_cast<size_t>(nw) * (LN_FUSED || staged ? 2048 : 4096);     // the wavefronts' transposition regions
     if (staged) {
         staged_bytes += smem;
@@ -738,7 +773,7 @@ static int launch_skinny(const void* A, int lda, const bf16_t* W, int ldw, const
                                            static_cast<int>(staged_bytes));                            \
         if (e != hipSuccess) return static_cast<int>(e);                                               \
         kernel<<<grid, block, staged_bytes, stream>>>(A, lda, W, ldw, bias, C, ldc, M, N, K, mode, gamma, beta, \
-                                                      eps, rows, col_blocks, row_blocks, 1, nullptr, nullptr); \
+                                                      eps, rows, col_blocks, row_blocks, 16, 1, nullptr, nullptr); \
         break;                                                                                         \
     }
         switch (mt) {
@@ -756,9 +791,9 @@ static int launch_skinny(const void* A, int lda, const bf16_t* W, int ldw, const
     }
     if (smem > MAX_DYNAMIC_LDS) return -2;
     constexpr int ASRC = LN_FUSED ? A_NORMED : A_GLOBAL;
-#define SKINNY_LAUNCH(SPLIT, UV, A2)                                                                   \
+#define SKINNY_LAUNCH(SPLIT, UV, A2, NTV)                                                              \
     do {                                                                                               \
-        auto kernel = gemm_bf16_skinny<1, ASRC, SPLIT, UV, A2>;                                        \
+        auto kernel = gemm_bf16_skinny<1, ASRC, SPLIT, UV, A2, NTV>;                                   \
         static bool lds_allowed = false;      /* more than 64 KB of dynamic LDS has to be asked for once */ \
         if (!lds_allowed) {                                                                            \
             hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),                  \
@@ -767,31 +802,37 @@ static int launch_skinny(const void* A, int lda, const bf16_t* W, int ldw, const
             lds_allowed = true;                                                                        \
         }                                                                                              \
         kernel<<<grid, block, smem, stream>>>(A, lda, W, ldw, bias, C, ldc, M, N, K, mode, gamma, beta, eps, rows, \
-                                              col_blocks, row_blocks, k_parts, part_sums, part_counters); \
+                                              col_blocks, row_blocks, cols_per_wg, k_parts, part_sums,    \
+                                              part_counters);                                          \
     } while (0)
     if (split_k) {
         // a chunk holds all k blocks of a wavefront when they are at most 3 (4 without the fused
-        // norm and with at most 8 rows; with more rows A takes two loads per block and 3 blocks
-        // are the most): two chunks of fragments must fit the registers
+        // norm and with at most 8 rows): whole chunks only, so nothing is requested twice. The
+        // largest chunks of the kernels without the norm spill a few registers, and are still
+        // faster than smaller chunks (measured)
         const int per_wave = (k_blocks + nw - 1) / nw;
-        if (LN_FUSED) {
+        if (two_tiles) {
+            // (two tiles per chunk slot: half the blocks per chunk)
+            if (per_wave <= 1 || !LN_FUSED) SKINNY_LAUNCH(true, 2, false, 2);
+            else SKINNY_LAUNCH(true, 4, false, 2);
+        } else if (LN_FUSED) {
             switch (std::min(per_wave, 3)) {
-                case 1: SKINNY_LAUNCH(true, 2, false); break;
-                case 2: SKINNY_LAUNCH(true, 4, false); break;
-                default: SKINNY_LAUNCH(true, 6, false); break;
+                case 1: SKINNY_LAUNCH(true, 2, false, 1); break;
+                case 2: SKINNY_LAUNCH(true, 4, false, 1); break;
+                default: SKINNY_LAUNCH(true, 6, false, 1); break;
             }
         } else if (M <= 8) {
             switch (std::min(per_wave, 4)) {
-                case 1: SKINNY_LAUNCH(true, 2, false); break;
-                case 2: SKINNY_LAUNCH(true, 4, false); break;
-                case 3: SKINNY_LAUNCH(true, 6, false); break;
-                default: SKINNY_LAUNCH(true, 8, false); break;
+                case 1: SKINNY_LAUNCH(true, 2, false, 1); break;
+                case 2: SKINNY_LAUNCH(true, 4, false, 1); break;
+                case 3: SKINNY_LAUNCH(true, 6, false, 1); break;
+                default: SKINNY_LAUNCH(true, 8, false, 1); break;
             }
         } else {
             switch (std::min(per_wave, 3)) {
-                case 1: SKINNY_LAUNCH(true, 2, true); break;
-                case 2: SKINNY_LAUNCH(true, 4, true); break;
-                default: SKINNY_LAUNCH(true, 6, true); break;
+                case 1: SKINNY_LAUNCH(true, 2, true, 1); break;
+                case 2: SKINNY_LAUNCH(true, 4, true, 1); break;
+                default: SKINNY_LAUNCH(true, 6, true, 1); break;
             }
         }
     } else {

@@ -174,7 +174,9 @@ def test_linear_bf16_scatters_keys_and_values(ops, M, H, Hkv, dh, K):
 
 @pytest.mark.parametrize("M", [1, 8, 16, 17, 48, 64])
 @pytest.mark.parametrize("N,K", [(2304, 768), (768, 3072), (1000, 96), (50257, 768), (72, 1600), (4800, 1600),
-                                 (1600, 6400), (1024, 4096)])
+                                 (1600, 6400), (1024, 4096),
+                                 # more than 256 tiles of 16 columns: two tiles per workgroup, the second narrower
+                                 (4104, 72), (6400, 1600), (8190, 200)])
 def test_linear_bf16_few_rows(ops, M, N, K):
     """The weight-streaming kernel of decode steps (M <= 64), every wavefront count and m-tile count."""
     g = torch.Generator().manual_seed(M + N + K)
@@ -231,6 +233,8 @@ def test_linear_bf16_few_rows_long_k_shares_tiles(ops, M, N, K):
 @pytest.mark.parametrize("M,N,K", [(1, 2304, 768), (8, 3072, 768), (16, 320, 96), (5, 200, 1600), (17, 96, 64),
                                    (3, 64, 4096), (16, 6400, 1600), (9, 50257, 1024), (16, 3072, 1024), (33, 2304, 768),
                                    (64, 50257, 768), (64, 104, 1600), (65, 96, 64),
+                                   # more than 256 tiles: two per workgroup
+                                   (8, 4800, 1600), (3, 4104, 72), (16, 8190, 200),
                                    # more than 16 rows: the norm runs as a kernel of its own
                                    (64, 3072, 768), (48, 4096, 1024), (17, 40, 72), (31, 1000, 2048), (50, 136, 200)])
 @pytest.mark.parametrize("epi", ["store", "gelu_tanh", "gelu_erf", "store_f32"])
