@@ -759,6 +759,11 @@ static int launch_skinny(const void* A, int lda, const bf16_t* W, int ldw, const
     const bool two_tiles = split_k && row_blocks == 1 && k_parts == 1 && tiles > 256 && tiles <= 512 &&
                            (LN_FUSED || M <= 8);
     if (two_tiles) cols_per_wg = (N + 255) / 256;
+    // Fewer than 256 tiles, one row block and a long K (the second product of the feed-forward):
+    // narrower tiles, down to 4 columns, so that more compute units share the weights. (Short K, or
+    // the fused norm: the kernel's time is latency, not bytes, and nothing is gained; measured.)
+    if (split_k && !LN_FUSED && row_blocks == 1 && k_parts == 1 && tiles < 256 && k_blocks >= 48)
+        cols_per_wg = std::min(16, std::max((N + 255) / 256, 4));
     const int col_blocks = split_k ? (N + cols_per_wg - 1) / cols_per_wg : (tiles + nw - 1) / nw;
     const dim3 grid((col_blocks + N_XCD - 1) / N_XCD * N_XCD * row_blocks, k_parts), block(nw * 64);
     size_t smem = split_k ? static_cast<size_t>(nw) * mt * (two_tiles ? 2 : 1) * 256 * sizeof(float) : 0;
