@@ -76,7 +76,7 @@ decode_attention_kernel(const T* __restrict__ q, int q_stride, int q_col,
     const int pair = blockIdx.x, split = blockIdx.y;
     const int t = pair / n_heads, h = pair % n_heads;
     const int hk = h / (n_heads / n_kv_heads);
-    const int wave = threadIdx.x / MLLM_WAVE, lane = threadIdx.x % MLLM_WAVE;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / MLLM_WAVE), lane = threadIdx.x % MLLM_WAVE;
     const int c = lane % LPK, g = lane / LPK;
     const int b = token_seq[t], p = positions[t];
     const int lo = (window > 0 && p - window + 1 > 0) ? p - window + 1 : 0;
