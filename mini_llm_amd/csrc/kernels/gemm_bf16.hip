@@ -348,6 +348,8 @@ gemm_bf16_skinny(const void* __restrict__ Ain, int lda, const bf16_t* __restrict
     bf16x8* stage_a = stage_w + 128;                                       // (A_GLOBAL only)
     bf16_t* a_s = reinterpret_cast<bf16_t*>(smem_raw + red_bytes + static_cast<size_t>(nw) * STAGE_BYTES);   // [16*MT][K+8]
     const int a_stride = K + 8;
+    // (fused norm only) the scale and shift vectors, loaded once per workgroup: [2][K] fp32
+    float4* gb_s = reinterpret_cast<float4*>(a_s + static_cast<size_t>(16) * MT * a_stride);
     const int n = n0 + row16;
     const bool n_ok = n < N;
     const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
@@ -504,7 +506,7 @@ gemm_bf16_skinny(const void* __restrict__ Ain, int lda, const bf16_t* __restrict
     // their requests, so the norm (whose rows come from L2) can be computed while the weights are
     // still on their way from memory, which it could not if it had to wait for them first.
     const int nq = K / 4, n_u = (nq + 63) / 64;       // float4 per row; per lane (uniform)
-    float4 gg[8], bb[8], v[2][8];
+    float4 gb_piece[2], v[2][8];
     // whether this wavefront's two rows exist is uniform over it: rows beyond M are not read
     const bool row_ok[2] = {m_base + wave < M, m_base + wave + 8 < M};
     if (LN_FUSED) {
@@ -522,13 +524,13 @@ gemm_bf16_skinny(const void* __restrict__ Ain, int lda, const bf16_t* __restrict
             }
         }
         __builtin_amdgcn_sched_barrier(0);
+        // scale and shift: 2 K / 4 pieces of 16 bytes over the workgroup's 512 threads (K <= 2048:
+        // at most two each), shared through LDS instead of every wavefront loading all of both
 #pragma unroll
-        for (int u = 0; u < 8; ++u) {
-            if (u < n_u) {
-                const int i = min(lane + 64 * u, nq - 1);
-                gg[u] = g4[i];
-                bb[u] = beta ? b4[i] : make_float4(0.f, 0.f, 0.f, 0.f);
-            }
+        for (int r = 0; r < 2; ++r) {
+            const int i = min(tid + 512 * r, 2 * nq - 1);
+            const float4* src = i < nq ? g4 + i : (beta ? b4 + (i - nq) : g4);
+            gb_piece[r] = *src;
         }
         __builtin_amdgcn_sched_barrier(0);
     }
@@ -560,6 +562,31 @@ gemm_bf16_skinny(const void* __restrict__ Ain, int lda, const bf16_t* __restrict
         // 8 wavefronts, two rows each; a row lives in registers (K <= 2048, K % 4 == 0): mean,
         // then variance of the centred values, all in fp32.
 #pragma unroll
+        for (int r = 0; r < 2; ++r) {
+            const int i = tid + 512 * r;
+            if (i < 2 * nq) gb_s[i] = (i >= nq && !beta) ? make_float4(0.f, 0.f, 0.f, 0.f) : gb_piece[r];
+        }
+        float mean[2] = {0.f, 0.f}, inv[2] = {0.f, 0.f};
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            if (!row_ok[j]) continue;
+            float sum = 0.f;
+#pragma unroll
+            for (int u = 0; u < 8; ++u)
+                if (u < n_u && lane + 64 * u < nq) sum += (v[j][u].x + v[j][u].y) + (v[j][u].z + v[j][u].w);
+            mean[j] = wave_sum(sum) / static_cast<float>(K);
+            float q = 0.f;
+#pragma unroll
+            for (int u = 0; u < 8; ++u) {
+                if (u < n_u && lane + 64 * u < nq) {
+                    const float a = v[j][u].x - mean[j], b = v[j][u].y - mean[j], c = v[j][u].z - mean[j], d = v[j][u].w - mean[j];
+                    q += (a * a + b * b) + (c * c + d * d);
+                }
+            }
+            inv[j] = 1.0f / sqrtf(wave_sum(q) / static_cast<float>(K) + eps);
+        }
+        lds_barrier();                 // scale and shift are in LDS (the weights stay in flight)
+#pragma unroll
         for (int j = 0; j < 2; ++j) {
             const int m = wave + 8 * j;
             bf16_t* dst = a_s + static_cast<size_t>(m) * a_stride;
@@ -567,32 +594,19 @@ gemm_bf16_skinny(const void* __restrict__ Ain, int lda, const bf16_t* __restrict
                 for (int i = lane; i < nq; i += 64) *reinterpret_cast<uint2*>(dst + 4 * i) = make_uint2(0, 0);
                 continue;
             }
-            float s = 0.f;
-#pragma unroll
-            for (int u = 0; u < 8; ++u)
-                if (u < n_u && lane + 64 * u < nq) s += (v[j][u].x + v[j][u].y) + (v[j][u].z + v[j][u].w);
-            const float mean = wave_sum(s) / static_cast<float>(K);
-            float q = 0.f;
-#pragma unroll
-            for (int u = 0; u < 8; ++u) {
-                if (u < n_u && lane + 64 * u < nq) {
-                    const float a = v[j][u].x - mean, b = v[j][u].y - mean, c = v[j][u].z - mean, d = v[j][u].w - mean;
-                    q += (a * a + b * b) + (c * c + d * d);
-                }
-            }
-            const float inv = 1.0f / sqrtf(wave_sum(q) / static_cast<float>(K) + eps);
 #pragma unroll
             for (int u = 0; u < 8; ++u) {
                 const int i = lane + 64 * u;
                 if (u < n_u && i < nq) {
+                    const float4 g = gb_s[i], b = gb_s[nq + i];
                     uint2 pk;
-                    pk.x = pack_bf16x2((v[j][u].x - mean) * inv * gg[u].x + bb[u].x, (v[j][u].y - mean) * inv * gg[u].y + bb[u].y);
-                    pk.y = pack_bf16x2((v[j][u].z - mean) * inv * gg[u].z + bb[u].z, (v[j][u].w - mean) * inv * gg[u].w + bb[u].w);
+                    pk.x = pack_bf16x2((v[j][u].x - mean[j]) * inv[j] * g.x + b.x, (v[j][u].y - mean[j]) * inv[j] * g.y + b.y);
+                    pk.y = pack_bf16x2((v[j][u].z - mean[j]) * inv[j] * g.z + b.z, (v[j][u].w - mean[j]) * inv[j] * g.w + b.w);
                     *reinterpret_cast<uint2*>(dst + 4 * i) = pk;
                 }
             }
         }
-        __syncthreads();
+        lds_barrier();
     }
 
     if (n_chunks == 1) {
@@ -789,7 +803,7 @@ static int launch_skinny(const void* A, int lda, const bf16_t* W, int ldw, const
         return 0;
     }
     if (LN_FUSED) {
-        smem += static_cast<size_t>(16) * mt * (K + 8) * sizeof(bf16_t);
+        smem += static_cast<size_t>(16) * mt * (K + 8) * sizeof(bf16_t) + static_cast<size_t>(2) * K * sizeof(float);
         if (K > 2048 || (reinterpret_cast<uintptr_t>(A) & 15) || lda % 4 != 0 ||
             (reinterpret_cast<uintptr_t>(gamma) & 15) || (reinterpret_cast<uintptr_t>(beta) & 15))
             return -2;
