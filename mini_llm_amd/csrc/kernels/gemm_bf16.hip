@@ -498,9 +498,16 @@ gemm_bf16_skinny(const void* __restrict__ Ain, int lda, const bf16_t* __restrict
             if (h < left) load_steps(c1, 2 * h, k_first + (first + h) * k_stride);
         __builtin_amdgcn_sched_barrier(0);
     };
+    // The first loads are one whole chunk for every wavefront, without a condition: a wavefront
+    // with fewer blocks than a chunk takes its last block again (its own line, requested a moment
+    // earlier) and leaves it unused. (Whole chunk or leftovers, decided by a branch, would hand the
+    // norm that follows registers that count as pending on one side of the branch, and it would
+    // wait for the weights.)
+    const int last_block = n_blocks > 0 ? n_blocks - 1 : 0;
     auto first_loads = [&]() {
-        if (n_chunks > 0) load_chunk(c0, 0);
-        else load_left();                                   // a wavefront without a whole chunk starts with these
+#pragma unroll
+        for (int h = 0; h < H; ++h) load_steps(c0, 2 * h, k_first + min(h, last_block) * k_stride);
+        __builtin_amdgcn_sched_barrier(0);
     };
     // The fused norm's operands are requested before the weights: loads return in the order of
     // their requests, so the norm (whose rows come from L2) can be computed while the weights are
@@ -561,11 +568,6 @@ gemm_bf16_skinny(const void* __restrict__ Ain, int lda, const bf16_t* __restrict
     if (LN_FUSED) {
         // 8 wavefronts, two rows each; a row lives in registers (K <= 2048, K % 4 == 0): mean,
         // then variance of the centred values, all in fp32.
-#pragma unroll
-        for (int r = 0; r < 2; ++r) {
-            const int i = tid + 512 * r;
-            if (i < 2 * nq) gb_s[i] = (i >= nq && !beta) ? make_float4(0.f, 0.f, 0.f, 0.f) : gb_piece[r];
-        }
         float mean[2] = {0.f, 0.f}, inv[2] = {0.f, 0.f};
 #pragma unroll
         for (int j = 0; j < 2; ++j) {
@@ -584,6 +586,11 @@ gemm_bf16_skinny(const void* __restrict__ Ain, int lda, const bf16_t* __restrict
                 }
             }
             inv[j] = 1.0f / sqrtf(wave_sum(q) / static_cast<float>(K) + eps);
+        }
+#pragma unroll
+        for (int r = 0; r < 2; ++r) {
+            const int i = tid + 512 * r;
+            if (i < 2 * nq) gb_s[i] = (i >= nq && !beta) ? make_float4(0.f, 0.f, 0.f, 0.f) : gb_piece[r];
         }
         lds_barrier();                 // scale and shift are in LDS (the weights stay in flight)
 #pragma unroll
@@ -609,7 +616,11 @@ gemm_bf16_skinny(const void* __restrict__ Ain, int lda, const bf16_t* __restrict
         lds_barrier();
     }
 
-    if (n_chunks == 1) {
+    if (n_chunks == 0) {
+#pragma unroll
+        for (int h = 0; h < H - 1; ++h)
+            if (h < n_blocks) mma_steps(c0, 2 * h, k_first + h * k_stride);
+    } else if (n_chunks == 1) {
         mma_chunk(c0, 0);
     } else if (n_chunks > 1) {
         // past the last chunk the prefetch takes chunk 0 again (long since arrived, never used)
@@ -622,8 +633,8 @@ gemm_bf16_skinny(const void* __restrict__ Ain, int lda, const bf16_t* __restrict
     }
     {
         // blocks left over: fewer than H, loaded together
-        const int first = n_chunks * H, left = n_blocks - first;
-        if (n_chunks > 0) load_left();
+        const int first = n_chunks * H, left = n_chunks > 0 ? n_blocks - first : 0;
+        if (left > 0) load_left();
 #pragma unroll
         for (int h = 0; h < H - 1; ++h)
             if (h < left) mma_steps(c1, 2 * h, k_first + (first + h) * k_stride);
