@@ -39,6 +39,12 @@ template <> struct Vec16<float> {
 };
 template <typename T>
 __device__ __forceinline__ uint4 load_raw16(const T* p) { return *reinterpret_cast<const uint4*>(p); }
+typedef unsigned int u32x4_nt __attribute__((ext_vector_type(4)));
+template <typename T>
+__device__ __forceinline__ uint4 load_stream16(const T* p) {
+    const u32x4_nt v = __builtin_nontemporal_load(reinterpret_cast<const u32x4_nt*>(p));
+    return make_uint4(v.x, v.y, v.z, v.w);
+}
 
 template <int N>
 __device__ __forceinline__ void merge_state(float& m, float& l, float (&o)[N], float m2, float l2,
@@ -138,8 +144,8 @@ decode_attention_kernel(const T* __restrict__ q, int q_stride, int q_col,
         for (int u = 0; u < DEC_UNROLL; ++u) {
             const int j = min(j0 + u * n_waves * KPW + g, ke_pages - 1);
             const size_t row = (static_cast<size_t>(sm_table[(j >> shift) - first_blk]) << shift) + (j & mask);
-            kraw[u] = load_raw16(k_pages + row * kv_dim + col);
-            vraw[u] = load_raw16(v_pages + row * kv_dim + col);
+            kraw[u] = load_stream16(k_pages + row * kv_dim + col);
+            vraw[u] = load_stream16(v_pages + row * kv_dim + col);
         }
         float dot[DEC_UNROLL];
         float mx = NEG;
