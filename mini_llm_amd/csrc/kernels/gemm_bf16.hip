@@ -425,13 +425,16 @@ gemm_bf16_skinny(const void* __restrict__ Ain, int lda, const bf16_t* __restrict
 #pragma unroll
         for (int j = 0; j < 2; ++j) {
             const int k = min(k0 + 8 * piece[j], K - 8);
-            // (the wide product's weights, the logits head, are read once a step and are as large as
-            // all the layers': a streaming load keeps them from displacing the layers' weights in
-            // the caches)
+            // Weights that one workgroup alone reads (one row block: at most 8 rows, or the fused
+            // norm's 16) and the wide product's (the logits head, as large as all the layers') are
+            // requested with streaming loads: read once a step, they would only displace what is
+            // read again (activations, scale and shift vectors, biases) from the caches. With
+            // several row blocks the later ones find the weights in L2 and plain loads are kept.
+            constexpr bool STREAM = ASRC != A_GLOBAL || !A_TWO;
 #pragma unroll
             for (int t = 0; t < NT; ++t) {
                 const bf16x8* src = reinterpret_cast<const bf16x8*>(wrow[t][j] + k);
-                c.b[t][u0 + j] = ASRC == A_STAGED ? __builtin_nontemporal_load(src) : *src;
+                c.b[t][u0 + j] = STREAM ? __builtin_nontemporal_load(src) : *src;
             }
             if (ASRC == A_GLOBAL && (j == 0 || a_two)) c.a[A_TWO ? u0 + j : u0 / 2] = *reinterpret_cast<const bf16x8*>(arow[j] + k);
         }
