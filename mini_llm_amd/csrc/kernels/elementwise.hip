@@ -94,27 +94,39 @@ __global__ void __launch_bounds__(256)
 layernorm_wave_kernel(const float* __restrict__ x, const int* __restrict__ rows,
                       const float* __restrict__ gamma, const float* __restrict__ beta,
                       OutT* __restrict__ y, int n, int D, float eps) {
-    const int wave = threadIdx.x / MLLM_WAVE, lane = threadIdx.x % MLLM_WAVE;
+    // (the wavefront's index as a scalar, so that the exit below is a real branch; every load is
+    // issued without a condition, from a clamped index, and all of them before the first use: a
+    // load under a condition, or one left inside the last loop, starts only when the statistics
+    // are done and adds its whole latency)
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / MLLM_WAVE), lane = threadIdx.x % MLLM_WAVE;
     const int r = blockIdx.x * 4 + wave;
     if (r >= n) return;
     const int src = rows ? rows[r] : r;
     const float4* xr = reinterpret_cast<const float4*>(x + static_cast<size_t>(src) * D);
     const float4* g4 = reinterpret_cast<const float4*>(gamma);
-    const float4* b4 = reinterpret_cast<const float4*>(beta);
-    const int nq = D / 4;
-    float4 v[8];
-    float s = 0.f;
+    const float4* b4 = reinterpret_cast<const float4*>(beta ? beta : gamma);
+    const int nq = D / 4, n_u = (nq + 63) / 64;
+    float4 v[8], gg[8], bb[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u)
+        if (u < n_u) v[u] = xr[min(lane + 64 * u, nq - 1)];
 #pragma unroll
     for (int u = 0; u < 8; ++u) {
-        const int i = lane + 64 * u;
-        v[u] = i < nq ? xr[i] : make_float4(0.f, 0.f, 0.f, 0.f);
-        s += (v[u].x + v[u].y) + (v[u].z + v[u].w);
+        if (u < n_u) {
+            const int i = min(lane + 64 * u, nq - 1);
+            gg[u] = g4[i];
+            bb[u] = b4[i];
+        }
     }
+    float s = 0.f;
+#pragma unroll
+    for (int u = 0; u < 8; ++u)
+        if (u < n_u && lane + 64 * u < nq) s += (v[u].x + v[u].y) + (v[u].z + v[u].w);
     const float mean = wave_sum(s) / static_cast<float>(D);
     float q = 0.f;
 #pragma unroll
     for (int u = 0; u < 8; ++u) {
-        if (lane + 64 * u < nq) {
+        if (u < n_u && lane + 64 * u < nq) {
             const float a = v[u].x - mean, b = v[u].y - mean, c = v[u].z - mean, d = v[u].w - mean;
             q += (a * a + b * b) + (c * c + d * d);
         }
@@ -124,11 +136,11 @@ layernorm_wave_kernel(const float* __restrict__ x, const int* __restrict__ rows,
 #pragma unroll
     for (int u = 0; u < 8; ++u) {
         const int i = lane + 64 * u;
-        if (i < nq) {
-            const float4 gg = g4[i];
-            const float4 bb = beta ? b4[i] : make_float4(0.f, 0.f, 0.f, 0.f);
-            const float o0 = (v[u].x - mean) * inv * gg.x + bb.x, o1 = (v[u].y - mean) * inv * gg.y + bb.y;
-            const float o2 = (v[u].z - mean) * inv * gg.z + bb.z, o3 = (v[u].w - mean) * inv * gg.w + bb.w;
+        if (u < n_u && i < nq) {
+            const float4 g = gg[u];
+            const float4 b = beta ? bb[u] : make_float4(0.f, 0.f, 0.f, 0.f);
+            const float o0 = (v[u].x - mean) * inv * g.x + b.x, o1 = (v[u].y - mean) * inv * g.y + b.y;
+            const float o2 = (v[u].z - mean) * inv * g.z + b.z, o3 = (v[u].w - mean) * inv * g.w + b.w;
             if (sizeof(OutT) == 2) {
                 uint2 pk;
                 pk.x = pack_bf16x2(o0, o1);
