@@ -251,12 +251,18 @@ decode_attention_kernel(const T* __restrict__ q, int q_stride, int q_col,
         for (int e = 0; e < EPL; ++e) ws_o[slot * DH + c * EPL + e] = o[e];
         if (c == 0) { ws_ml[slot * 2] = m; ws_ml[slot * 2 + 1] = l; }
     }
-    __threadfence();
+    // One thread's fences order the partial results around the counter (after the barrier its
+    // release covers every thread's stores); a fence in every thread would write back and
+    // invalidate the L2 once per wavefront, tens of microseconds in all.
     __syncthreads();
-    if (threadIdx.x == 0) sm_last = (atomicAdd(&counters[pair], 1) == nsplit - 1) ? 1 : 0;
+    if (threadIdx.x == 0) {
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
+        const int arrived = __hip_atomic_fetch_add(&counters[pair], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        sm_last = (arrived == nsplit - 1) ? 1 : 0;
+        if (sm_last) __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+    }
     __syncthreads();
     if (!sm_last) return;
-    __threadfence();
     // Last workgroup of this (token, head): lane group G takes split G (all loads in flight at
     // once), then the same merge as above.
     m = NEG; l = 0.f;

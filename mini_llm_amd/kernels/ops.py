@@ -388,8 +388,9 @@ def _decode_launch_shape(pairs: int, max_ctx_len: int):
     """How many workgroups share one (token, head) pair's keys, and wavefronts per workgroup."""
     if DECODE_SHAPE_OVERRIDE is not None:
         return DECODE_SHAPE_OVERRIDE
-    # One workgroup per pair: merging splits needs a device-wide fence, which costs more than the
-    # parallelism gains at these context lengths. Few pairs get more wavefronts each instead.
+    # One workgroup per pair: merging splits (fences, a second merge) costs about 3 us, more than
+    # the parallelism gains below about 2,000 keys (measured at 12 to 96 pairs). Few pairs get more
+    # wavefronts each instead.
     return 1, (4 if pairs >= 512 else 8)
 
 
