@@ -381,7 +381,7 @@ def paged_attention(q: torch.Tensor, q_col: int, n_heads: int, n_kv_heads: int, 
 
 
 _DECODE_WS = {}
-DECODE_SHAPE_OVERRIDE = None      # (nsplit, waves): set by tuning scripts only
+DECODE_SHAPE_OVERRIDE = None      # (nsplit, waves): set by tests of the split path and by tuning scripts
 
 
 def _decode_launch_shape(pairs: int, max_ctx_len: int):

@@ -366,18 +366,25 @@ def test_paged_attention_mixed_batch(ops, dtype, H, Hkv, dh, page):
 @pytest.mark.parametrize("H,Hkv,dh,page", [(12, 12, 64, 16), (4, 4, 16, 4), (3, 3, 32, 8), (6, 2, 128, 16),
                                            (2, 1, 256, 64), (5, 5, 48, 16)])
 @pytest.mark.parametrize("window", [0, 33])
-def test_paged_attention_decode_only(ops, dtype, H, Hkv, dh, page, window):
-    """Every query a single token: the split-key decode kernel (power-of-two head sizes; others
-    fall back), contexts from 1 token to a thousand so that splits are empty, partial and full."""
+@pytest.mark.parametrize("shape", [None, (3, 4), (8, 2)])
+def test_paged_attention_decode_only(ops, dtype, H, Hkv, dh, page, window, shape):
+    """Every query a single token: the decode kernel (power-of-two head sizes; others fall back),
+    in its default launch shape and with the keys of a query split over 3 and 8 workgroups whose
+    partial results the last one merges; contexts from 1 token to a thousand so that splits are
+    empty, partial and full."""
     g = torch.Generator().manual_seed(H * 10 + dh + window)
-    for seqs in ([(0, 1)], [(1023, 1), (0, 1), (63, 1), (64, 1), (500, 1), (17, 1), (129, 1), (255, 1)],
-                 [(s, 1) for s in range(3, 300, 7)]):
-        out, ref = _attention_case(ops, dtype, H, Hkv, dh, page, seqs, window, g)
-        assert torch.isfinite(out).all()
+    ops.DECODE_SHAPE_OVERRIDE = shape
+    try:
+        for seqs in ([(0, 1)], [(1023, 1), (0, 1), (63, 1), (64, 1), (500, 1), (17, 1), (129, 1), (255, 1)],
+                     [(s, 1) for s in range(3, 300, 7)]):
+            out, ref = _attention_case(ops, dtype, H, Hkv, dh, page, seqs, window, g)
+            assert torch.isfinite(out).all()
+            assert (out - ref).abs().max() <= _tol(dtype, 2)
+        # run twice in a row: the split counters must be back at zero
+        out, ref = _attention_case(ops, dtype, H, Hkv, dh, page, [(700, 1), (2, 1)], window, g)
         assert (out - ref).abs().max() <= _tol(dtype, 2)
-    # run twice in a row: the split counters must be back at zero
-    out, ref = _attention_case(ops, dtype, H, Hkv, dh, page, [(700, 1), (2, 1)], window, g)
-    assert (out - ref).abs().max() <= _tol(dtype, 2)
+    finally:
+        ops.DECODE_SHAPE_OVERRIDE = None
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
