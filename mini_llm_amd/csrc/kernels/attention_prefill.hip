@@ -65,7 +65,7 @@ prefill_attention_kernel(const bf16_t* __restrict__ q, int q_stride, int q_col,
     if (b >= n_seqs) return;               // surplus workgroup; the whole workgroup leaves
 
     const int h = blockIdx.x, hk = h / (n_heads / n_kv_heads);
-    const int tid = threadIdx.x, wave = tid / 64, lane = tid % 64;
+    const int tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid / 64), lane = tid % 64;
     const int G = lane / 16, c16 = lane % 16;
     const int start = ctx_len[b] - q_len;                 // position of the step's first query
     const int q0 = tile * PF_BM;
