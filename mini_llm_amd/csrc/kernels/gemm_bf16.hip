@@ -893,7 +893,14 @@ static int gemm_bf16_dispatch(const void* A, int lda, const void* W, int ldw, co
     const bf16_t* a = static_cast<const bf16_t*>(A);
     const bf16_t* w = static_cast<const bf16_t*>(W);
     const bool scatter = kv.slots != nullptr;       // only the many-row kernel scatters
-    if (!scatter && M <= 64 && launch_skinny<false>(A, lda, w, ldw, bias, C, ldc, M, N, K, mode, nullptr, nullptr,
+    // The weight-streaming kernel takes up to 64 rows always, and up to 256 rows while its 16-row
+    // by 16-column workgroups stay within about four rounds over the compute units (measured
+    // against the tiled kernel on GPT-2 small to XL shapes at 64 to 256 rows: narrow outputs such
+    // as the attention and feed-forward output projections stay with it up to 256 rows, the wide
+    // ones leave it between 64 and 128 rows)
+    const long skinny_wgs = static_cast<long>((N + 15) / 16) * ((M + 15) / 16);
+    const bool few_rows = M <= 64 ? ((N + 15) / 16 >= 1024 || skinny_wgs <= 1024) : (M <= 256 && skinny_wgs <= 1024);
+    if (!scatter && few_rows && launch_skinny<false>(A, lda, w, ldw, bias, C, ldc, M, N, K, mode, nullptr, nullptr,
                                                     0.f, nullptr, stream, workspace, workspace_bytes) == 0) {
         // few rows: weight-streaming kernel
     } else if (M <= 32) {

@@ -194,9 +194,9 @@ def linear(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], out: 
                                        M, N, K, _p(slots), _p(k_pages), _p(v_pages), int(q_cols), int(kv_dim),
                                        _stream())
         else:
-            ws = _gemm_workspace(a.device) if M <= 64 else None
+            ws = _gemm_workspace(a.device) if M <= 256 else None
             rc = lib.mllm_gemm_bf16(_p(a), a.stride(0), _p(w), w.stride(0), _p(bias), _p(out), out.stride(0),
-                                    M, N, K, mode, _p(ws), ctypes.c_size_t(GEMM_WORKSPACE_BYTES if M <= 64 else 0),
+                                    M, N, K, mode, _p(ws), ctypes.c_size_t(GEMM_WORKSPACE_BYTES if M <= 256 else 0),
                                     _stream())
         if rc == -1:
             raise KernelError(

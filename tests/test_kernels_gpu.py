@@ -162,7 +162,10 @@ def test_linear_bf16_scatters_keys_and_values(ops, M, H, Hkv, dh, K):
     ops.linear(a.to(DEV), w.to(DEV), bias.to(DEV), out, "store", kv_scatter=(perm.to(DEV), kp, vp, q_cols))
     plain = torch.empty((M, N), dtype=torch.bfloat16, device=DEV)
     ops.linear(a.to(DEV), w.to(DEV), bias.to(DEV), plain, "store")
-    assert torch.equal(out, plain)
+    if M > 256:
+        assert torch.equal(out, plain)               # the same kernel with and without the page write
+    else:                                            # without, fewer rows may take the weight-streaming kernel
+        assert (out.float() - plain.float()).abs().max().item() <= 4e-2
     ref = plain_ops.linear(a, w, bias, torch.empty((M, N), dtype=torch.float64))
     assert (out.cpu().double() - ref).abs().max().item() <= 4e-2
     kr, vr = k0.clone(), v0.clone()
@@ -185,6 +188,25 @@ def test_linear_bf16_few_rows(ops, M, N, K):
     bias = 0.5 * _rand((N,), torch.float32, g)
     for epi in ("store_f32", "add_residual", "gelu_tanh"):
         f32_out = epi != "gelu_tanh"
+        out0 = _rand((M, N), torch.float32 if f32_out else torch.bfloat16, g)
+        out = out0.clone().to(DEV)
+        ops.linear(a.to(DEV), w.to(DEV), bias.to(DEV), out, epi)
+        ref = plain_ops.linear(a, w, bias, out0.double().clone(), epi)
+        err = (out.cpu().double() - ref).abs().max().item()
+        assert err <= (2e-5 + 2e-5 * math.sqrt(K) if f32_out else 4e-2), (epi, err)
+
+
+@pytest.mark.parametrize("M,N,K", [(65, 768, 768), (96, 2304, 768), (100, 1000, 96), (128, 768, 3072), (200, 72, 1600),
+                                   (256, 768, 768), (256, 1024, 4096), (250, 40, 6400), (129, 2304, 768), (64, 6400, 1600)])
+def test_linear_bf16_up_to_256_rows(ops, M, N, K):
+    """Between 65 and 256 rows the weight-streaming kernel (many 16-row blocks) or the tiled kernel
+    runs, by the number of workgroups the former would need."""
+    g = torch.Generator().manual_seed(M + N + K)
+    a = _rand((M, K), torch.bfloat16, g)
+    w = _rand((N, K), torch.bfloat16, g, std=1.0 / math.sqrt(K))
+    bias = 0.5 * _rand((N,), torch.float32, g)
+    for epi in ("store", "add_residual", "gelu_erf"):
+        f32_out = epi == "add_residual"
         out0 = _rand((M, N), torch.float32 if f32_out else torch.bfloat16, g)
         out = out0.clone().to(DEV)
         ops.linear(a.to(DEV), w.to(DEV), bias.to(DEV), out, epi)
