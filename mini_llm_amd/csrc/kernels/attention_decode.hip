@@ -60,12 +60,13 @@ __device__ __forceinline__ void merge_state(float& m, float& l, float (&o)[N], f
 
 template <typename T, int LPK, int UNR>
 __global__ void __launch_bounds__(UNR > 8 ? 512 : DEC_MAX_WAVES * MLLM_WAVE)
-decode_attention_kernel(const T* __restrict__ q, int q_stride, int q_col,
-                        const T* __restrict__ k_pages, const T* __restrict__ v_pages, int kv_dim,
-                        const int* __restrict__ block_tables, int max_blocks,
+decode_attention_kernel(// the first 16 dwords arrive in registers with the wavefront: what the first loads need
                         const int* __restrict__ token_seq, const int* __restrict__ positions,
-                        int n_heads, int n_kv_heads, int page_size, float scale_log2e, int window,
-                        int nsplit, T* __restrict__ out, int out_stride,
+                        const int* __restrict__ block_tables, int max_blocks, int n_heads, int n_kv_heads,
+                        int page_size, int window, int nsplit, const T* __restrict__ q, int q_stride, int q_col,
+                        // the rest is loaded by the kernel
+                        const T* __restrict__ k_pages, const T* __restrict__ v_pages, int kv_dim,
+                        float scale_log2e, T* __restrict__ out, int out_stride,
                         float* __restrict__ ws_o, float* __restrict__ ws_ml, int* __restrict__ counters,
                         T* __restrict__ k_pages_w, T* __restrict__ v_pages_w, int k_col, int v_col,
                         const int* __restrict__ slots) {
@@ -297,8 +298,8 @@ static int launch_decode(int lpk, dim3 grid, int waves, hipStream_t stream, cons
                          int n_kv_heads, int page_size, float scale_log2e, int window, int nsplit, T* out,
                          int out_stride, float* ws_o, float* ws_ml, int* counters, T* k_pages_w, T* v_pages_w,
                          int k_col, int v_col, const int* slots) {
-#define DEC_ARGS q, q_stride, q_col, k_pages, v_pages, kv_dim, block_tables, max_blocks, token_seq,        \
-            positions, n_heads, n_kv_heads, page_size, scale_log2e, window, nsplit, out, out_stride,   \
+#define DEC_ARGS token_seq, positions, block_tables, max_blocks, n_heads, n_kv_heads, page_size, window,  \
+            nsplit, q, q_stride, q_col, k_pages, v_pages, kv_dim, scale_log2e, out, out_stride,        \
             ws_o, ws_ml, counters, k_pages_w, v_pages_w, k_col, v_col, slots
 #define DEC_CASE(L)                                                                                    \
     case L:                                                                                            \

@@ -305,11 +305,14 @@ enum { A_GLOBAL = 0, A_NORMED = 1, A_STAGED = 2 };
 
 template <int MT, int ASRC, bool SPLIT_K, int U, bool A_TWO = true, int NT = 1>
 __global__ void __launch_bounds__(ASRC == A_NORMED ? 512 : (ASRC == A_GLOBAL ? 768 : 1024))
-gemm_bf16_skinny(const void* __restrict__ Ain, int lda, const bf16_t* __restrict__ W, int ldw,
-                 const float* __restrict__ bias, void* __restrict__ C, int ldc, int M, int N, int K, int mode,
-                 const float* __restrict__ gamma, const float* __restrict__ beta, float eps,
-                 const int* __restrict__ rows, int col_blocks, int row_blocks, int cols_per_wg, int k_parts,
-                 float* __restrict__ part_sums, int* __restrict__ part_counters) {
+gemm_bf16_skinny(// the first 16 dwords arrive in registers with the wavefront: what the first loads need
+                 const bf16_t* __restrict__ W, int ldw, int N, int K, int M, int col_blocks, int row_blocks,
+                 int cols_per_wg, int k_parts, const void* __restrict__ Ain, int lda, int mode,
+                 const float* __restrict__ bias,
+                 // the rest is loaded by the kernel and needed later
+                 void* __restrict__ C, int ldc, const float* __restrict__ gamma, const float* __restrict__ beta,
+                 float eps, const int* __restrict__ rows, float* __restrict__ part_sums,
+                 int* __restrict__ part_counters) {
     // NT > 1 (SPLIT_K, MT == 1): the workgroup owns cols_per_wg <= 16 NT columns, NT tiles that share
     // the rows of A, the last one possibly narrower: for products with more than 256 tiles, whose
     // columns are dealt out evenly to 256 workgroups (one per compute unit; a kernel of this size
@@ -811,8 +814,8 @@ static int launch_skinny(const void* A, int lda, const bf16_t* W, int ldw, const
                                            hipFuncAttributeMaxDynamicSharedMemorySize,                 \
                                            static_cast<int>(staged_bytes));                            \
         if (e != hipSuccess) return static_cast<int>(e);                                               \
-        kernel<<<grid, block, staged_bytes, stream>>>(A, lda, W, ldw, bias, C, ldc, M, N, K, mode, gamma, beta, \
-                                                      eps, rows, col_blocks, row_blocks, 16, 1, nullptr, nullptr); \
+        kernel<<<grid, block, staged_bytes, stream>>>(W, ldw, N, K, M, col_blocks, row_blocks, 16, 1, A, lda, mode, \
+                                                      bias, C, ldc, gamma, beta, eps, rows, nullptr, nullptr); \
         break;                                                                                         \
     }
         switch (mt) {
@@ -840,8 +843,8 @@ static int launch_skinny(const void* A, int lda, const bf16_t* W, int ldw, const
             if (e != hipSuccess) return static_cast<int>(e);                                           \
             lds_allowed = true;                                                                        \
         }                                                                                              \
-        kernel<<<grid, block, smem, stream>>>(A, lda, W, ldw, bias, C, ldc, M, N, K, mode, gamma, beta, eps, rows, \
-                                              col_blocks, row_blocks, cols_per_wg, k_parts, part_sums,    \
+        kernel<<<grid, block, smem, stream>>>(W, ldw, N, K, M, col_blocks, row_blocks, cols_per_wg, k_parts, A, lda, \
+                                              mode, bias, C, ldc, gamma, beta, eps, rows, part_sums,      \
                                               part_counters);                                          \
     } while (0)
     if (split_k) {
