@@ -11,6 +11,7 @@
 #include "common.h"
 
 #include <algorithm>
+#include <type_traits>
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
@@ -345,10 +346,12 @@ gemm_bf16_skinny(// the first 16 dwords arrive in registers with the wavefront: 
     const int k_first = SPLIT_K ? (part * nw + wave) * 64 : 0;      // first k block of this wavefront
     const int k_stride = SPLIT_K ? nw * k_parts * 64 : 64;         // distance between its k blocks
     const size_t red_bytes = SPLIT_K ? static_cast<size_t>(nw) * T * 256 * sizeof(float) : 0;
-    constexpr int STAGE_BYTES = ASRC == A_GLOBAL ? 4096 : 2048;            // per wavefront: W block (+ A block)
+    // per wavefront: SB k blocks at a time change lanes through LDS, each NT weight tiles (+ the A block)
+    constexpr int SB = (ASRC == A_STAGED || (ASRC == A_GLOBAL && NT > 1) || U < 4) ? 1 : 2;
+    constexpr int STAGE_BYTES = SB * (NT * 2048 + (ASRC == A_GLOBAL ? 2048 : 0));
     float* red = reinterpret_cast<float*>(smem_raw);                       // [nw][T][256]
     bf16x8* stage_w = reinterpret_cast<bf16x8*>(smem_raw + red_bytes + static_cast<size_t>(wave) * STAGE_BYTES);
-    bf16x8* stage_a = stage_w + 128;                                       // (A_GLOBAL only)
+    bf16x8* stage_a = stage_w + SB * NT * 128;                             // (A_GLOBAL only)
     bf16_t* a_s = reinterpret_cast<bf16_t*>(smem_raw + red_bytes + static_cast<size_t>(nw) * STAGE_BYTES);   // [16*MT][K+8]
     const int a_stride = K + 8;
     // (fused norm only) the scale and shift vectors, loaded once per workgroup: [2][K] fp32
@@ -447,38 +450,63 @@ gemm_bf16_skinny(// the first 16 dwords arrive in registers with the wavefront: 
         __builtin_amdgcn_wave_barrier();
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
     };
-    auto mma_steps = [&](const Chunk& c, int u0, int k0) {
-        // through the wavefront's LDS region into the operand layout
-        bf16x8 af[2];
-        if (ASRC == A_GLOBAL) {
-            stage_a[lane] = c.a[A_TWO ? u0 : u0 / 2];
-            if (a_two) stage_a[64 + lane] = c.a[A_TWO ? u0 + 1 : 0];
-            wave_lds_order();
+    // CNT (1 or 2) consecutive k blocks of a chunk, slots u0.., first k index k0: all their pieces go
+    // through the wavefront's LDS region in one round trip (writes, then reads, then the MFMAs)
+    auto mma_blocks = [&](const Chunk& c, int u0, int k0, auto cnt_tag) {
+        constexpr int CNT = decltype(cnt_tag)::value;
+        static_assert(CNT <= SB, "staging room");
 #pragma unroll
-            for (int half = 0; half < 2; ++half) af[half] = stage_a[row16 * 8 + ((2 * kq + half) ^ rd_swz)];
+        for (int i = 0; i < CNT; ++i) {
+            if (ASRC == A_GLOBAL) {
+                stage_a[i * 128 + lane] = c.a[A_TWO ? u0 + 2 * i : (u0 + 2 * i) / 2];
+                if (a_two) stage_a[i * 128 + 64 + lane] = c.a[A_TWO ? u0 + 2 * i + 1 : 0];
+            }
+#pragma unroll
+            for (int t = 0; t < NT; ++t) {
+                stage_w[(i * NT + t) * 128 + lane] = c.b[t][u0 + 2 * i];
+                stage_w[(i * NT + t) * 128 + 64 + lane] = c.b[t][u0 + 2 * i + 1];
+            }
         }
+        wave_lds_order();
+        bf16x8 af[CNT][2], bf[CNT][NT][2];
 #pragma unroll
-        for (int t = 0; t < NT; ++t) {
-            stage_w[lane] = c.b[t][u0];
-            stage_w[64 + lane] = c.b[t][u0 + 1];
-            wave_lds_order();
-            bf16x8 bf[2];
-#pragma unroll
-            for (int half = 0; half < 2; ++half) bf[half] = stage_w[row16 * 8 + ((2 * kq + half) ^ rd_swz)];
-            wave_lds_order();
+        for (int i = 0; i < CNT; ++i)
 #pragma unroll
             for (int half = 0; half < 2; ++half) {
-                const int k = k0 + 16 * kq + 8 * half;
-                const bf16x8 b = k < K ? bf[half] : zero;
+                const int slot = row16 * 8 + ((2 * kq + half) ^ rd_swz);
+                if (ASRC == A_GLOBAL) af[i][half] = stage_a[i * 128 + slot];
+#pragma unroll
+                for (int t = 0; t < NT; ++t) bf[i][t][half] = stage_w[(i * NT + t) * 128 + slot];
+            }
+        wave_lds_order();
+#pragma unroll
+        for (int i = 0; i < CNT; ++i)
+#pragma unroll
+            for (int half = 0; half < 2; ++half) {
+                const int k = k0 + i * k_stride + 16 * kq + 8 * half;
                 const int kc = min(k, K - 8);
 #pragma unroll
-                for (int i = 0; i < MT; ++i) {
+                for (int mi = 0; mi < MT; ++mi) {
                     bf16x8 a;
-                    if (IN_LDS) a = *reinterpret_cast<const bf16x8*>(a_s + static_cast<size_t>(i * 16 + row16) * a_stride + kc);
-                    else a = af[half];
-                    acc[i * NT + t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, acc[i * NT + t], 0, 0, 0);
+                    if (IN_LDS) a = *reinterpret_cast<const bf16x8*>(a_s + static_cast<size_t>(mi * 16 + row16) * a_stride + kc);
+                    else a = af[i][half];
+#pragma unroll
+                    for (int t = 0; t < NT; ++t) {
+                        const bf16x8 b = k < K ? bf[i][t][half] : zero;
+                        acc[mi * NT + t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, acc[mi * NT + t], 0, 0, 0);
+                    }
                 }
             }
+    };
+    // `count` of the blocks in slots 0, 2, 4, ... of a chunk (count is uniform over the wavefront), k
+    // indices from k0 on
+    auto mma_some = [&](const Chunk& c, int count, int k0) {
+#pragma unroll
+        for (int h = 0; h < H; h += SB) {
+            if (SB == 2 && h + 1 < H && h + 1 < count)
+                mma_blocks(c, 2 * h, k0 + h * k_stride, std::integral_constant<int, SB>{});
+            else if (h < count)
+                mma_blocks(c, 2 * h, k0 + h * k_stride, std::integral_constant<int, 1>{});
         }
     };
     auto load_chunk = [&](Chunk& c, int chunk) {            // chunk index within this wavefront's blocks
@@ -488,10 +516,7 @@ gemm_bf16_skinny(// the first 16 dwords arrive in registers with the wavefront: 
         // here to be in flight together
         __builtin_amdgcn_sched_barrier(0);
     };
-    auto mma_chunk = [&](const Chunk& c, int chunk) {
-#pragma unroll
-        for (int h = 0; h < H; ++h) mma_steps(c, 2 * h, k_first + (chunk * H + h) * k_stride);
-    };
+    auto mma_chunk = [&](const Chunk& c, int chunk) { mma_some(c, H, k_first + chunk * H * k_stride); };
     // rows of the fp32 stream that this wavefront normalises (read before the weights are
     // requested: loads complete in order, and the row addresses depend on these)
     int src_row[2] = {0, 0};
@@ -629,9 +654,7 @@ gemm_bf16_skinny(// the first 16 dwords arrive in registers with the wavefront: 
     }
 
     if (n_chunks == 0) {
-#pragma unroll
-        for (int h = 0; h < H - 1; ++h)
-            if (h < n_blocks) mma_steps(c0, 2 * h, k_first + h * k_stride);
+        mma_some(c0, n_blocks, k_first);
     } else if (n_chunks == 1) {
         mma_chunk(c0, 0);
     } else if (n_chunks > 1) {
@@ -647,9 +670,7 @@ gemm_bf16_skinny(// the first 16 dwords arrive in registers with the wavefront: 
         // blocks left over: fewer than H, loaded together
         const int first = n_chunks * H, left = n_chunks > 0 ? n_blocks - first : 0;
         if (left > 0) load_left();
-#pragma unroll
-        for (int h = 0; h < H - 1; ++h)
-            if (h < left) mma_steps(c1, 2 * h, k_first + (first + h) * k_stride);
+        mma_some(c1, left, k_first + first * k_stride);
     }
     // accumulator layout of the 16x16 tile: register r of lane l holds row 4*(l/16) + r, column l%16
     if (!SPLIT_K) {
@@ -804,7 +825,8 @@ static int launch_skinny(const void* A, int lda, const bf16_t* W, int ldw, const
     const int col_blocks = split_k ? (N + cols_per_wg - 1) / cols_per_wg : (tiles + nw - 1) / nw;
     const dim3 grid((col_blocks + N_XCD - 1) / N_XCD * N_XCD * row_blocks, k_parts), block(nw * 64);
     size_t smem = split_k ? static_cast<size_t>(nw) * mt * (two_tiles ? 2 : 1) * 256 * sizeof(float) : 0;
-    smem += static_cast<size_t>(nw) * (LN_FUSED || staged ? 2048 : 4096);     // the wavefronts' transposition regions
+    // the wavefronts' transposition regions (two k blocks at a time where the kernel stages two)
+    smem += static_cast<size_t>(nw) * (staged ? 2048 : LN_FUSED ? (two_tiles ? 8192 : 4096) : (two_tiles ? 6144 : 8192));
     if (staged) {
         staged_bytes += smem;
 #define SKINNY_STAGED(MTV)                                                                             \
