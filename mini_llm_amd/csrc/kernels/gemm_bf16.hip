@@ -277,13 +277,15 @@ static void launch_tiled(const bf16_t* a, int lda, const bf16_t* w, int ldw, con
 }
 
 // ---------------------------------------------------------------------------------------------
-// Few rows (decode): M <= 64. The product is bound by streaming W once, and how fast a compute
+// Few rows (decode; up to 64 rows always, up to 256 while the workgroups stay few, see the
+// dispatch). The product is bound by streaming W once, and how fast a compute
 // unit streams depends on the shape of a wavefront's load: 8 consecutive lanes take one 128-byte
 // line (8 weight rows x 1 line per load) at up to 90 GB/s per unit, but the MFMA operand layout
 // (consecutive lanes = consecutive weight rows, 4 lines per 4 lanes) at under 40 (measured). So
-// the loads use the first shape and the 16-byte pieces change lanes through a 2 KB region of LDS
-// private to the wavefront (no barrier: LDS serves a wavefront's requests in order), swizzled so
-// that neither the writes nor the reads conflict. A workgroup owns 16 rows of the output (more
+// the loads use the first shape and the 16-byte pieces change lanes through a region of LDS
+// private to the wavefront (2 KB per weight tile and k block, up to two k blocks at a time; no
+// barrier: LDS serves a wavefront's requests in order), swizzled so that neither the writes nor
+// the reads conflict. A workgroup owns 16 rows of the output (more
 // rows: more workgroups per column range, placed on the same XCD so that the weights they share
 // come from its L2).
 //   SPLIT_K:  one workgroup per 16-column tile, its wavefronts split K (wavefront w takes the
