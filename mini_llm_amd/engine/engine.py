@@ -6,9 +6,9 @@ for every request whose newest token was in the batch, finished requests give th
 pages back. The reference's loop: /root/reference/src/runtime/scheduler.cpp:322-356;
 its offline use of the model: /root/reference/benchmarks/gpt2/bench_batch_vs_single_wall.cu:157-171.
 
-Steps that hold only decoded tokens run one ahead of the host: a step is launched with its
-input tokens taken on the device from the step before, and only then are that earlier step's
-tokens read. The GPU so never waits for the host between decode steps. What the host learns
+Steps run one ahead of the host: a step is launched with the decoded tokens among its
+inputs taken on the device from the step before, and only then are that earlier step's
+tokens read. The GPU so never waits for the host between steps. What the host learns
 late is only whether a token was the end of sequence; such a request has then run one step
 too many, whose token is dropped.
 """
@@ -20,7 +20,7 @@ from typing import Dict, List, Optional, Sequence, Union
 import torch
 
 from ..models import load_model
-from ..sampling.sampler import Sampler, SamplingParams, uniform01
+from ..sampling.sampler import SamplingParams, uniform01
 from .scheduler import Scheduler
 from .step import ModelRunner, StepEntry
 
@@ -32,7 +32,7 @@ class EngineOptions:
     max_batch_num: int = 16             # sequences in one step (reference: MAX_BATCH_NUM, constants.h:20)
     max_tokens_per_step: int = 2048     # token budget of one step
     prefill_chunk: int = 512            # longest prompt portion
-    overlap_decode: bool = True         # launch a decode step before the previous one's tokens are read
+    overlap_decode: bool = True         # launch a step before the previous one's tokens are read
 
 
 @dataclass
@@ -66,7 +66,6 @@ class Engine:
         self.runner = ModelRunner(model, o.kv_block_size, o.total_kv_blocks, o.max_batch_num)
         self.scheduler = Scheduler(self.runner.manager, o.max_batch_num, o.max_tokens_per_step,
                                    o.prefill_chunk, model.max_positions)
-        self.sampler = Sampler(model.device, o.max_batch_num)
         self.eos_token_id = model.config.eos_token_id
         self.requests: Dict[int, _Request] = {}
         self._next_id = 0
@@ -133,7 +132,7 @@ class Engine:
         return (not r.params.ignore_eos) and self.eos_token_id is not None and tok == self.eos_token_id
 
     def _collect(self) -> List[RequestOutput]:
-        """Reads the tokens of the decode step in flight, if any. A request that an earlier token
+        """Reads the tokens of the step in flight, if any. A request that an earlier token
         already ended (seen late) or that was aborted drops its token."""
         if self._pending is None:
             return []
@@ -166,8 +165,12 @@ class Engine:
             return outputs + self._collect()
         sampled = [e for e in plan if e.want_last]
         fast = (self.runner.fast_decode and len(sampled) == len(plan) and all(e.n_tokens == 1 for e in plan))
-        if not (fast and self.options.overlap_decode):
-            # the host must know every token it feeds: read what is in flight first
+        # only a single decoded token can be fed on the device; a portion that reaches past what the
+        # host has read (a request recomputed right after it was preempted) waits for the read
+        unread_portion = any(e.n_tokens > 1 and e.start + e.n_tokens > len(self.requests[e.request_id].tokens)
+                             for e in plan)
+        if not self.options.overlap_decode or unread_portion:
+            # the host knows every token it feeds: read what is in flight first
             outputs += self._collect()
             live = [e for e in plan if not self.requests[e.request_id].finished]
             if len(live) != len(plan):        # ended by a token just read; the scheduler dropped them too
@@ -180,40 +183,40 @@ class Engine:
             temps.append(r.params.temperature)
             us.append(uniform01(r.params.seed, r.n_launched) if r.params.temperature > 0 else 0.0)
             r.n_launched += 1
+        # A token that the step in flight has sampled and the host has not read is fed on the device:
+        # its row among that step's sampled tokens stands in for it.
+        in_flight = {rid: i for i, (rid, _) in enumerate(self._pending[1])} if self._pending else {}
         if fast:
             # every entry is one decoded token: the whole step runs from static buffers (a HIP graph)
-            in_flight = {rid: i for i, (rid, _) in enumerate(self._pending[1])} if self._pending else {}
             toks, src = [], []
             for e in plan:
                 r = self.requests[e.request_id]
                 if e.start < len(r.tokens):
                     toks.append(r.tokens[e.start])
                     src.append(-1)
-                else:                          # sampled by the step in flight, not read yet
+                else:
                     toks.append(0)
                     src.append(in_flight[e.request_id])
             handle = self.runner.launch_decode([e.request_id for e in plan], toks, src, temps, us)
-            self.scheduler.commit()
-            # the scheduler moves on as if no token were the end of sequence; `_collect` corrects it
-            rows = [(e.request_id, self.scheduler.on_token(e.request_id, False)) for e in plan]
-            outputs += self._collect()
-            self._pending = (handle, rows)
-            if not self.options.overlap_decode:
-                outputs += self._collect()
-            return outputs
-        entries = []
-        for e in plan:
-            r = self.requests[e.request_id]
-            entries.append(StepEntry(e.request_id, r.tokens[e.start:e.start + e.n_tokens],
-                                     [e.n_tokens - 1] if e.want_last else []))
-        logits = self.runner.step(entries, manage_cache=False)
+        else:
+            entries, feed = [], []
+            for e in plan:
+                r = self.requests[e.request_id]
+                known = r.tokens[e.start:e.start + e.n_tokens]
+                if len(known) < e.n_tokens:        # a decoded token still in flight
+                    known, row = [0], in_flight[e.request_id]
+                else:
+                    row = -1
+                entries.append(StepEntry(e.request_id, known, [e.n_tokens - 1] if e.want_last else []))
+                feed.append(row)
+            handle = self.runner.launch_step(entries, feed, temps, us)
         self.scheduler.commit()
-        tokens = self.sampler.sample(logits, temps, us) if sampled else []
-        for e, tok in zip(sampled, tokens):
-            r = self.requests[e.request_id]
-            r.tokens.append(tok)
-            r.finished = self.scheduler.on_token(e.request_id, self._is_eos(r, tok))
-            outputs.append(RequestOutput(e.request_id, tok, r.finished))
+        # the scheduler moves on as if no token were the end of sequence; `_collect` corrects it
+        rows = [(e.request_id, self.scheduler.on_token(e.request_id, False)) for e in sampled]
+        outputs += self._collect()
+        self._pending = (handle, rows) if handle is not None else None
+        if not self.options.overlap_decode:
+            outputs += self._collect()
         return outputs
 
     # -- offline generation --------------------------------------------------------------

@@ -19,6 +19,7 @@ import numpy as np
 import torch
 
 from ..cache.manager import CacheStorage
+from ..sampling.sampler import Sampler
 
 
 @dataclass
@@ -113,8 +114,12 @@ class ModelRunner:
         self.page_size = page_size
         self.n_pages = n_pages
         self._staging = _Staging(self.device)
+        self._staging_src = _Staging(self.device)      # rows that feed tokens from the previous launch
         self._graphs: Dict[tuple, "DecodeGraph"] = {}
-        self._tok_out: Optional[torch.Tensor] = None      # sampled tokens of the last launched decode step
+        self._tok_out: Optional[torch.Tensor] = None      # sampled tokens of the last launched step
+        self._host_tok = None
+        self._turn_out = 0
+        self.sampler = Sampler(self.device, max_num_seqs)
         # Pure-decode batches may run from static buffers (`launch_decode`) unless a part of the model
         # plans on the host; on the GPU those steps are captured and replayed as HIP graphs.
         self.fast_decode = bool(getattr(model, "graph_safe", True))
@@ -228,6 +233,65 @@ class ModelRunner:
                 mgr.commit(e.request_id, mgr.length(e.request_id) + len(e.tokens))
         return logits
 
+    # -- steps whose sampled tokens stay on the device until asked for -------------------------
+    def _room_for_tokens(self, n_rows: int) -> None:
+        if self._tok_out is None or self._tok_out.numel() < n_rows:
+            # (sized for the most requests the cache manager admits, so this happens once)
+            n = max(n_rows, -(-self.manager.n_state_slots // 8) * 8, 8)
+            grown = torch.zeros(n, dtype=torch.int32, device=self.device)
+            if self._tok_out is not None:
+                grown[:self._tok_out.numel()].copy_(self._tok_out)     # tokens a later launch may still take
+                self._graphs.clear()                                   # captured graphs hold the old address
+            self._tok_out = grown
+
+    def launch_step(self, entries: Sequence[StepEntry], feed_rows: Sequence[int],
+                    temperatures: Sequence[float], uniforms: Sequence[float]) -> Optional["PendingTokens"]:
+        """Starts one step of any mixture (pages already reserved; the caller commits the lengths)
+        and returns at once. Entry i's single token is taken from row ``feed_rows[i]`` of what the
+        previous launch sampled where that is >= 0 (the host need not have read it); other entries
+        bring their tokens. One token is sampled for every wanted place, in the order of the
+        entries, and left on the device for the next launch; ``PendingTokens.result()`` waits for
+        them. None if nothing is wanted."""
+        from ..kernels import ops
+        ctx = self.build_context(entries)
+        if any(f >= 0 for f in feed_rows):
+            src = np.full(ctx.n_tokens, -1, dtype=np.int32)
+            t = 0
+            for e, f in zip(entries, feed_rows):
+                if f >= 0:
+                    if len(e.tokens) != 1:
+                        raise StepError("only a single token can come from the previous launch")
+                    src[t] = f
+                t += len(e.tokens)
+            if self._tok_out is None:
+                raise StepError("no earlier launch has sampled a token")
+            host, buf = self._staging_src.take(ctx.n_tokens)
+            host[:] = src
+            ops.select_tokens(ctx.token_ids, _Staging.upload(buf, ctx.n_tokens)[:ctx.n_tokens], self._tok_out)
+        logits = self.model.forward(ctx, self.cache)
+        if logits is None:
+            return None
+        n = logits.shape[0]
+        self._room_for_tokens(n)
+        out = self._tok_out[:n]
+        self.sampler.choose(logits, temperatures, uniforms, out)
+        self._turn_out ^= 1
+        host_out = self._host_tokens(n)[self._turn_out]
+        host_out[:n].copy_(out, non_blocking=True)
+        event = None
+        if self.device.type == "cuda":
+            event = torch.cuda.Event()
+            event.record()
+        return PendingTokens(host_out, n, event)
+
+    def _host_tokens(self, n: int):
+        # two host buffers in turn: one may still be unread when the next step's copy is queued
+        if self._host_tok is None or self._host_tok[0].numel() < n:
+            cap = max(n, 64)
+            pin = self.device.type == "cuda"
+            self._host_tok = [torch.zeros(cap, dtype=torch.int32, pin_memory=pin) for _ in range(2)]
+        return self._host_tok
+
     # -- decode steps through a captured HIP graph ------------------------------------------
     def launch_decode(self, request_ids: Sequence[int], tokens: Sequence[int], src_rows: Sequence[int],
                       temperatures: Optional[Sequence[float]] = None,
@@ -241,14 +305,7 @@ class ModelRunner:
         B = len(request_ids)
         greedy = temperatures is None or all(t <= 0 for t in temperatures)
         bucket = B if B <= 8 else -(-B // 8) * 8
-        if self._tok_out is None or self._tok_out.numel() < bucket:
-            # (sized for the most requests the cache manager admits, so this happens once)
-            n = max(bucket, -(-self.manager.n_state_slots // 8) * 8, 8)
-            grown = torch.zeros(n, dtype=torch.int32, device=self.device)
-            if self._tok_out is not None:
-                grown[:self._tok_out.numel()].copy_(self._tok_out)     # tokens a later launch may still take
-                self._graphs.clear()                                   # captured graphs hold the old address
-            self._tok_out = grown
+        self._room_for_tokens(bucket)
         key = (bucket, greedy)
         g = self._graphs.get(key)
         if g is None:

@@ -54,27 +54,44 @@ class Sampler:
     def __init__(self, device, max_rows: int = 64):
         self.device = torch.device(device)
         self._cap = 0
+        self._turn = 0
         self._grow(max_rows)
 
     def _grow(self, n: int) -> None:
         if n <= self._cap:
             return
         self._cap = max(n, 2 * self._cap)
-        pin = self.device.type == "cuda"
-        self._h = torch.empty((2, self._cap), dtype=torch.float32, pin_memory=pin)
+        on_gpu = self.device.type == "cuda"
+        # two pinned buffers in turn: the host fills one while the copy out of the other may still be queued
+        self._h = [torch.empty((2, self._cap), dtype=torch.float32, pin_memory=on_gpu) for _ in range(2)]
+        self._copied = [torch.cuda.Event() if on_gpu else None for _ in range(2)]
         self._d = torch.empty((2, self._cap), dtype=torch.float32, device=self.device)
         self._out = torch.empty(self._cap, dtype=torch.int32, device=self.device)
 
+    def choose(self, logits: torch.Tensor, temperatures: Sequence[float], uniforms: Sequence[float],
+               out: torch.Tensor) -> None:
+        """Queues the choice of one token per row of ``logits`` into ``out`` (int32, on the device)
+        and returns without waiting for it."""
+        n = logits.shape[0]
+        assert len(temperatures) == n and len(uniforms) == n and out.numel() >= n
+        if all(t <= 0 for t in temperatures):
+            ops.argmax(logits, out[:n])
+            return
+        self._grow(n)
+        self._turn ^= 1
+        h, copied = self._h[self._turn], self._copied[self._turn]
+        if copied is not None:
+            copied.synchronize()          # the copy that last read this buffer is done
+        hv = h.numpy()
+        hv[0, :n] = temperatures
+        hv[1, :n] = uniforms
+        self._d.copy_(h, non_blocking=True)
+        if copied is not None:
+            copied.record()
+        ops.sample(logits, self._d[0], self._d[1], out[:n])
+
     def sample(self, logits: torch.Tensor, temperatures: Sequence[float], uniforms: Sequence[float]) -> List[int]:
         n = logits.shape[0]
-        assert len(temperatures) == n and len(uniforms) == n
         self._grow(n)
-        if all(t <= 0 for t in temperatures):
-            ops.argmax(logits, self._out[:n])
-        else:
-            h = self._h.numpy()
-            h[0, :n] = temperatures
-            h[1, :n] = uniforms
-            self._d.copy_(self._h, non_blocking=False)
-            ops.sample(logits, self._d[0], self._d[1], self._out[:n])
+        self.choose(logits, temperatures, uniforms, self._out)
         return self._out[:n].tolist()
