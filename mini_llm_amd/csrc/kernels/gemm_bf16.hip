@@ -22,9 +22,10 @@ typedef float f32x16 __attribute__((ext_vector_type(16)));
 // Many rows (prefill): WM x WN wavefronts, each TM x TN MFMA tiles of 32x32. LDS is double
 // buffered (one barrier per k tile), global loads run DEPTH-1 tiles ahead in rotating register
 // sets, per-thread pointers only advance, and blocks that lie fully inside the matrices take an
-// edge-free path chosen at compile time. The weight fragment is the MFMA's A operand, so a lane's
-// accumulator registers hold 4 consecutive columns of one output row: the epilogue stores them
-// as one 8- or 16-byte access.
+// edge-free path chosen at compile time. Within a tile the memory instructions are spread between
+// the MFMA groups of its k steps, so that the matrix units work while they queue. The weight
+// fragment is the MFMA's A operand, so a lane's accumulator registers hold 4 consecutive columns
+// of one output row; the epilogue turns that, through LDS, into stores of whole rows.
 // ---------------------------------------------------------------------------------------------
 // Optional second destination of a plain bf16 store: columns [q_cols, q_cols + kv_dim) of output row
 // m also go to row slots[m] of the key pages and the next kv_dim columns to the value pages (the
@@ -78,9 +79,16 @@ gemm_bf16_mfma(const bf16_t* __restrict__ A, int lda, const bf16_t* __restrict__
     constexpr int BM = WM * TM * 32, BN = WN * TN * 32;
     constexpr int STRIDE = BKP + 8;
     constexpr int CPR = BKP / 8;                      // 16-byte chunks per row
-    constexpr int A_CH = (BM * CPR + NT - 1) / NT, W_CH = (BN * CPR + NT - 1) / NT;
-    __shared__ __attribute__((aligned(16))) bf16_t As[2][BM * STRIDE];
-    __shared__ __attribute__((aligned(16))) bf16_t Ws[2][BN * STRIDE];
+    constexpr int KS = BKP / 16;                      // MFMA k steps per tile
+    constexpr int A_CH = (BM * CPR + NT - 1) / NT, W_CH = (BN * CPR + NT - 1) / NT, N_LOADS = A_CH + W_CH;
+    constexpr int EPI_STRIDE = 36;                    // floats per row of a 32x32 sub-tile in the epilogue
+    static_assert(KS % 2 == 0 && DEPTH >= 3, "the k loop alternates two fragment sets and three register sets");
+    static_assert(2 * (BM + BN) * STRIDE * 2 >= WM * WN * 32 * EPI_STRIDE * 4, "the tiles' LDS holds the epilogue's regions");
+    // one array: two buffers of A rows, two of W rows; the epilogue reuses it, a region per wavefront
+    __shared__ __attribute__((aligned(16))) bf16_t smem[2 * (BM + BN) * STRIDE];
+    __shared__ __attribute__((aligned(16))) float bias_s[BN];
+    bf16_t (*As)[BM * STRIDE] = reinterpret_cast<bf16_t (*)[BM * STRIDE]>(smem);
+    bf16_t (*Ws)[BN * STRIDE] = reinterpret_cast<bf16_t (*)[BN * STRIDE]>(smem + 2 * BM * STRIDE);
 
     const int tid = threadIdx.x, wave = tid / 64, lane = tid % 64;
     const int wm = wave / WN, wn = wave % WN;
@@ -92,6 +100,8 @@ gemm_bf16_mfma(const bf16_t* __restrict__ A, int lda, const bf16_t* __restrict__
     const int tm = (xcd / xn) * rect_m + local / rect_n, tn = (xcd % xn) * rect_n + local % rect_n;
     if (local >= rect_m * rect_n || tm >= tiles_m || tn >= tiles_n) return;      // padding of the grid
     const int m0 = tm * BM, n0 = tn * BN;
+    if (bias != nullptr)         // read again in the epilogue, after the k loop's barriers
+        for (int c = tid; c < BN; c += NT) bias_s[c] = n0 + c < N ? bias[n0 + c] : 0.f;
 
     f32x16 acc[TM][TN];
 #pragma unroll
@@ -124,28 +134,32 @@ gemm_bf16_mfma(const bf16_t* __restrict__ A, int lda, const bf16_t* __restrict__
         uint4 ra[A_CH], rw[W_CH];
     };
     TileRegs regs[DEPTH];
-    // Every thread issues every load of every fetch, with the address clamped into the matrix:
-    // the number of loads in flight is then the same on every path through the loop, and only so
-    // does the compiler wait for exactly the tile that is staged next while later ones stay in
-    // flight (a skipped load on any path makes it wait for all of them). What lies outside the
-    // matrices is zeroed when the tile is staged.
-    auto fetch = [&](TileRegs& t, int k0) {
+    // A tile's loads and its LDS writes are cut into KS portions (portion `part`, or all of them
+    // with part < 0), so that they can be issued between the MFMA groups of the tile in work.
+    // Every thread issues every load, with the address clamped into the matrix: the number of loads
+    // in flight is then the same on every path through the loop, and only so does the compiler wait
+    // for exactly the registers that are staged next while later loads stay in flight. What lies
+    // outside the matrices is zeroed when the tile is staged.
+    auto fetch = [&](TileRegs& t, int k0, int part) {
 #pragma unroll
         for (int i = 0; i < A_CH; ++i) {
+            if (part >= 0 && i * KS / N_LOADS != part) continue;
             const int kc8 = (tid + i * NT) % CPR * 8;
             const int k = EDGE ? min(k0 + kc8, K - 8) - kc8 : k0;
             t.ra[i] = *reinterpret_cast<const uint4*>(pa[i] + k);
         }
 #pragma unroll
         for (int i = 0; i < W_CH; ++i) {
+            if (part >= 0 && (A_CH + i) * KS / N_LOADS != part) continue;
             const int kc8 = (tid + i * NT) % CPR * 8;
             const int k = EDGE ? min(k0 + kc8, K - 8) - kc8 : k0;
             t.rw[i] = *reinterpret_cast<const uint4*>(pw[i] + k);
         }
     };
-    auto stage = [&](const TileRegs& t, int buf, int k0) {
+    auto stage = [&](const TileRegs& t, int buf, int k0, int part) {
 #pragma unroll
         for (int i = 0; i < A_CH; ++i) {
+            if (part >= 0 && i * KS / N_LOADS != part) continue;
             const int kc8 = (tid + i * NT) % CPR * 8;
             const bool ok = !EDGE || (va[i] && k0 + kc8 < K);
             if (BM * CPR % NT == 0 || tid + i * NT < BM * CPR)
@@ -153,96 +167,129 @@ gemm_bf16_mfma(const bf16_t* __restrict__ A, int lda, const bf16_t* __restrict__
         }
 #pragma unroll
         for (int i = 0; i < W_CH; ++i) {
+            if (part >= 0 && (A_CH + i) * KS / N_LOADS != part) continue;
             const int kc8 = (tid + i * NT) % CPR * 8;
             const bool ok = !EDGE || (vw[i] && k0 + kc8 < K);
             if (BN * CPR % NT == 0 || tid + i * NT < BN * CPR)
                 *reinterpret_cast<uint4*>(&Ws[buf][lw[i]]) = ok ? t.rw[i] : make_uint4(0, 0, 0, 0);
         }
     };
+    // two sets of MFMA operands: the fragments of k step ks+1 are read while step ks multiplies
     const int a_off = (wm * TM * 32 + lane % 32) * STRIDE + 8 * (lane / 32);
     const int w_off = (wn * TN * 32 + lane % 32) * STRIDE + 8 * (lane / 32);
-    auto compute = [&](int buf) {
+    bf16x8 fa[2][TM], fb[2][TN];
+    auto read_frags = [&](int buf, int ks, int set) {
 #pragma unroll
-        for (int ks = 0; ks < BKP / 16; ++ks) {
-            bf16x8 a[TM], b[TN];
+        for (int i = 0; i < TM; ++i)
+            fa[set][i] = *reinterpret_cast<const bf16x8*>(&As[buf][a_off + i * 32 * STRIDE + ks * 16]);
 #pragma unroll
-            for (int i = 0; i < TM; ++i)
-                a[i] = *reinterpret_cast<const bf16x8*>(&As[buf][a_off + i * 32 * STRIDE + ks * 16]);
+        for (int j = 0; j < TN; ++j)
+            fb[set][j] = *reinterpret_cast<const bf16x8*>(&Ws[buf][w_off + j * 32 * STRIDE + ks * 16]);
+    };
+    auto mma = [&](int set) {
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
 #pragma unroll
             for (int j = 0; j < TN; ++j)
-                b[j] = *reinterpret_cast<const bf16x8*>(&Ws[buf][w_off + j * 32 * STRIDE + ks * 16]);
-#pragma unroll
-            for (int i = 0; i < TM; ++i)
-#pragma unroll
-                for (int j = 0; j < TN; ++j)
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(b[j], a[i], acc[i][j], 0, 0, 0);
-        }
+                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[set][j], fa[set][i], acc[i][j], 0, 0, 0);
     };
 
     const int nk = (K + BKP - 1) / BKP;
     // tiles 0 .. DEPTH-2 are requested (past the last tile: the last one again, never used);
     // tile 0 is staged
 #pragma unroll
-    for (int d = 0; d < DEPTH - 1; ++d) fetch(regs[d], min(d, nk - 1) * BKP);
-    stage(regs[0], 0, 0);
+    for (int d = 0; d < DEPTH - 1; ++d) fetch(regs[d], min(d, nk - 1) * BKP, -1);
+    stage(regs[0], 0, 0, -1);
     lds_barrier();
+    read_frags(0, 0, 0);
     // Whole groups of DEPTH tiles run without a branch in the body (a load or a use of it under a
     // condition would be moved or waited for conservatively); the last nk % DEPTH tiles, which
-    // fetch nothing any more, follow under conditions.
+    // fetch nothing any more, follow under conditions. In the body, tile t is in LDS buffer t%2
+    // and every k step issues, in this order: its share of the loads of tile t+DEPTH-1, its share
+    // of the LDS writes of tile t+1 (into the other buffer, whose last readers passed the barrier
+    // that ended the previous iteration), the fragment reads of the next k step, its MFMAs. The
+    // scheduling barriers keep that order: left alone, the compiler gathers the loads at the end
+    // of the iteration and the writes at its start, and a wavefront then issues nothing else while
+    // its memory instructions queue up.
     const int n_groups = nk / DEPTH, n_tail = nk % DEPTH;
     for (int g = 0; g < n_groups; ++g) {
 #pragma unroll
         for (int d = 0; d < DEPTH; ++d) {
             const int t = g * DEPTH + d;
-            // tile t is in LDS buffer t%2; tile t+1 goes to the other buffer (its last readers
-            // passed the barrier that ended the previous iteration)
-            fetch(regs[(d + DEPTH - 1) % DEPTH], min(t + DEPTH - 1, nk - 1) * BKP);
-            stage(regs[(d + 1) % DEPTH], (t + 1) & 1, (t + 1) * BKP);
-            compute(t & 1);
+            const int k_fetch = min(t + DEPTH - 1, nk - 1) * BKP;
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks) {
+                fetch(regs[(d + DEPTH - 1) % DEPTH], k_fetch, ks);
+                stage(regs[(d + 1) % DEPTH], (t + 1) & 1, (t + 1) * BKP, ks);
+                if (ks + 1 < KS) read_frags(t & 1, ks + 1, (ks + 1) & 1);
+                mma(ks & 1);
+                __builtin_amdgcn_sched_barrier(0);
+            }
             lds_barrier();
+            read_frags((t + 1) & 1, 0, 0);
         }
     }
 #pragma unroll
     for (int d = 0; d < DEPTH - 1; ++d) {
         const int t = n_groups * DEPTH + d;
         if (d < n_tail) {
-            if (d + 1 < n_tail) stage(regs[(d + 1) % DEPTH], (t + 1) & 1, (t + 1) * BKP);
-            compute(t & 1);
+            if (d + 1 < n_tail) stage(regs[(d + 1) % DEPTH], (t + 1) & 1, (t + 1) * BKP, -1);
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks) {
+                if (ks + 1 < KS) read_frags(t & 1, ks + 1, (ks + 1) & 1);
+                mma(ks & 1);
+            }
             lds_barrier();
+            if (d + 1 < n_tail) read_frags((t + 1) & 1, 0, 0);
         }
     }
 
     // With the weights as the A operand, register r of lane l holds output row l%32 and column
-    // 8*(r/4) + 4*(l/32) + r%4 of the 32x32 tile: 4 consecutive columns per register quad.
+    // 8*(r/4) + 4*(l/32) + r%4 of a 32x32 sub-tile. Stored from there, one instruction would touch
+    // 16 bytes in each of 32 rows. So each sub-tile goes through the wavefront's own region of LDS
+    // (the tiles are done with theirs): written as the MFMA left it, read back with 8 lanes per row,
+    // and a store instruction then covers 8 whole rows of the sub-tile.
     const bool vec = (ldc % 4 == 0) && ((reinterpret_cast<uintptr_t>(C) & 15) == 0);
+    float* epi = reinterpret_cast<float*>(smem) + wave * (32 * EPI_STRIDE);
 #pragma unroll
     for (int i = 0; i < TM; ++i) {
-        const int m = m0 + (wm * TM + i) * 32 + lane % 32;
-        if (EDGE && m >= M) continue;
-        const int slot = (MODE == EPI_STORE && kv.slots != nullptr) ? kv.slots[m] : -1;
 #pragma unroll
         for (int j = 0; j < TN; ++j) {
+            wave_lds_sync();          // the reads of the sub-tile before are done
 #pragma unroll
-            for (int g = 0; g < 4; ++g) {
-                const int n = n0 + (wn * TN + j) * 32 + 8 * g + 4 * (lane / 32);
-                if (EDGE && n >= N) continue;
+            for (int g = 0; g < 4; ++g)
+                *reinterpret_cast<float4*>(&epi[(lane % 32) * EPI_STRIDE + 8 * g + 4 * (lane / 32)]) =
+                    make_float4(acc[i][j][4 * g], acc[i][j][4 * g + 1], acc[i][j][4 * g + 2], acc[i][j][4 * g + 3]);
+            wave_lds_sync();
+            const int mb = m0 + (wm * TM + i) * 32, nb = n0 + (wn * TN + j) * 32;
+#pragma unroll
+            for (int it = 0; it < 4; ++it) {
+                const int r = it * 8 + lane / 8, c4 = (lane % 8) * 4;
+                const int m = mb + r, n = nb + c4;
+                if (EDGE && (m >= M || n >= N)) continue;
                 const int n_left = EDGE ? min(4, N - n) : 4;
-                float v[4];
-#pragma unroll
-                for (int e = 0; e < 4; ++e) v[e] = acc[i][j][4 * g + e] + ((bias && e < n_left) ? bias[n + e] : 0.f);
+                const float4 t = *reinterpret_cast<const float4*>(&epi[r * EPI_STRIDE + c4]);
+                float v[4] = {t.x, t.y, t.z, t.w};
+                if (bias != nullptr) {
+                    const float4 b = *reinterpret_cast<const float4*>(&bias_s[nb - n0 + c4]);
+                    v[0] += b.x; v[1] += b.y; v[2] += b.z; v[3] += b.w;
+                }
                 store4<MODE>(C, static_cast<size_t>(m) * ldc + n, v, vec, n_left);
-                if (MODE == EPI_STORE && slot >= 0 && n >= kv.q_cols) {
-                    // q_cols and kv_dim are multiples of 4: the four columns lie in one of the two parts
-                    const int c = n - kv.q_cols;
-                    bf16_t* dst = (c < kv.kv_dim ? kv.k_pages + c : kv.v_pages + (c - kv.kv_dim)) +
-                                  static_cast<size_t>(slot) * kv.kv_dim;
-                    if (n_left >= 4) {
-                        uint2 pk;
-                        pk.x = pack_bf16x2(v[0], v[1]);
-                        pk.y = pack_bf16x2(v[2], v[3]);
-                        *reinterpret_cast<uint2*>(dst) = pk;
-                    } else {
-                        for (int e = 0; e < n_left; ++e) dst[e] = float_to_bf16(v[e]);
+                if (MODE == EPI_STORE && kv.slots != nullptr && n >= kv.q_cols) {
+                    const int slot = kv.slots[m];
+                    if (slot >= 0) {
+                        // q_cols and kv_dim are multiples of 4: the four columns lie in one of the two parts
+                        const int c = n - kv.q_cols;
+                        bf16_t* dst = (c < kv.kv_dim ? kv.k_pages + c : kv.v_pages + (c - kv.kv_dim)) +
+                                      static_cast<size_t>(slot) * kv.kv_dim;
+                        if (n_left >= 4) {
+                            uint2 pk;
+                            pk.x = pack_bf16x2(v[0], v[1]);
+                            pk.y = pack_bf16x2(v[2], v[3]);
+                            *reinterpret_cast<uint2*>(dst) = pk;
+                        } else {
+                            for (int e = 0; e < n_left; ++e) dst[e] = float_to_bf16(v[e]);
+                        }
                     }
                 }
             }
@@ -933,19 +980,28 @@ static int gemm_bf16_dispatch(const void* A, int lda, const void* W, int ldw, co
     } else if (M <= 32) {
         launch_tiled<1, 4, 1, 1, 64, 3>(a, lda, w, ldw, bias, C, ldc, M, N, K, mode, stream, kv);
     } else {
-        // Tile choice, measured at 2048 rows on GPT-2 shapes: a large tile moves fewer bytes per
-        // flop, but pays only when its workgroups fill the 256 compute units in one round (or in
-        // many); otherwise 64x64 tiles, several of them resident per unit, balance best.
-        auto blocks = [&](int bm, int bn) { return static_cast<long>((M + bm - 1) / bm) * ((N + bn - 1) / bn); };
-        auto one_round = [](long n) { return n >= 192 && n <= 256; };
-        if (one_round(blocks(128, 192))) {
-            launch_tiled<4, 2, 1, 3, 32, 4>(a, lda, w, ldw, bias, C, ldc, M, N, K, mode, stream, kv);     // 128x192
-        } else if (blocks(128, 128) >= 512 || one_round(blocks(128, 128))) {
-            launch_tiled<2, 2, 2, 2, 32, 6>(a, lda, w, ldw, bias, C, ldc, M, N, K, mode, stream, kv);     // 128x128
-        } else if (one_round(blocks(64, 96))) {
-            launch_tiled<2, 3, 1, 1, 64, 3>(a, lda, w, ldw, bias, C, ldc, M, N, K, mode, stream, kv);     // 64x96
-        } else {
-            launch_tiled<2, 2, 1, 1, 64, 4>(a, lda, w, ldw, bias, C, ldc, M, N, K, mode, stream, kv);     // 64x64
+        // Tile choice. The compute units run the workgroups in rounds of 256, and a workgroup's time
+        // grows with its tile's area, less so for large tiles (they move fewer bytes per flop). So
+        // each shape is priced as rounds x area / efficiency, the efficiencies fitted to measurements
+        // at 2048 rows on the products of GPT-2 small to XL, and the cheapest runs. Few workgroups
+        // (one round for every shape) thus take the smallest tiles, which spread over more units.
+        struct Shape { int bm, bn; double efficiency; };
+        static const Shape shapes[] = {{128, 256, 1.05}, {128, 192, 1.0}, {128, 128, 0.9},
+                                       {64, 128, 0.7},   {64, 96, 0.65},  {64, 64, 0.55}};
+        int best = 0;
+        double best_cost = 1e300;
+        for (int c = 0; c < 6; ++c) {
+            const long blocks = static_cast<long>((M + shapes[c].bm - 1) / shapes[c].bm) * ((N + shapes[c].bn - 1) / shapes[c].bn);
+            const double cost = static_cast<double>((blocks + 255) / 256) * shapes[c].bm * shapes[c].bn / shapes[c].efficiency;
+            if (cost < best_cost) { best_cost = cost; best = c; }
+        }
+        switch (best) {
+            case 0: launch_tiled<2, 4, 2, 2, 64, 4>(a, lda, w, ldw, bias, C, ldc, M, N, K, mode, stream, kv); break;
+            case 1: launch_tiled<4, 2, 1, 3, 64, 3>(a, lda, w, ldw, bias, C, ldc, M, N, K, mode, stream, kv); break;
+            case 2: launch_tiled<2, 4, 2, 1, 64, 3>(a, lda, w, ldw, bias, C, ldc, M, N, K, mode, stream, kv); break;
+            case 3: launch_tiled<1, 4, 2, 1, 64, 4>(a, lda, w, ldw, bias, C, ldc, M, N, K, mode, stream, kv); break;
+            case 4: launch_tiled<2, 3, 1, 1, 64, 3>(a, lda, w, ldw, bias, C, ldc, M, N, K, mode, stream, kv); break;
+            default: launch_tiled<2, 2, 1, 1, 64, 4>(a, lda, w, ldw, bias, C, ldc, M, N, K, mode, stream, kv); break;
         }
     }
     MLLM_LAUNCH_CHECK();
