@@ -999,8 +999,8 @@ static int gemm_bf16_dispatch(const void* A, int lda, const void* W, int ldw, co
             case 0: launch_tiled<2, 4, 2, 2, 64, 4>(a, lda, w, ldw, bias, C, ldc, M, N, K, mode, stream, kv); break;
             case 1: launch_tiled<4, 2, 1, 3, 64, 3>(a, lda, w, ldw, bias, C, ldc, M, N, K, mode, stream, kv); break;
             case 2: launch_tiled<2, 4, 2, 1, 64, 3>(a, lda, w, ldw, bias, C, ldc, M, N, K, mode, stream, kv); break;
-            case 3: launch_tiled<1, 4, 2, 1, 64, 4>(a, lda, w, ldw, bias, C, ldc, M, N, K, mode, stream, kv); break;
-            case 4: launch_tiled<2, 3, 1, 1, 64, 3>(a, lda, w, ldw, bias, C, ldc, M, N, K, mode, stream, kv); break;
+            case 3: launch_tiled<2, 4, 1, 1, 64, 4>(a, lda, w, ldw, bias, C, ldc, M, N, K, mode, stream, kv); break;
+            case 4: launch_tiled<2, 3, 1, 1, 64, 5>(a, lda, w, ldw, bias, C, ldc, M, N, K, mode, stream, kv); break;
             default: launch_tiled<2, 2, 1, 1, 64, 4>(a, lda, w, ldw, bias, C, ldc, M, N, K, mode, stream, kv); break;
         }
     }
