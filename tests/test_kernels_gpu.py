@@ -116,12 +116,14 @@ def test_linear(ops, dtype, M, N, K, epi):
 
 @pytest.mark.parametrize("M,N,K", [(2000, 2300, 776),      # 128x192 tiles, one round, ragged in M, N and K
                                    (2048, 3072, 768),      # 128x192 tiles, no edge
+                                   (2900, 3000, 72),       # 128x192 tiles, two rounds, ragged
+                                   (2040, 4090, 136),      # 128x256 tiles, ragged
                                    (2040, 1800, 200),      # 128x128 tiles, one round, ragged
-                                   (2900, 3000, 72),       # 128x128 tiles, many rounds, ragged
+                                   (2040, 1000, 200),      # 64x128 tiles, ragged
                                    (2040, 760, 136),       # 64x96 tiles, one round, ragged
                                    (2048, 768, 3072),      # 64x96 tiles, long K
                                    (1000, 1000, 40),       # 64x64 tiles, K below one k tile
-                                   (512, 2304, 768)])      # 64x64 tiles
+                                   (257, 257, 264)])       # 64x64 tiles, few workgroups
 @pytest.mark.parametrize("epi", ["store", "add_residual"])
 def test_linear_bf16_tile_choices(ops, M, N, K, epi):
     """Every tile shape of the many-row product, with edges in all three dimensions."""
