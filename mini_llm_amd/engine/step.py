@@ -12,6 +12,8 @@ here they are built once per step and reach the device in one copy.
 """
 from __future__ import annotations
 
+import gc
+import weakref
 from dataclasses import dataclass, field
 from typing import Dict, List, Optional, Sequence
 
@@ -346,7 +348,8 @@ class DecodeGraph:
 
     def __init__(self, runner: ModelRunner, batch: int, greedy: bool):
         from ..kernels import ops
-        self.runner, self.batch, self.greedy = runner, batch, greedy
+        self.runner = weakref.proxy(runner)      # the runner owns this object: no reference cycle between them
+        self.batch, self.greedy = batch, greedy
         model, cache = runner.model, runner.cache
         dev = runner.device
         on_gpu = dev.type == "cuda"
@@ -422,8 +425,18 @@ class DecodeGraph:
                 torch.cuda.synchronize()
                 self.runner._tok_out.copy_(fed)
                 self.graph = torch.cuda.CUDAGraph()
-                with torch.cuda.graph(self.graph):
-                    self._forward()
+                # No graph may be destroyed while the stream captures (HIP refuses it and the process
+                # ends), and a dropped engine's graphs sit in reference cycles until the collector
+                # runs: so it runs now, and not during the capture.
+                gc.collect()
+                gc_was_enabled = gc.isenabled()
+                gc.disable()
+                try:
+                    with torch.cuda.graph(self.graph):
+                        self._forward()
+                finally:
+                    if gc_was_enabled:
+                        gc.enable()
             self.graph.replay()
         self._turn ^= 1
         host = self.h_out[self._turn]

@@ -185,3 +185,28 @@ def test_end_of_sequence_under_overlapped_graph_decode(tiny_model_dirs, dtype):
     assert len(expect[1]) == j + 1
     for pages, overlap in ((64, True), (64, False), (22, True)):
         assert run(eos, pages, overlap) == expect
+
+
+def test_a_dropped_engine_is_not_collected_while_a_graph_is_captured(tiny_model_dirs):
+    """An engine that nobody holds any more, but that sits in a reference cycle, keeps its HIP graphs
+    until Python's collector runs. Destroying a graph while another is captured ends the process,
+    so the collector runs before a capture and not during it: engines made one after the other,
+    with the collector set to run as often as it can, all generate the same tokens."""
+    import gc
+    from mini_llm_amd import Engine, EngineOptions, SamplingParams
+    prompts = _prompts("a", (9, 21), 6)
+    params = SamplingParams(max_new_tokens=6, ignore_eos=True)
+    old = gc.get_threshold()
+    gc.set_threshold(1, 1, 1)
+    try:
+        outs = []
+        for _ in range(4):
+            e = Engine.from_pretrained(tiny_model_dirs["a"], dtype="bfloat16",
+                                       options=EngineOptions(kv_block_size=8, total_kv_blocks=32, max_batch_num=4))
+            outs.append(e.generate(prompts, params))
+            cycle = [e]
+            cycle.append(cycle)                 # garbage only the collector can free
+            del e, cycle
+    finally:
+        gc.set_threshold(*old)
+    assert all(o == outs[0] for o in outs) and all(len(x) == 6 for x in outs[0])
