@@ -470,6 +470,20 @@ def test_paged_attention_prefill_tiles(ops, H, Hkv, dh, page, window):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("H,Hkv,dh,page", [(4, 4, 64, 4), (2, 1, 128, 16)])
+def test_paged_attention_long_contexts(ops, dtype, H, Hkv, dh, page):
+    """Contexts far beyond the tiny models': block tables longer than the prefill kernel stages in
+    LDS (2048 blocks), decode over 20,000 keys, a portion that ends a long prompt, with and without
+    a window."""
+    g = torch.Generator().manual_seed(dh + page)
+    for seqs, window in (([(9000, 1), (5, 1)], 0), ([(8300, 200)], 0), ([(0, 2300)], 777), ([(20000, 1)], 0),
+                         ([(8190, 3), (100, 40)], 777)):
+        out, ref = _attention_case(ops, dtype, H, Hkv, dh, page, seqs, window, g)
+        assert torch.isfinite(out).all()
+        assert (out - ref).abs().max() <= _tol(dtype, 2), (seqs, window)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
 def test_paged_attention_far_key_stands_out(ops, dtype):
     """One key hundreds of positions back carries almost all the weight of the last query."""
     g = torch.Generator().manual_seed(7)
