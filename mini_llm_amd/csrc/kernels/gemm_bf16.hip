@@ -23,7 +23,9 @@ typedef float f32x16 __attribute__((ext_vector_type(16)));
 // buffered (one barrier per k tile), global loads run DEPTH-1 tiles ahead in rotating register
 // sets, per-thread pointers only advance, and blocks that lie fully inside the matrices take an
 // edge-free path chosen at compile time. Within a tile the memory instructions are spread between
-// the MFMA groups of its k steps, so that the matrix units work while they queue. The weight
+// the MFMA groups of its k steps, so that the matrix units work while they queue. For a long K
+// two such groups of wavefronts share a workgroup's tile, each on half of a twice as wide k tile,
+// and add their sums in LDS. The weight
 // fragment is the MFMA's A operand, so a lane's accumulator registers hold 4 consecutive columns
 // of one output row; the epilogue turns that, through LDS, into stores of whole rows.
 // ---------------------------------------------------------------------------------------------
@@ -70,27 +72,32 @@ __device__ __forceinline__ void store4(void* C, size_t idx, const float (&v)[4],
     }
 }
 
-template <int WM, int WN, int TM, int TN, int BKP, int DEPTH, bool EDGE, int MODE>
-__global__ void __launch_bounds__(WM * WN * 64)
+template <int WM, int WN, int TM, int TN, int BKP, int DEPTH, bool EDGE, int MODE, int KG = 1>
+__global__ void __launch_bounds__(WM * WN * KG * 64)
 gemm_bf16_mfma(const bf16_t* __restrict__ A, int lda, const bf16_t* __restrict__ W, int ldw,
                const float* __restrict__ bias, void* __restrict__ C, int ldc, int M, int N, int K,
                int tiles_m, int tiles_n, int xm, int xn, KvScatter kv) {
-    constexpr int NT = WM * WN * 64;
+    // KG groups of WM x WN wavefronts share the tile: a k tile is KG * BKP wide and group g multiplies
+    // its g-th part, so a barrier interval covers KG times the depth; the groups' sums meet in LDS.
+    constexpr int NT = WM * WN * KG * 64;
     constexpr int BM = WM * TM * 32, BN = WN * TN * 32;
-    constexpr int STRIDE = BKP + 8;
-    constexpr int CPR = BKP / 8;                      // 16-byte chunks per row
+    constexpr int BKT = BKP * KG;
+    constexpr int STRIDE = BKT + 8;
+    constexpr int CPR = BKT / 8;                      // 16-byte chunks per row
     constexpr int KS = BKP / 16;                      // MFMA k steps per tile
     constexpr int A_CH = (BM * CPR + NT - 1) / NT, W_CH = (BN * CPR + NT - 1) / NT, N_LOADS = A_CH + W_CH;
     constexpr int EPI_STRIDE = 36;                    // floats per row of a 32x32 sub-tile in the epilogue
     static_assert(KS % 2 == 0 && DEPTH >= 3, "the k loop alternates two fragment sets and three register sets");
-    static_assert(2 * (BM + BN) * STRIDE * 2 >= WM * WN * 32 * EPI_STRIDE * 4, "the tiles' LDS holds the epilogue's regions");
+    constexpr int EPI_BASE = KG > 1 ? BM * BN : 0;    // floats: behind the groups' sums
+    static_assert(2 * (BM + BN) * STRIDE * 2 >= (EPI_BASE + WM * WN * 32 * EPI_STRIDE) * 4, "the tiles' LDS holds the epilogue's regions");
     // one array: two buffers of A rows, two of W rows; the epilogue reuses it, a region per wavefront
     __shared__ __attribute__((aligned(16))) bf16_t smem[2 * (BM + BN) * STRIDE];
     __shared__ __attribute__((aligned(16))) float bias_s[BN];
     bf16_t (*As)[BM * STRIDE] = reinterpret_cast<bf16_t (*)[BM * STRIDE]>(smem);
     bf16_t (*Ws)[BN * STRIDE] = reinterpret_cast<bf16_t (*)[BN * STRIDE]>(smem + 2 * BM * STRIDE);
 
-    const int tid = threadIdx.x, wave = tid / 64, lane = tid % 64;
+    const int tid = threadIdx.x, lane = tid % 64;
+    const int kg = tid / 64 / (WM * WN), wave = tid / 64 % (WM * WN);      // k group; wavefront within it
     const int wm = wave / WN, wn = wave % WN;
     // Workgroups are handed to the 8 XCDs round-robin and every XCD has an L2 of its own, so the
     // tiles of one XCD (workgroup id % 8) form one compact rectangle of the output: the rows of A
@@ -175,8 +182,8 @@ gemm_bf16_mfma(const bf16_t* __restrict__ A, int lda, const bf16_t* __restrict__
         }
     };
     // two sets of MFMA operands: the fragments of k step ks+1 are read while step ks multiplies
-    const int a_off = (wm * TM * 32 + lane % 32) * STRIDE + 8 * (lane / 32);
-    const int w_off = (wn * TN * 32 + lane % 32) * STRIDE + 8 * (lane / 32);
+    const int a_off = (wm * TM * 32 + lane % 32) * STRIDE + kg * BKP + 8 * (lane / 32);
+    const int w_off = (wn * TN * 32 + lane % 32) * STRIDE + kg * BKP + 8 * (lane / 32);
     bf16x8 fa[2][TM], fb[2][TN];
     auto read_frags = [&](int buf, int ks, int set) {
 #pragma unroll
@@ -194,11 +201,11 @@ gemm_bf16_mfma(const bf16_t* __restrict__ A, int lda, const bf16_t* __restrict__
                 acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[set][j], fa[set][i], acc[i][j], 0, 0, 0);
     };
 
-    const int nk = (K + BKP - 1) / BKP;
+    const int nk = (K + BKT - 1) / BKT;
     // tiles 0 .. DEPTH-2 are requested (past the last tile: the last one again, never used);
     // tile 0 is staged
 #pragma unroll
-    for (int d = 0; d < DEPTH - 1; ++d) fetch(regs[d], min(d, nk - 1) * BKP, -1);
+    for (int d = 0; d < DEPTH - 1; ++d) fetch(regs[d], min(d, nk - 1) * BKT, -1);
     stage(regs[0], 0, 0, -1);
     lds_barrier();
     read_frags(0, 0, 0);
@@ -216,11 +223,11 @@ gemm_bf16_mfma(const bf16_t* __restrict__ A, int lda, const bf16_t* __restrict__
 #pragma unroll
         for (int d = 0; d < DEPTH; ++d) {
             const int t = g * DEPTH + d;
-            const int k_fetch = min(t + DEPTH - 1, nk - 1) * BKP;
+            const int k_fetch = min(t + DEPTH - 1, nk - 1) * BKT;
 #pragma unroll
             for (int ks = 0; ks < KS; ++ks) {
                 fetch(regs[(d + DEPTH - 1) % DEPTH], k_fetch, ks);
-                stage(regs[(d + 1) % DEPTH], (t + 1) & 1, (t + 1) * BKP, ks);
+                stage(regs[(d + 1) % DEPTH], (t + 1) & 1, (t + 1) * BKT, ks);
                 if (ks + 1 < KS) read_frags(t & 1, ks + 1, (ks + 1) & 1);
                 mma(ks & 1);
                 __builtin_amdgcn_sched_barrier(0);
@@ -233,7 +240,7 @@ gemm_bf16_mfma(const bf16_t* __restrict__ A, int lda, const bf16_t* __restrict__
     for (int d = 0; d < DEPTH - 1; ++d) {
         const int t = n_groups * DEPTH + d;
         if (d < n_tail) {
-            if (d + 1 < n_tail) stage(regs[(d + 1) % DEPTH], (t + 1) & 1, (t + 1) * BKP, -1);
+            if (d + 1 < n_tail) stage(regs[(d + 1) % DEPTH], (t + 1) & 1, (t + 1) * BKT, -1);
 #pragma unroll
             for (int ks = 0; ks < KS; ++ks) {
                 if (ks + 1 < KS) read_frags(t & 1, ks + 1, (ks + 1) & 1);
@@ -249,8 +256,34 @@ gemm_bf16_mfma(const bf16_t* __restrict__ A, int lda, const bf16_t* __restrict__
     // 16 bytes in each of 32 rows. So each sub-tile goes through the wavefront's own region of LDS
     // (the tiles are done with theirs): written as the MFMA left it, read back with 8 lanes per row,
     // and a store instruction then covers 8 whole rows of the sub-tile.
+    if constexpr (KG > 1) {
+        // the other groups leave their sums in LDS, register by register, and go; group 0 adds them
+        float4* sums = reinterpret_cast<float4*>(smem);
+        if (kg > 0) {
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+#pragma unroll
+                for (int j = 0; j < TN; ++j)
+#pragma unroll
+                    for (int g = 0; g < 4; ++g)
+                        sums[((wave * TM * TN + i * TN + j) * 4 + g) * 64 + lane] =
+                            make_float4(acc[i][j][4 * g], acc[i][j][4 * g + 1], acc[i][j][4 * g + 2], acc[i][j][4 * g + 3]);
+        }
+        lds_barrier();
+        if (kg > 0) return;
+        static_assert(KG == 2, "one other group's sums fit in front of the epilogue's regions");
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+#pragma unroll
+                for (int g = 0; g < 4; ++g) {
+                    const float4 t = sums[((wave * TM * TN + i * TN + j) * 4 + g) * 64 + lane];
+                    acc[i][j][4 * g] += t.x; acc[i][j][4 * g + 1] += t.y; acc[i][j][4 * g + 2] += t.z; acc[i][j][4 * g + 3] += t.w;
+                }
+    }
     const bool vec = (ldc % 4 == 0) && ((reinterpret_cast<uintptr_t>(C) & 15) == 0);
-    float* epi = reinterpret_cast<float*>(smem) + wave * (32 * EPI_STRIDE);
+    float* epi = reinterpret_cast<float*>(smem) + EPI_BASE + wave * (32 * EPI_STRIDE);
 #pragma unroll
     for (int i = 0; i < TM; ++i) {
 #pragma unroll
@@ -297,7 +330,7 @@ gemm_bf16_mfma(const bf16_t* __restrict__ A, int lda, const bf16_t* __restrict__
     }
 }
 
-template <int WM, int WN, int TM, int TN, int BKP, int DEPTH>
+template <int WM, int WN, int TM, int TN, int BKP, int DEPTH, int KG = 1>
 static void launch_tiled(const bf16_t* a, int lda, const bf16_t* w, int ldw, const float* bias, void* C, int ldc,
                          int M, int N, int K, int mode, hipStream_t stream, KvScatter kv = KvScatter{}) {
     constexpr int BM = WM * TM * 32, BN = WN * TN * 32;
@@ -311,9 +344,9 @@ static void launch_tiled(const bf16_t* a, int lda, const bf16_t* w, int ldw, con
         if (rows < best) { best = rows; xm = cm; xn = cn; }
     }
     const int per_xcd = ((tiles_m + xm - 1) / xm) * ((tiles_n + xn - 1) / xn);
-    const dim3 grid(per_xcd * N_XCD), block(WM * WN * 64);
-    const bool edge = !(M % BM == 0 && N % BN == 0 && K % BKP == 0);
-#define TILED(E, MD) gemm_bf16_mfma<WM, WN, TM, TN, BKP, DEPTH, E, MD><<<grid, block, 0, stream>>>(a, lda, w, ldw, bias, C, ldc, M, N, K, tiles_m, tiles_n, xm, xn, kv)
+    const dim3 grid(per_xcd * N_XCD), block(WM * WN * KG * 64);
+    const bool edge = !(M % BM == 0 && N % BN == 0 && K % (BKP * KG) == 0);
+#define TILED(E, MD) gemm_bf16_mfma<WM, WN, TM, TN, BKP, DEPTH, E, MD, KG><<<grid, block, 0, stream>>>(a, lda, w, ldw, bias, C, ldc, M, N, K, tiles_m, tiles_n, xm, xn, kv)
 #define TILED_MODE(MD) case MD: if (edge) TILED(true, MD); else TILED(false, MD); break;
     switch (mode) {
         TILED_MODE(EPI_STORE) TILED_MODE(EPI_GELU_TANH) TILED_MODE(EPI_GELU_ERF) TILED_MODE(EPI_ADD_RESIDUAL)
@@ -995,14 +1028,20 @@ static int gemm_bf16_dispatch(const void* A, int lda, const void* W, int ldw, co
             const double cost = static_cast<double>((blocks + 255) / 256) * shapes[c].bm * shapes[c].bn / shapes[c].efficiency;
             if (cost < best_cost) { best_cost = cost; best = c; }
         }
+        // With a long K the smaller tiles' time goes to the barrier intervals of the k loop, and two
+        // groups of wavefronts per workgroup, each on half of a twice as wide k tile, halve their
+        // number (measured at K of 3072 to 6400: 9 to 17 % less time; at K of 768 to 1600: none).
+        const bool long_k = K >= 2048;
+#define TILE(...) launch_tiled<__VA_ARGS__>(a, lda, w, ldw, bias, C, ldc, M, N, K, mode, stream, kv)
         switch (best) {
-            case 0: launch_tiled<2, 4, 2, 2, 64, 4>(a, lda, w, ldw, bias, C, ldc, M, N, K, mode, stream, kv); break;
-            case 1: launch_tiled<4, 2, 1, 3, 64, 3>(a, lda, w, ldw, bias, C, ldc, M, N, K, mode, stream, kv); break;
-            case 2: launch_tiled<2, 4, 2, 1, 64, 3>(a, lda, w, ldw, bias, C, ldc, M, N, K, mode, stream, kv); break;
-            case 3: launch_tiled<2, 4, 1, 1, 64, 4>(a, lda, w, ldw, bias, C, ldc, M, N, K, mode, stream, kv); break;
-            case 4: launch_tiled<2, 3, 1, 1, 64, 5>(a, lda, w, ldw, bias, C, ldc, M, N, K, mode, stream, kv); break;
-            default: launch_tiled<2, 2, 1, 1, 64, 4>(a, lda, w, ldw, bias, C, ldc, M, N, K, mode, stream, kv); break;
+            case 0: TILE(2, 4, 2, 2, 64, 4); break;
+            case 1: TILE(4, 2, 1, 3, 64, 3); break;
+            case 2: if (long_k) TILE(2, 4, 2, 1, 64, 3, 2); else TILE(2, 4, 2, 1, 64, 3); break;
+            case 3: TILE(2, 4, 1, 1, 64, 4); break;
+            case 4: if (long_k) TILE(2, 3, 1, 1, 64, 5, 2); else TILE(2, 3, 1, 1, 64, 5); break;
+            default: if (long_k) TILE(2, 2, 1, 1, 64, 4, 2); else TILE(2, 2, 1, 1, 64, 4); break;
         }
+#undef TILE
     }
     MLLM_LAUNCH_CHECK();
     return 0;

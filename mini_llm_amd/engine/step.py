@@ -426,9 +426,9 @@ class DecodeGraph:
                 self.runner._tok_out.copy_(fed)
                 self.graph = torch.cuda.CUDAGraph()
                 # No graph may be destroyed while the stream captures (HIP refuses it and the process
-                # ends), and a dropped engine's graphs sit in reference cycles until the collector
-                # runs: so it runs now, and not during the capture.
-                gc.collect()
+                # ends), and a dropped engine's graphs may sit in a reference cycle until the collector
+                # runs: so it does not run during the capture. (Running it before every capture instead
+                # costs more than the capture.)
                 gc_was_enabled = gc.isenabled()
                 gc.disable()
                 try:

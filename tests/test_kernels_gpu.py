@@ -121,7 +121,9 @@ def test_linear(ops, dtype, M, N, K, epi):
                                    (2040, 1800, 200),      # 128x128 tiles, one round, ragged
                                    (2040, 1000, 200),      # 64x128 tiles, ragged
                                    (2040, 760, 136),       # 64x96 tiles, one round, ragged
-                                   (2048, 768, 3072),      # 64x96 tiles, long K
+                                   (2048, 768, 3072),      # 64x96 tiles, long K: two wavefront groups per workgroup
+                                   (2040, 1800, 2056),     # 128x128 tiles, two groups, K not a multiple of their k tile
+                                   (300, 500, 4104),       # 64x64 tiles, two groups, ragged
                                    (1000, 1000, 40),       # 64x64 tiles, K below one k tile
                                    (257, 257, 264)])       # 64x64 tiles, few workgroups
 @pytest.mark.parametrize("epi", ["store", "add_residual"])
