@@ -122,13 +122,12 @@ def serving_run(model_dir, dtype, cfg, n_req, prompt_lo, prompt_hi, new_tokens, 
                                                           max_batch_num=max_batch,
                                                           max_tokens_per_step=max(2048, max_batch + chunk),
                                                           prefill_chunk=chunk))
+    engine.warmup()      # untimed, as a server does before it takes requests: the decode graphs are captured
     g = torch.Generator().manual_seed(seed)
     lens = torch.randint(prompt_lo, prompt_hi + 1, (n_req,), generator=g).tolist()
     params = SamplingParams(max_new_tokens=new_tokens, ignore_eos=True)
     for n in lens:
         engine.add_request(torch.randint(0, cfg["vocab_size"], (n,), generator=g).tolist(), params)
-    # untimed: one short request through prefill and decode loads the kernels and captures nothing that
-    # the timed run would not capture itself
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     n_out = n_steps = 0
@@ -167,7 +166,7 @@ def serving_main(args, cfg, model_dir):
            "steps": r["steps"], "warmup": 0, "ms_per_step": round(1e3 * r["seconds"] / r["steps"], 4),
            "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
            "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
-           "data": "synthetic (random weights seed 2, uniform random token ids and prompt lengths, seed 7)",
+           "data": "synthetic (random weights seed 2, uniform random token ids and prompt lengths, seed 7); decode graphs captured before the clock starts",
            "config": {"model": args.size + "-sizes", "n_layer": cfg["n_layer"], "n_layer_full": SIZES[args.size][0],
                       "requests": n_req, "prompt_min": lo, "prompt_max": hi, "new_tokens": new,
                       "max_batch_num": max_batch, "prefill_chunk": chunk, "kv_blocks": pages, "kv_block_size": 16,

@@ -236,6 +236,24 @@ class Engine:
             out.append(r.output)
         return out
 
+    def warmup(self, sampling: bool = False) -> List[int]:
+        """Captures the decode graphs before the first real request needs them: for every batch size
+        that decode steps are captured at (1 to 8, then multiples of 8 up to ``max_batch_num``) that
+        many one-token requests run one step. With ``sampling`` the graphs that sample at a
+        temperature are captured too. Returns the batch sizes. Call it on an idle engine."""
+        if self.has_unfinished():
+            raise RuntimeError("warmup wants an idle engine")
+        if not self.runner.fast_decode:
+            return []
+        top = self.options.max_batch_num
+        sizes = sorted({b for b in range(1, min(top, 8) + 1)} | {b for b in range(16, top + 1, 8)} | {top}, reverse=True)
+        pages = self.runner.manager.total_pages(0) if self.runner.cache.n_groups else top
+        sizes = [b for b in sizes if b <= pages]
+        for temperature in ([0.0, 1.0] if sampling else [0.0]):
+            for b in sizes:
+                self.generate([[0]] * b, SamplingParams(temperature=temperature, max_new_tokens=1, ignore_eos=True))
+        return sizes
+
     def stats(self) -> Dict[str, int]:
         s = self.scheduler.counters()
         s["free_pages"] = self.runner.manager.free_pages(0) if self.runner.cache.n_groups else 0

@@ -210,3 +210,20 @@ def test_a_dropped_engine_is_not_collected_while_a_graph_is_captured(tiny_model_
     finally:
         gc.set_threshold(*old)
     assert all(o == outs[0] for o in outs) and all(len(x) == 6 for x in outs[0])
+
+
+def test_warmup_captures_the_decode_graphs_and_changes_nothing(tiny_model_dirs):
+    from mini_llm_amd import Engine, EngineOptions, SamplingParams
+    prompts = _prompts("b", (3, 30, 11), 8)
+    params = [SamplingParams(temperature=t, seed=4, max_new_tokens=9, ignore_eos=True) for t in (0.0, 0.9, 0.0)]
+    opts = dict(kv_block_size=8, total_kv_blocks=40, max_batch_num=20)
+    cold = Engine.from_pretrained(tiny_model_dirs["b"], dtype="bfloat16", options=EngineOptions(**opts))
+    expect = cold.generate(prompts, params)
+    warm = Engine.from_pretrained(tiny_model_dirs["b"], dtype="bfloat16", options=EngineOptions(**opts))
+    sizes = warm.warmup(sampling=True)
+    assert sizes == [20, 16, 8, 7, 6, 5, 4, 3, 2, 1]
+    captured = dict(warm.runner._graphs)
+    assert {k[0] for k in captured} == {24, 16, 8, 7, 6, 5, 4, 3, 2, 1} and len(captured) == 20
+    assert warm.stats()["free_pages"] == 40 and not warm.has_unfinished() and not warm.requests
+    assert warm.generate(prompts, params) == expect
+    assert all(warm.runner._graphs[k] is g for k, g in captured.items())        # nothing captured again
