@@ -1,7 +1,8 @@
 // True fp32 matrix product for the 32-bit path: C[M,N] = A[M,K] * W[N,K]^T (+ bias, epilogue).
-// Plain FMA in fp32, every output accumulated over k in ascending order, so a row's
-// result does not depend on which other rows share the launch. No reduced-precision
-// matrix mode is involved. Any M, N, K.
+// Plain FMA in fp32, every output accumulated over k in a fixed order, so a row's
+// result does not depend on which other rows share the launch (beyond the choice between the
+// two kernels below, which add in different orders). No reduced-precision matrix mode is
+// involved. Any M, N, K.
 //
 // Same contract as the reference's bounds-safe kernel
 // (/root/reference/src/kernels/gemm.cu:238-392: alpha*acc + beta*old + bias, optional GELU),
@@ -81,11 +82,73 @@ gemm_f32_kernel(const float* __restrict__ A, int lda, const float* __restrict__ 
     }
 }
 
+// Few rows (decode): the product is bound by reading W once, and the tiled kernel above would
+// start N/64 workgroups for it. Here a wavefront owns one output column: its lanes walk the
+// column's weights in 16-byte steps (a wavefront's load is 1 KB of one row), the activations of
+// up to ROWS rows wait in LDS in chunks of F32R_KC floats, and a lane's partial sums (k ascending)
+// are added over the wavefront in a fixed order. More rows than ROWS take further passes over W.
+// Needs K and the row strides in multiples of 4 floats and 16-byte aligned operands.
+#define F32R_KC 512
+
+template <int ROWS>
+__global__ void __launch_bounds__(256)
+gemm_f32_rows_kernel(const float* __restrict__ A, int lda, const float* __restrict__ W, int ldw,
+                     const float* __restrict__ bias, void* __restrict__ C, int ldc, int M, int N, int K, int mode) {
+    __shared__ __attribute__((aligned(16))) float a_s[ROWS][F32R_KC];
+    const int tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid / 64), lane = tid % 64;
+    const int n = blockIdx.x * 4 + wave;
+    const float* wrow = W + static_cast<size_t>(min(n, N - 1)) * ldw;       // a surplus wavefront repeats the last column
+    for (int m0 = 0; m0 < M; m0 += ROWS) {
+        float acc[ROWS];
+#pragma unroll
+        for (int r = 0; r < ROWS; ++r) acc[r] = 0.f;
+        for (int kc0 = 0; kc0 < K; kc0 += F32R_KC) {
+            const int quads = min(F32R_KC, K - kc0) / 4;
+            __syncthreads();          // the chunk before has been read
+            for (int idx = tid; idx < ROWS * quads; idx += 256) {
+                const int r = idx / quads, q = idx % quads;
+                float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+                if (m0 + r < M) v = *reinterpret_cast<const float4*>(A + static_cast<size_t>(m0 + r) * lda + kc0 + 4 * q);
+                *reinterpret_cast<float4*>(&a_s[r][4 * q]) = v;
+            }
+            __syncthreads();
+            for (int q = lane; q < quads; q += 64) {
+                const float4 w4 = *reinterpret_cast<const float4*>(wrow + kc0 + 4 * q);
+#pragma unroll
+                for (int r = 0; r < ROWS; ++r) {
+                    const float4 a4 = *reinterpret_cast<const float4*>(&a_s[r][4 * q]);
+                    acc[r] = fmaf(a4.x, w4.x, acc[r]);
+                    acc[r] = fmaf(a4.y, w4.y, acc[r]);
+                    acc[r] = fmaf(a4.z, w4.z, acc[r]);
+                    acc[r] = fmaf(a4.w, w4.w, acc[r]);
+                }
+            }
+        }
+        float mine = 0.f;
+#pragma unroll
+        for (int r = 0; r < ROWS; ++r) {
+            const float t = wave_sum(acc[r]);
+            if (lane == r) mine = t;
+        }
+        if (n < N && lane < ROWS && m0 + lane < M)
+            epilogue<float>(mode, mine, bias ? bias[n] : 0.f, C, static_cast<size_t>(m0 + lane) * ldc + n);
+    }
+}
+
 extern "C" {
 
 int mllm_gemm_f32(const float* A, int lda, const float* W, int ldw, const float* bias, void* C, int ldc,
                   int M, int N, int K, int mode, hipStream_t stream) {
     if (M <= 0 || N <= 0) return 0;
+    const bool quads = K % 4 == 0 && lda % 4 == 0 && ldw % 4 == 0 &&
+                       ((reinterpret_cast<uintptr_t>(A) | reinterpret_cast<uintptr_t>(W)) & 15) == 0;
+    if (M <= 64 && quads && K > 0) {
+        const dim3 rows_grid((N + 3) / 4);
+        if (M <= 8) gemm_f32_rows_kernel<8><<<rows_grid, 256, 0, stream>>>(A, lda, W, ldw, bias, C, ldc, M, N, K, mode);
+        else gemm_f32_rows_kernel<16><<<rows_grid, 256, 0, stream>>>(A, lda, W, ldw, bias, C, ldc, M, N, K, mode);
+        MLLM_LAUNCH_CHECK();
+        return 0;
+    }
     dim3 grid((N + F32_BN - 1) / F32_BN, (M + F32_BM - 1) / F32_BM);
     gemm_f32_kernel<<<grid, 256, 0, stream>>>(A, lda, W, ldw, bias, C, ldc, M, N, K, mode);
     MLLM_LAUNCH_CHECK();

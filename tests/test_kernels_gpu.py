@@ -300,6 +300,26 @@ def test_linear_fp32_is_true_fp32(ops):
     assert out[0, 0].item() == 2.0 ** -20
 
 
+@pytest.mark.parametrize("M,N,K,pad", [(5, 70, 42, 0),        # K no multiple of 4: the tiled kernel
+                                         (7, 33, 1028, 3),      # row strides no multiple of 4 floats
+                                         (8, 50257, 64, 0),     # the few-row kernel, one pass, wide
+                                         (64, 130, 1600, 0),    # four passes of 16 rows, k chunks with a rest
+                                         (17, 5, 8, 4)])        # fewer columns than a workgroup has wavefronts
+def test_linear_fp32_few_rows(ops, M, N, K, pad):
+    """The 32-bit product of few rows streams the weights, one column per wavefront, where the operands
+    are 16-byte aligned, and falls back to the tiled kernel where they are not."""
+    g = torch.Generator().manual_seed(M + N + K)
+    a = _rand((M, K + pad), torch.float32, g).to(DEV)[:, :K]
+    w = _rand((N, K + pad), torch.float32, g, std=1.0 / math.sqrt(K)).to(DEV)[:, :K]
+    bias = 0.5 * _rand((N,), torch.float32, g)
+    for epi in ("store", "add_residual", "gelu_tanh"):
+        out0 = _rand((M, N), torch.float32, g)
+        out = out0.clone().to(DEV)
+        ops.linear(a, w, bias.to(DEV), out, epi)
+        ref = plain_ops.linear(a.cpu(), w.cpu(), bias, out0.double().clone(), epi)
+        assert (out.cpu().double() - ref).abs().max().item() <= 3e-5
+
+
 def test_linear_bf16_refuses_odd_k(ops):
     a = torch.zeros(4, 36, dtype=torch.bfloat16, device=DEV)
     w = torch.zeros(8, 36, dtype=torch.bfloat16, device=DEV)
