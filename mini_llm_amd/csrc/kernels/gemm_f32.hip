@@ -88,7 +88,7 @@ gemm_f32_kernel(const float* __restrict__ A, int lda, const float* __restrict__ 
 // up to ROWS rows wait in LDS in chunks of F32R_KC floats, and a lane's partial sums (k ascending)
 // are added over the wavefront in a fixed order. More rows than ROWS take further passes over W.
 // Needs K and the row strides in multiples of 4 floats and 16-byte aligned operands.
-#define F32R_KC 512
+#define F32R_KC 512      // 128 16-byte steps: two per lane
 
 template <int ROWS>
 __global__ void __launch_bounds__(256)
@@ -104,6 +104,12 @@ gemm_f32_rows_kernel(const float* __restrict__ A, int lda, const float* __restri
         for (int r = 0; r < ROWS; ++r) acc[r] = 0.f;
         for (int kc0 = 0; kc0 < K; kc0 += F32R_KC) {
             const int quads = min(F32R_KC, K - kc0) / 4;
+            // a chunk is at most two 16-byte steps per lane: both loads are issued here, ahead of the
+            // staging of the activations (the second from a clamped address; its product is left out
+            // where it is past the chunk)
+            const int q0 = lane, q1 = lane + 64;
+            const float4 w0 = *reinterpret_cast<const float4*>(wrow + kc0 + 4 * min(q0, quads - 1));
+            const float4 w1 = *reinterpret_cast<const float4*>(wrow + kc0 + 4 * min(q1, quads - 1));
             __syncthreads();          // the chunk before has been read
             for (int idx = tid; idx < ROWS * quads; idx += 256) {
                 const int r = idx / quads, q = idx % quads;
@@ -112,15 +118,24 @@ gemm_f32_rows_kernel(const float* __restrict__ A, int lda, const float* __restri
                 *reinterpret_cast<float4*>(&a_s[r][4 * q]) = v;
             }
             __syncthreads();
-            for (int q = lane; q < quads; q += 64) {
-                const float4 w4 = *reinterpret_cast<const float4*>(wrow + kc0 + 4 * q);
+            if (q0 < quads) {
 #pragma unroll
                 for (int r = 0; r < ROWS; ++r) {
-                    const float4 a4 = *reinterpret_cast<const float4*>(&a_s[r][4 * q]);
-                    acc[r] = fmaf(a4.x, w4.x, acc[r]);
-                    acc[r] = fmaf(a4.y, w4.y, acc[r]);
-                    acc[r] = fmaf(a4.z, w4.z, acc[r]);
-                    acc[r] = fmaf(a4.w, w4.w, acc[r]);
+                    const float4 a4 = *reinterpret_cast<const float4*>(&a_s[r][4 * q0]);
+                    acc[r] = fmaf(a4.x, w0.x, acc[r]);
+                    acc[r] = fmaf(a4.y, w0.y, acc[r]);
+                    acc[r] = fmaf(a4.z, w0.z, acc[r]);
+                    acc[r] = fmaf(a4.w, w0.w, acc[r]);
+                }
+            }
+            if (q1 < quads) {
+#pragma unroll
+                for (int r = 0; r < ROWS; ++r) {
+                    const float4 a4 = *reinterpret_cast<const float4*>(&a_s[r][4 * q1]);
+                    acc[r] = fmaf(a4.x, w1.x, acc[r]);
+                    acc[r] = fmaf(a4.y, w1.y, acc[r]);
+                    acc[r] = fmaf(a4.z, w1.z, acc[r]);
+                    acc[r] = fmaf(a4.w, w1.w, acc[r]);
                 }
             }
         }
