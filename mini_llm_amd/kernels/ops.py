@@ -221,7 +221,8 @@ def _gemm_workspace(device) -> torch.Tensor:
     return ws
 
 
-LN_FUSE_MAX_ROWS = 16      # above this many rows the norm is faster as a kernel of its own (measured)
+LN_FUSE_MAX_ROWS = 32      # above this many rows the norm is faster as a kernel of its own (measured: 1-2 % of a
+                           # decode step gained at 24 and 32 rows, 3 % lost at 64)
 
 
 def ln_linear(x: torch.Tensor, gamma: torch.Tensor, beta: Optional[torch.Tensor], eps: float,
@@ -230,7 +231,7 @@ def ln_linear(x: torch.Tensor, gamma: torch.Tensor, beta: Optional[torch.Tensor]
     """out = epilogue(LayerNorm(x) @ w.T + bias) with x the fp32 stream [*,K] and w [N,K]; with
     ``rows`` (int32 [M]) row m of the input is x[rows[m]].
 
-    For bfloat16 weights, at most 16 rows and fewer than 16384 columns the norm is fused into the
+    For bfloat16 weights, at most 32 rows and fewer than 16384 columns the norm is fused into the
     product (one kernel);
     otherwise the norm and the product run one after the other. Same numerics either way:
     statistics in fp32, the normalised rows rounded to w's dtype before the product.
