@@ -1000,13 +1000,23 @@ static int gemm_bf16_dispatch(const void* A, int lda, const void* W, int ldw, co
     const bf16_t* a = static_cast<const bf16_t*>(A);
     const bf16_t* w = static_cast<const bf16_t*>(W);
     const bool scatter = kv.slots != nullptr;       // only the many-row kernel scatters
-    // The weight-streaming kernel takes up to 64 rows always, and up to 256 rows while its 16-row
-    // by 16-column workgroups stay within about four rounds over the compute units (measured
-    // against the tiled kernel on GPT-2 small to XL shapes at 64 to 256 rows: narrow outputs such
-    // as the attention and feed-forward output projections stay with it up to 256 rows, the wide
-    // ones leave it between 64 and 128 rows)
-    const long skinny_wgs = static_cast<long>((N + 15) / 16) * ((M + 15) / 16);
-    const bool few_rows = M <= 64 ? ((N + 15) / 16 >= 1024 || skinny_wgs <= 1024) : (M <= 256 && skinny_wgs <= 1024);
+    // Which kernel for up to 256 rows. Up to 16 rows (one row block) and for the widest products (the
+    // logits head) the weight-streaming kernel, always. In between both are priced, in microseconds,
+    // by formulas fitted to measurements on the products of GPT-2 small to XL at 24 to 256 rows: the
+    // weight-streaming kernel runs its 16-row by 16-column workgroups in rounds of 256 whose time
+    // grows with K (steeply beyond 3072, where a wavefront's share of K no longer fits its chunks);
+    // the tiled kernel's time is its k loop, a little more where edges make it take the checked path.
+    const int col_tiles = (N + 15) / 16, row_blocks16 = (M + 15) / 16;
+    auto streaming_is_faster = [&]() {
+        const double rounds = static_cast<double>((static_cast<long>(col_tiles) * row_blocks16 + 255) / 256);
+        const double streaming = 2.0 + rounds * (K <= 3072 ? 1.2 + 0.0008 * K : 0.0025 * K);
+        const double blocks = static_cast<double>((M + 63) / 64) * ((N + 63) / 64);
+        const bool ragged = M % 64 != 0 || N % 64 != 0 || K % 64 != 0;
+        const double tiled = 5.0 + 0.18 * (K / 64.0) * std::max(1.0, blocks / 256.0) + (ragged ? 2.0 : 0.0) +
+                             (M <= 32 ? 4.0 : 0.0);       // (up to 32 rows the tiled kernel has one shape, 32x128)
+        return streaming <= tiled;
+    };
+    const bool few_rows = M <= 16 || (M <= 64 && col_tiles >= 1024) || (M <= 256 && streaming_is_faster());
     if (!scatter && few_rows && launch_skinny<false>(A, lda, w, ldw, bias, C, ldc, M, N, K, mode, nullptr, nullptr,
                                                     0.f, nullptr, stream, workspace, workspace_bytes) == 0) {
         // few rows: weight-streaming kernel
