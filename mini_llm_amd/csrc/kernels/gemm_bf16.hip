@@ -21,8 +21,8 @@ typedef float f32x16 __attribute__((ext_vector_type(16)));
 // ---------------------------------------------------------------------------------------------
 // Many rows (prefill): WM x WN wavefronts, each TM x TN MFMA tiles of 32x32. LDS is double
 // buffered (one barrier per k tile), global loads run DEPTH-1 tiles ahead in rotating register
-// sets, per-thread pointers only advance, and blocks that lie fully inside the matrices take an
-// edge-free path chosen at compile time. Within a tile the memory instructions are spread between
+// sets, per-thread pointers only advance, and a K that is a multiple of the k tile takes a k loop
+// without checks, chosen at compile time (rows and columns beyond the matrices cost nothing there). Within a tile the memory instructions are spread between
 // the MFMA groups of its k steps, so that the matrix units work while they queue. For a long K
 // two such groups of wavefronts share a workgroup's tile, each on half of a twice as wide k tile,
 // and add their sums in LDS. The weight
@@ -126,14 +126,14 @@ gemm_bf16_mfma(const bf16_t* __restrict__ A, int lda, const bf16_t* __restrict__
 #pragma unroll
     for (int i = 0; i < A_CH; ++i) {
         const int c = tid + i * NT, row = c / CPR, kc = c % CPR;
-        va[i] = (BM * CPR % NT == 0 || c < BM * CPR) && (!EDGE || m0 + row < M);
+        va[i] = (BM * CPR % NT == 0 || c < BM * CPR) && m0 + row < M;
         pa[i] = A + static_cast<size_t>(va[i] ? m0 + row : 0) * lda + kc * 8;
         la[i] = row * STRIDE + kc * 8;
     }
 #pragma unroll
     for (int i = 0; i < W_CH; ++i) {
         const int c = tid + i * NT, row = c / CPR, kc = c % CPR;
-        vw[i] = (BN * CPR % NT == 0 || c < BN * CPR) && (!EDGE || n0 + row < N);
+        vw[i] = (BN * CPR % NT == 0 || c < BN * CPR) && n0 + row < N;
         pw[i] = W + static_cast<size_t>(vw[i] ? n0 + row : 0) * ldw + kc * 8;
         lw[i] = row * STRIDE + kc * 8;
     }
@@ -141,12 +141,16 @@ gemm_bf16_mfma(const bf16_t* __restrict__ A, int lda, const bf16_t* __restrict__
         uint4 ra[A_CH], rw[W_CH];
     };
     TileRegs regs[DEPTH];
+    // (Rows of A or W beyond the matrix: the pointer stays on a row that exists, and what is computed
+    // from it lands in output rows or columns that are never stored. Only a K that is no multiple of
+    // the k tile needs care in the loop, EDGE: addresses clamped into the row, and zeros staged for
+    // what lies beyond K.)
     // A tile's loads and its LDS writes are cut into KS portions (portion `part`, or all of them
     // with part < 0), so that they can be issued between the MFMA groups of the tile in work.
     // Every thread issues every load, with the address clamped into the matrix: the number of loads
     // in flight is then the same on every path through the loop, and only so does the compiler wait
     // for exactly the registers that are staged next while later loads stay in flight. What lies
-    // outside the matrices is zeroed when the tile is staged.
+    // beyond K is zeroed when the tile is staged.
     auto fetch = [&](TileRegs& t, int k0, int part) {
 #pragma unroll
         for (int i = 0; i < A_CH; ++i) {
@@ -168,7 +172,7 @@ gemm_bf16_mfma(const bf16_t* __restrict__ A, int lda, const bf16_t* __restrict__
         for (int i = 0; i < A_CH; ++i) {
             if (part >= 0 && i * KS / N_LOADS != part) continue;
             const int kc8 = (tid + i * NT) % CPR * 8;
-            const bool ok = !EDGE || (va[i] && k0 + kc8 < K);
+            const bool ok = !EDGE || k0 + kc8 < K;
             if (BM * CPR % NT == 0 || tid + i * NT < BM * CPR)
                 *reinterpret_cast<uint4*>(&As[buf][la[i]]) = ok ? t.ra[i] : make_uint4(0, 0, 0, 0);
         }
@@ -176,7 +180,7 @@ gemm_bf16_mfma(const bf16_t* __restrict__ A, int lda, const bf16_t* __restrict__
         for (int i = 0; i < W_CH; ++i) {
             if (part >= 0 && (A_CH + i) * KS / N_LOADS != part) continue;
             const int kc8 = (tid + i * NT) % CPR * 8;
-            const bool ok = !EDGE || (vw[i] && k0 + kc8 < K);
+            const bool ok = !EDGE || k0 + kc8 < K;
             if (BN * CPR % NT == 0 || tid + i * NT < BN * CPR)
                 *reinterpret_cast<uint4*>(&Ws[buf][lw[i]]) = ok ? t.rw[i] : make_uint4(0, 0, 0, 0);
         }
@@ -299,8 +303,8 @@ gemm_bf16_mfma(const bf16_t* __restrict__ A, int lda, const bf16_t* __restrict__
             for (int it = 0; it < 4; ++it) {
                 const int r = it * 8 + lane / 8, c4 = (lane % 8) * 4;
                 const int m = mb + r, n = nb + c4;
-                if (EDGE && (m >= M || n >= N)) continue;
-                const int n_left = EDGE ? min(4, N - n) : 4;
+                if (m >= M || n >= N) continue;
+                const int n_left = min(4, N - n);
                 const float4 t = *reinterpret_cast<const float4*>(&epi[r * EPI_STRIDE + c4]);
                 float v[4] = {t.x, t.y, t.z, t.w};
                 if (bias != nullptr) {
@@ -345,7 +349,7 @@ static void launch_tiled(const bf16_t* a, int lda, const bf16_t* w, int ldw, con
     }
     const int per_xcd = ((tiles_m + xm - 1) / xm) * ((tiles_n + xn - 1) / xn);
     const dim3 grid(per_xcd * N_XCD), block(WM * WN * KG * 64);
-    const bool edge = !(M % BM == 0 && N % BN == 0 && K % (BKP * KG) == 0);
+    const bool edge = K % (BKP * KG) != 0;      // rows and columns beyond the matrices need no other kernel, see EDGE
 #define TILED(E, MD) gemm_bf16_mfma<WM, WN, TM, TN, BKP, DEPTH, E, MD, KG><<<grid, block, 0, stream>>>(a, lda, w, ldw, bias, C, ldc, M, N, K, tiles_m, tiles_n, xm, xn, kv)
 #define TILED_MODE(MD) case MD: if (edge) TILED(true, MD); else TILED(false, MD); break;
     switch (mode) {
@@ -1005,13 +1009,13 @@ static int gemm_bf16_dispatch(const void* A, int lda, const void* W, int ldw, co
     // by formulas fitted to measurements on the products of GPT-2 small to XL at 24 to 256 rows: the
     // weight-streaming kernel runs its 16-row by 16-column workgroups in rounds of 256 whose time
     // grows with K (steeply beyond 3072, where a wavefront's share of K no longer fits its chunks);
-    // the tiled kernel's time is its k loop, a little more where edges make it take the checked path.
+    // the tiled kernel's time is its k loop, a little more where K makes it take the checked loop.
     const int col_tiles = (N + 15) / 16, row_blocks16 = (M + 15) / 16;
     auto streaming_is_faster = [&]() {
         const double rounds = static_cast<double>((static_cast<long>(col_tiles) * row_blocks16 + 255) / 256);
         const double streaming = 2.0 + rounds * (K <= 3072 ? 1.2 + 0.0008 * K : 0.0025 * K);
         const double blocks = static_cast<double>((M + 63) / 64) * ((N + 63) / 64);
-        const bool ragged = M % 64 != 0 || N % 64 != 0 || K % 64 != 0;
+        const bool ragged = K % 64 != 0;
         const double tiled = 5.0 + 0.18 * (K / 64.0) * std::max(1.0, blocks / 256.0) + (ragged ? 2.0 : 0.0) +
                              (M <= 32 ? 4.0 : 0.0);       // (up to 32 rows the tiled kernel has one shape, 32x128)
         return streaming <= tiled;
