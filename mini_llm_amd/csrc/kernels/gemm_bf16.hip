@@ -1016,7 +1016,7 @@ static int gemm_bf16_dispatch(const void* A, int lda, const void* W, int ldw, co
         const double streaming = 2.0 + rounds * (K <= 3072 ? 1.2 + 0.0008 * K : 0.0025 * K);
         const double blocks = static_cast<double>((M + 63) / 64) * ((N + 63) / 64);
         const bool ragged = K % 64 != 0;
-        const double tiled = 5.0 + 0.18 * (K / 64.0) * std::max(1.0, blocks / 256.0) + (ragged ? 2.0 : 0.0) +
+        const double tiled = (blocks <= 128 ? 4.0 : 5.0) + 0.18 * (K / 64.0) * std::max(1.0, blocks / 256.0) + (ragged ? 2.0 : 0.0) +
                              (M <= 32 ? 4.0 : 0.0);       // (up to 32 rows the tiled kernel has one shape, 32x128)
         return streaming <= tiled;
     };
@@ -1031,13 +1031,14 @@ static int gemm_bf16_dispatch(const void* A, int lda, const void* W, int ldw, co
         // grows with its tile's area, less so for large tiles (they move fewer bytes per flop). So
         // each shape is priced as rounds x area / efficiency, the efficiencies fitted to measurements
         // at 2048 rows on the products of GPT-2 small to XL, and the cheapest runs. Few workgroups
-        // (one round for every shape) thus take the smallest tiles, which spread over more units.
+        // (one round for every shape) thus take the smallest tiles, which spread over more units
+        // (64x32 where even 64x64 tiles leave most units idle: decode at 48 to 128 rows).
         struct Shape { int bm, bn; double efficiency; };
-        static const Shape shapes[] = {{128, 256, 1.05}, {128, 192, 1.0}, {128, 128, 0.9},
-                                       {64, 128, 0.7},   {64, 96, 0.65},  {64, 64, 0.55}};
+        static const Shape shapes[] = {{128, 256, 1.05}, {128, 192, 1.0}, {128, 128, 0.9}, {64, 128, 0.7},
+                                       {64, 96, 0.65},   {64, 64, 0.55}, {64, 32, 0.4}};
         int best = 0;
         double best_cost = 1e300;
-        for (int c = 0; c < 6; ++c) {
+        for (int c = 0; c < 7; ++c) {
             const long blocks = static_cast<long>((M + shapes[c].bm - 1) / shapes[c].bm) * ((N + shapes[c].bn - 1) / shapes[c].bn);
             const double cost = static_cast<double>((blocks + 255) / 256) * shapes[c].bm * shapes[c].bn / shapes[c].efficiency;
             if (cost < best_cost) { best_cost = cost; best = c; }
@@ -1053,7 +1054,8 @@ static int gemm_bf16_dispatch(const void* A, int lda, const void* W, int ldw, co
             case 2: if (long_k) TILE(2, 4, 2, 1, 64, 3, 2); else TILE(2, 4, 2, 1, 64, 3); break;
             case 3: TILE(2, 4, 1, 1, 64, 4); break;
             case 4: if (long_k) TILE(2, 3, 1, 1, 64, 5, 2); else TILE(2, 3, 1, 1, 64, 5); break;
-            default: if (long_k) TILE(2, 2, 1, 1, 64, 4, 2); else TILE(2, 2, 1, 1, 64, 4); break;
+            case 5: if (long_k) TILE(2, 2, 1, 1, 64, 4, 2); else TILE(2, 2, 1, 1, 64, 4); break;
+            default: TILE(2, 1, 1, 1, 64, 4, 2); break;     // 64x32 (few workgroups in all): two wavefronts, always two groups
         }
 #undef TILE
     }

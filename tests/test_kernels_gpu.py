@@ -123,9 +123,10 @@ def test_linear(ops, dtype, M, N, K, epi):
                                    (2040, 760, 136),       # 64x96 tiles, one round, ragged
                                    (2048, 768, 3072),      # 64x96 tiles, long K: two wavefront groups per workgroup
                                    (2040, 1800, 2056),     # 128x128 tiles, two groups, K not a multiple of their k tile
-                                   (300, 500, 4104),       # 64x64 tiles, two groups, ragged
+                                   (1000, 1000, 2056),     # 64x64 tiles, two groups, ragged
+                                   (300, 500, 4104),       # 64x32 tiles (few workgroups), long ragged K
                                    (1000, 1000, 40),       # 64x64 tiles, K below one k tile
-                                   (257, 257, 264)])       # 64x64 tiles, few workgroups
+                                   (257, 257, 264)])       # 64x32 tiles, few workgroups
 @pytest.mark.parametrize("epi", ["store", "add_residual"])
 def test_linear_bf16_tile_choices(ops, M, N, K, epi):
     """Every tile shape of the many-row product, with edges in all three dimensions."""
