@@ -393,7 +393,7 @@ def _decode_launch_shape(pairs: int, max_ctx_len: int):
     # the parallelism gains below about 2,000 keys (measured at 12 to 96 pairs). Few pairs get more
     # wavefronts each instead (measured: 12 are 1 to 3 % of a decode step faster than 8 up to 200
     # pairs at GPT-2 small to XL sizes, 3 % slower from 384 pairs).
-    return 1, (4 if pairs >= 512 else 8 if pairs > 256 else 12)
+    return 1, (4 if pairs >= 512 else 6 if pairs > 256 else 12)
 
 
 

@@ -413,7 +413,7 @@ def test_paged_attention_mixed_batch(ops, dtype, H, Hkv, dh, page):
 @pytest.mark.parametrize("H,Hkv,dh,page", [(12, 12, 64, 16), (4, 4, 16, 4), (3, 3, 32, 8), (6, 2, 128, 16),
                                            (2, 1, 256, 64), (5, 5, 48, 16)])
 @pytest.mark.parametrize("window", [0, 33])
-@pytest.mark.parametrize("shape", [None, (3, 4), (8, 2), (1, 8), (1, 16)])
+@pytest.mark.parametrize("shape", [None, (3, 4), (8, 2), (1, 6), (1, 16)])
 def test_paged_attention_decode_only(ops, dtype, H, Hkv, dh, page, window, shape):
     """Every query a single token: the decode kernel (power-of-two head sizes; others fall back),
     in its default launch shape and with the keys of a query split over 3 and 8 workgroups whose
