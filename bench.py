@@ -32,58 +32,62 @@ def small_config(n_layer, size="gpt2-small"):
                 activation_function="gelu_new", eos_token_id=50256, bos_token_id=50256)
 
 
-def matmul_params(cfg):
-    D, F = cfg["n_embd"], cfg["n_inner"]
-    return cfg["n_layer"] * (3 * D * D + D * D + 2 * D * F)
-
-
-def weight_bytes(cfg, esz):
-    D, F, L, V = cfg["n_embd"], cfg["n_inner"], cfg["n_layer"], cfg["vocab_size"]
-    vec = L * (3 * D + D + F + D + 4 * D) + 2 * D
-    return (matmul_params(cfg) + V * D) * esz + vec * 4
-
-
-def kv_bytes_per_token(cfg, esz):
-    return cfg["n_layer"] * 2 * cfg["n_embd"] * esz
-
-
 def decode_run(model_dir, dtype, batch, prompt_len, steps, warmup, cfg):
+    """Decode steps of `batch` requests through the whole engine. Every prompt is fed in ONE step before
+    the clock starts, so that all requests decode in lockstep from position prompt_len on. Returns
+    tokens/s, mean and median seconds per step, the mean context length, and the bytes one step has to
+    read (every weight once, and the cache of the live requests), taken from the model and the cache."""
     import torch
     from mini_llm_amd import Engine, EngineOptions, SamplingParams
     pages = batch * (cfg["n_positions"] // 16) + 16
     engine = Engine.from_pretrained(model_dir, dtype=dtype, device="cuda:0",
                                     options=EngineOptions(kv_block_size=16, total_kv_blocks=pages,
                                                           max_batch_num=max(batch, 1),
-                                                          max_tokens_per_step=max(2048, batch),
-                                                          prefill_chunk=1024))
+                                                          max_tokens_per_step=batch * prompt_len,
+                                                          prefill_chunk=prompt_len))
     g = torch.Generator().manual_seed(2)
     prompts = [torch.randint(0, cfg["vocab_size"], (prompt_len,), generator=g).tolist() for _ in range(batch)]
-    total_new = warmup + steps + 1 + batch      # requests that were prefilled first decode longer
+    # The workload generates up to 512 tokens per request (as many as the positions allow); the timed
+    # steps are taken from the middle of that stretch, so that their mean context is the workload's.
+    room = cfg["n_positions"] - prompt_len - 1
+    skip = max(0, min(512, room) // 2 - steps // 2 - warmup)
+    total_new = 1 + skip + warmup + steps
     assert prompt_len + total_new <= cfg["n_positions"], "the run would pass the last position"
     params = SamplingParams(max_new_tokens=total_new, ignore_eos=True)
     for p in prompts:
         engine.add_request(p, params)
-    # untimed: prefill until every request is decoding
-    while engine.scheduler.queue_length("decode") < batch:
-        engine.step()
-    for _ in range(warmup):
+    # untimed: the prompts (one step), then the warm-up steps
+    engine.step()
+    assert engine.scheduler.queue_length("decode") == batch, "the prompts did not fit one step"
+    for _ in range(skip + warmup):
         engine.step()
     torch.cuda.synchronize()
-    ctx0 = prompt_len + 1 + warmup
-    t0 = time.perf_counter()
+    ctx0 = prompt_len + 1 + skip + warmup
+    per_step = []
     n_tok = 0
+    t0 = t_prev = time.perf_counter()
     for _ in range(steps):
         n_tok += len(engine.step())
+        t_now = time.perf_counter()
+        per_step.append(t_now - t_prev)
+        t_prev = t_now
     torch.cuda.synchronize()
     dt = time.perf_counter() - t0
     assert n_tok == batch * steps, (n_tok, batch, steps)
     mean_ctx = ctx0 + (steps - 1) / 2.0
+    cost = engine.model.step_cost()
+    bytes_step = cost["weight_bytes"] + batch * mean_ctx * engine.runner.cache.bytes_per_token()
+    per_step.sort()
+    p50 = per_step[len(per_step) // 2]
     del engine
     torch.cuda.empty_cache()
-    return n_tok / dt, dt / steps, mean_ctx
+    return n_tok / dt, dt / steps, p50, mean_ctx, bytes_step
 
 
 def prefill_run(model_dir, dtype, cfg, n_req=2, n_tok=1024, reps=5):
+    """One step of n_req whole prompts of n_tok tokens (logits at the last place of each); the best of
+    `reps` runs. Flops from the model: products of every token, attention over the causal triangle,
+    the head's rows."""
     import torch
     from mini_llm_amd.engine.step import ModelRunner, StepEntry
     from mini_llm_amd.models import load_model
@@ -103,8 +107,9 @@ def prefill_run(model_dir, dtype, cfg, n_req=2, n_tok=1024, reps=5):
             runner.end_request(i)
     dt = min(times[2:])
     T = n_req * n_tok
-    D, V, L = cfg["n_embd"], cfg["vocab_size"], cfg["n_layer"]
-    flops = 2.0 * T * matmul_params(cfg) + L * n_req * 4.0 * D * (n_tok * (n_tok + 1) / 2) + 2.0 * D * V * n_req
+    cost = model.step_cost()
+    flops = (float(T) * cost["flops_per_token"] + n_req * cost["attention_flops_per_key"] * (n_tok * (n_tok + 1) / 2)
+             + float(n_req) * cost["flops_per_logits_row"])
     del runner, model
     torch.cuda.empty_cache()
     return T / dt, dt, flops
@@ -130,7 +135,7 @@ def serving_run(model_dir, dtype, cfg, n_req, prompt_lo, prompt_hi, new_tokens, 
         engine.add_request(torch.randint(0, cfg["vocab_size"], (n,), generator=g).tolist(), params)
     torch.cuda.synchronize()
     t0 = time.perf_counter()
-    n_out = n_steps = 0
+    n_out = n_steps = failed = 0
     first = None
     while engine.has_unfinished():
         outs = engine.step()
@@ -139,10 +144,10 @@ def serving_run(model_dir, dtype, cfg, n_req, prompt_lo, prompt_hi, new_tokens, 
             torch.cuda.synchronize()
             first = time.perf_counter() - t0
         n_out += sum(1 for o in outs if o.token >= 0)
+        failed += sum(1 for o in outs if o.token < 0)
     torch.cuda.synchronize()
     dt = time.perf_counter() - t0
     st = engine.stats()
-    failed = sum(1 for r in engine.requests.values() if r.failed)
     assert n_out == (n_req - failed) * new_tokens, (n_out, n_req, failed, new_tokens)
     assert st["free_pages"] == pages and engine.runner.manager.check() == ""
     return {"seconds": dt, "generated": n_out, "prompt_tokens": sum(lens), "steps": n_steps,
@@ -190,7 +195,11 @@ def main():
     ap.add_argument("--size", default="gpt2-small", choices=sorted(SIZES), help="layer sizes (default: configs[2])")
     ap.add_argument("--prompt-len", type=int, default=512)
     ap.add_argument("--no-points", action="store_true", help="skip the batch-1/64 and prefill measurements")
-    ap.add_argument("--prefill-only", action="store_true", help="measure only the 2,048-token prefill (profiling)")
+    ap.add_argument("--prefill-only", action="store_true", help="measure only the prefill step (profiling)")
+    ap.add_argument("--prefill-requests", type=int, default=2, help="with --prefill-only: prompts in the step")
+    ap.add_argument("--prefill-tokens", type=int, default=1024, help="with --prefill-only: tokens of each prompt")
+    ap.add_argument("--peaks-only", action="store_true",
+                    help="measure this GPU's streaming bandwidth and matrix-core rate and print them")
     ap.add_argument("--workload", default="decode", choices=["decode", "continuous", "kv-pressure"],
                     help="decode: the headline measurement; continuous / kv-pressure: a queue of requests "
                          "through the scheduler (BASELINE.json configs[3] and configs[4])")
@@ -202,28 +211,41 @@ def main():
     from mini_llm_amd import write_random_model
 
     cfg = small_config(args.layers, args.size)
-    esz = 2 if args.dtype == "bfloat16" else 4
-    steps = min(args.steps, cfg["n_positions"] - args.prompt_len - args.warmup - 2 - 64)
+    if args.peaks_only:
+        from mini_llm_amd.kernels.peaks import NOMINAL, measure_peaks
+        print(json.dumps({"metric": "measured peaks of this GPU", "measured": measure_peaks("cuda:0"),
+                          "published": NOMINAL}))
+        return 0
+    # all prompts are fed in one step, then 1 + warmup + steps tokens are generated for each request
+    room = cfg["n_positions"] - args.prompt_len - 1
+    if room < 2:
+        print(f"bench.py: prompts of {args.prompt_len} tokens leave no room to decode in {cfg['n_positions']} positions")
+        return 2
+    warmup = min(args.warmup, max(1, room // 6)) if args.warmup + args.steps > room else args.warmup
+    steps = min(args.steps, room - warmup)
     with tempfile.TemporaryDirectory() as d:
         write_random_model(dict(cfg), d, seed=2)
         if args.workload != "decode":
             return serving_main(args, cfg, d)
         if args.prefill_only:
-            ptps, pdt, flops = prefill_run(d, args.dtype, cfg)
-            print(json.dumps({"metric": "prefill tok/s at 2,048 tokens", "value": round(ptps, 1), "unit": "tok/s",
-                              "ms": round(pdt * 1e3, 4), "frac": round(flops / pdt / MFMA_PEAK[args.dtype], 5)}))
+            ptps, pdt, flops = prefill_run(d, args.dtype, cfg, args.prefill_requests, args.prefill_tokens)
+            print(json.dumps({"metric": f"prefill tok/s at {args.prefill_requests} x {args.prefill_tokens} tokens "
+                                        f"({args.size} sizes)", "value": round(ptps, 1), "unit": "tok/s",
+                              "ms": round(pdt * 1e3, 4), "tflops": round(flops / pdt / 1e12, 1),
+                              "frac": round(flops / pdt / MFMA_PEAK[args.dtype], 5)}))
             return 0
-        tps, step_s, mean_ctx = decode_run(d, args.dtype, args.batch, args.prompt_len, steps, args.warmup, cfg)
+        tps, step_s, p50_s, mean_ctx, bytes_step = decode_run(d, args.dtype, args.batch, args.prompt_len, steps,
+                                                             warmup, cfg)
         # The reference's own decode numbers at this workload (GPT-2 small, 512-token prompts; fp32 on a
         # TITAN V: /root/reference benchmark gpt2_decode_batch_sweep_512.csv:2-5), where it has one.
         reference_tps = {1: 116.9, 2: 223.1, 4: 438.6, 8: 854.4}.get(args.batch) \
             if (args.size == "gpt2-small" and args.prompt_len == 512 and cfg["n_layer"] == SIZES[args.size][0]) else None
-        bytes_step = weight_bytes(cfg, esz) + args.batch * mean_ctx * kv_bytes_per_token(cfg, esz)
         achieved = bytes_step / step_s
         rec = {
             "metric": f"decode tok/s at batch {args.batch} ({args.size} sizes, {args.prompt_len}-token prompts)",
-            "value": round(tps, 1), "unit": "tok/s", "n_gpus": 1, "steps": steps, "warmup": args.warmup,
-            "ms_per_step": round(step_s * 1e3, 4), "higher_is_better": True, "scaling": "weak",
+            "value": round(tps, 1), "unit": "tok/s", "n_gpus": 1, "steps": steps, "warmup": warmup,
+            "ms_per_step": round(step_s * 1e3, 4), "ms_per_step_p50": round(p50_s * 1e3, 4),
+            "higher_is_better": True, "scaling": "weak",
             "vs_baseline": round(tps / reference_tps, 2) if reference_tps else None, "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
             "data": "synthetic (random weights seed 2, uniform random token ids)",
             "config": {"model": args.size + "-sizes", "n_layer": cfg["n_layer"], "n_layer_full": SIZES[args.size][0],
@@ -234,7 +256,8 @@ def main():
                        "mean_context": round(mean_ctx, 1), "kv_block_size": 16, "parallelism": "single-gpu",
                        "baseline": (f"{reference_tps} tok/s: the reference, fp32, TITAN V" if reference_tps else "none")},
             "roofline": {"bound": "hbm", "achieved": round(achieved / 1e9, 2), "peak": HBM_PEAK / 1e9,
-                         "unit": "GB/s", "frac": round(achieved / HBM_PEAK, 5)},
+                         "unit": "GB/s", "frac": round(achieved / HBM_PEAK, 5),
+                         "bytes_per_step": int(bytes_step)},
         }
         if not args.no_points:
             ptps, pdt, flops = prefill_run(d, args.dtype, cfg)
@@ -243,9 +266,16 @@ def main():
             points = {}
             for b in (1, 64):
                 s = min(steps, 128)
-                v, _, _ = decode_run(d, args.dtype, b, args.prompt_len, s, min(args.warmup, 16), cfg)
+                v = decode_run(d, args.dtype, b, args.prompt_len, s, min(warmup, 16), cfg)[0]
                 points[f"decode_b{b}"] = round(v, 1)
             rec["points"] = points
+            # what this GPU gives on the engine's own micro-benchmarks, beside the published peaks
+            from mini_llm_amd.kernels.peaks import measure_peaks
+            peaks = measure_peaks("cuda:0")
+            rec["measured_peaks"] = peaks
+            rec["roofline"]["frac_of_measured"] = round(achieved / (peaks["hbm_read_GBps"] * 1e9), 5)
+            mfma = peaks["mfma_bf16_TFLOPs" if args.dtype == "bfloat16" else "mfma_f32_TFLOPs"] * 1e12
+            rec["prefill"]["frac_of_measured"] = round(flops / pdt / mfma, 5)
     print(json.dumps(rec))
     return 0
 

@@ -52,6 +52,7 @@ LIBRARIES: Dict[str, dict] = {
     "attention_decode": {"kind": "hip", "sources": ["kernels/attention_decode.hip"], "headers": ["kernels/common.h"]},
     "attention_prefill": {"kind": "hip", "sources": ["kernels/attention_prefill.hip"], "headers": ["kernels/common.h"]},
     "sampling": {"kind": "hip", "sources": ["kernels/sampling.hip"], "headers": ["kernels/common.h"]},
+    "peaks": {"kind": "hip", "sources": ["kernels/peaks.hip"], "headers": ["kernels/common.h"]},
 }
 
 _loaded: Dict[str, ctypes.CDLL] = {}

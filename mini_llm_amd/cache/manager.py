@@ -56,6 +56,8 @@ def _rt():
         "mllm_sched_on_token": (i, [vp, i64, i]),
         "mllm_sched_abort": (i, [vp, i64]),
         "mllm_sched_stop": (i, [vp, i64]),
+        "mllm_sched_forget": (i, [vp, i64]),
+        "mllm_sched_n_known": (i, [vp]),
         "mllm_sched_has_work": (i, [vp]),
         "mllm_sched_state": (i, [vp, i64]),
         "mllm_sched_generated": (i, [vp, i64]),
@@ -289,11 +291,13 @@ class CacheStorage:
             self._pools.append(pool)
             for j, c in enumerate(members[g]):
                 self._views[c] = KVCacheView(pool[j, 0], pool[j, 1], g, self.page_size, window)
+        self._state_views: List[StateCacheView] = []
         for c, spec in enumerate(specs):
             if isinstance(spec, StateCacheSpec):
                 slots = torch.zeros((self.n_state_slots,) + tuple(spec.shape), dtype=spec.dtype,
                                     device=self.device)
                 self._views[c] = StateCacheView(slots)
+                self._state_views.append(self._views[c])
         self.manager = CacheManager(self.group_specs, self.n_state_slots)
 
     @property
@@ -303,10 +307,26 @@ class CacheStorage:
     def view(self, cache: int):
         return self._views[cache]
 
+    def reset_fresh_states(self, ctx) -> None:
+        """Clears, on the device, the state slot of every request of the step that has no token
+        cached yet (``ctx.starts == 0``; a request that begins, or begins again after it was
+        preempted). Nothing to do for a model without state caches."""
+        if not self._state_views:
+            return
+        from ..kernels import ops
+        for view in self._state_views:
+            ops.reset_state(view.slots, ctx.state_slots, ctx.starts)
+
     def bytes_per_token(self) -> int:
         return sum(p.shape[0] * 2 * p.shape[3] * p.element_size() for p in self._pools)
 
+    def state_bytes_per_request(self) -> int:
+        return sum(v.slots[0].numel() * v.slots.element_size() for v in self._state_views)
+
     def poison(self, value: float = float("nan")) -> None:
-        """Fills every page with a value (tests: stale or unwritten pages must never be read)."""
+        """Fills every page and every state slot with a value (tests: a stale or unwritten page, or
+        a state that was not cleared when its request began, must never be read)."""
         for p in self._pools:
             p.fill_(value)
+        for v in self._state_views:
+            v.slots.fill_(value)

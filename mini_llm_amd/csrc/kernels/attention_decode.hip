@@ -45,13 +45,13 @@ __device__ __forceinline__ uint4 load_stream16(const T* p) {
     return make_uint4(v.x, v.y, v.z, v.w);
 }
 
-template <int N>
+template <typename T, int N>
 __device__ __forceinline__ void merge_state(float& m, float& l, float (&o)[N], float m2, float l2,
                                             const float (&o2)[N]) {
     // empty states carry a large negative finite maximum and zero sums: their weight is 0 or
     // (both empty) irrelevant
     const float mn = fmaxf(m, m2);
-    const float a = fast_exp2(m - mn), b = fast_exp2(m2 - mn);
+    const float a = exp2_for<T>(m - mn), b = exp2_for<T>(m2 - mn);
     l = l * a + l2 * b;
 #pragma unroll
     for (int e = 0; e < N; ++e) o[e] = o[e] * a + o2[e] * b;
@@ -165,13 +165,13 @@ decode_attention_kernel(// the first 16 dwords arrive in registers with the wave
         }
         // one rescale of the state for the whole batch of keys
         const float mn = fmaxf(m, mx);
-        const float a = fast_exp2(m - mn);
+        const float a = exp2_for<T>(m - mn);
         l *= a;
 #pragma unroll
         for (int e = 0; e < EPL; ++e) o[e] *= a;
 #pragma unroll
         for (int u = 0; u < UNR; ++u) {
-            const float pj = dot[u] > NEG ? fast_exp2(dot[u] - mn) : 0.f;
+            const float pj = dot[u] > NEG ? exp2_for<T>(dot[u] - mn) : 0.f;
             float vf[EPL];
             Vec16<T>::widen(vraw[u], vf);
             l += pj;
@@ -189,7 +189,7 @@ decode_attention_kernel(// the first 16 dwords arrive in registers with the wave
         for (int e = 0; e < EPL; ++e) d = fmaf(qf[e], kf[e], d);
         d = group_sum<LPK>(d);
         const float mn = fmaxf(m, d);
-        const float a = fast_exp2(m - mn), pj = fast_exp2(d - mn);
+        const float a = exp2_for<T>(m - mn), pj = exp2_for<T>(d - mn);
         l = l * a + pj;
 #pragma unroll
         for (int e = 0; e < EPL; ++e) o[e] = o[e] * a + pj * vf[e];
@@ -204,7 +204,7 @@ decode_attention_kernel(// the first 16 dwords arrive in registers with the wave
             float o2[EPL];
 #pragma unroll
             for (int e = 0; e < EPL; ++e) o2[e] = __shfl_xor(o[e], off, MLLM_WAVE);
-            merge_state<EPL>(m, l, o, m2, l2, o2);
+            merge_state<T, EPL>(m, l, o, m2, l2, o2);
         }
         __syncthreads();                      // earlier readers of the LDS arrays are done
         if (g == 0) {
@@ -223,7 +223,7 @@ decode_attention_kernel(// the first 16 dwords arrive in registers with the wave
                 float o2[EPL];
 #pragma unroll
                 for (int e = 0; e < EPL; ++e) o2[e] = sm_o[w][c * EPL + e];
-                merge_state<EPL>(m, l, o, sm_m[w], sm_l[w], o2);
+                merge_state<T, EPL>(m, l, o, sm_m[w], sm_l[w], o2);
             }
 #pragma unroll
             for (int off = LPK; off < MLLM_WAVE; off <<= 1) {
@@ -231,7 +231,7 @@ decode_attention_kernel(// the first 16 dwords arrive in registers with the wave
                 float o2[EPL];
 #pragma unroll
                 for (int e = 0; e < EPL; ++e) o2[e] = __shfl_xor(o[e], off, MLLM_WAVE);
-                merge_state<EPL>(m, l, o, m2, l2, o2);
+                merge_state<T, EPL>(m, l, o, m2, l2, o2);
             }
         }
     };
@@ -279,7 +279,7 @@ decode_attention_kernel(// the first 16 dwords arrive in registers with the wave
 #pragma unroll
             for (int e = 0; e < EPL; ++e)
                 o2[e] = __hip_atomic_load(&ws_o[sl * DH + c * EPL + e], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            merge_state<EPL>(m, l, o, m2, l2, o2);
+            merge_state<T, EPL>(m, l, o, m2, l2, o2);
         }
     }
     block_merge();

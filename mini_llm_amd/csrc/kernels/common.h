@@ -41,6 +41,11 @@ __device__ __forceinline__ uint32_t pack_bf16x2(float a, float b) {
 // 2^x by the hardware instruction alone: for arguments <= 0, where results below the normal
 // range may flush to zero (softmax weights).
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+// 2^x for a kernel instantiated for element type T: the bare instruction for bfloat16, the library's
+// full-range, full-precision exp2f for the 32-bit path.
+template <typename T> __device__ __forceinline__ float exp2_for(float x) {
+    return sizeof(T) == 4 ? exp2f(x) : __builtin_amdgcn_exp2f(x);
+}
 
 __device__ __forceinline__ float to_float(float v) { return v; }
 __device__ __forceinline__ float to_float(bf16_t v) { return bf16_to_float(v); }
@@ -158,17 +163,25 @@ __device__ __forceinline__ float gelu_tanh(float v) {
     const float u = 0.7978845608f * (v + 0.044715f * v * v * v);
     return v * __builtin_amdgcn_rcpf(1.f + __expf(-2.f * u));
 }
+// The same in full 32-bit precision (library tanhf, no approximate reciprocal): the 32-bit path.
+__device__ __forceinline__ float gelu_tanh_precise(float v) {
+    const float u = 0.7978845608f * (v + 0.044715f * v * v * v);
+    return 0.5f * v * (1.f + tanhf(u));
+}
 // GELU, exact form 0.5 v (1 + erf(v / sqrt 2)); the reference has only the tanh form.
 __device__ __forceinline__ float gelu_erf(float v) {
     return 0.5f * v * (1.f + erff(v * 0.70710678118654752440f));
 }
 
+// (a 32-bit output takes the full-precision activation: the 32-bit path has no fast approximations)
 template <typename OutT>
 __device__ __forceinline__ void epilogue(int mode, float acc, float bias, void* out, size_t idx) {
     float v = acc + bias;
     switch (mode) {
         case EPI_STORE: reinterpret_cast<OutT*>(out)[idx] = from_float<OutT>(v); break;
-        case EPI_GELU_TANH: reinterpret_cast<OutT*>(out)[idx] = from_float<OutT>(gelu_tanh(v)); break;
+        case EPI_GELU_TANH:
+            reinterpret_cast<OutT*>(out)[idx] = from_float<OutT>(sizeof(OutT) == 4 ? gelu_tanh_precise(v) : gelu_tanh(v));
+            break;
         case EPI_GELU_ERF: reinterpret_cast<OutT*>(out)[idx] = from_float<OutT>(gelu_erf(v)); break;
         case EPI_ADD_RESIDUAL: reinterpret_cast<float*>(out)[idx] += v; break;
         default: reinterpret_cast<float*>(out)[idx] = v; break;

@@ -1,4 +1,6 @@
 // Embedding, LayerNorm and key/value page writes for gfx950.
+#include <algorithm>
+
 #include "common.h"
 
 // ---------------------------------------------------------------------------
@@ -175,7 +177,35 @@ __global__ void kv_append_kernel(const T* __restrict__ src, int src_stride, int 
     }
 }
 
+// ---------------------------------------------------------------------------
+// Fixed-size per-request state: the slot of every request that starts at position 0 in this
+// step (starts[b] == 0: nothing of it is cached yet) is cleared before the layers run, on the
+// device, so that the step can be replayed as a graph. Slots < 0 (padding rows) are skipped.
+// One workgroup column per request; `words` 4-byte words per slot.
+// ---------------------------------------------------------------------------
+__global__ void reset_state_kernel(uint32_t* __restrict__ state, size_t words, const int* __restrict__ slots,
+                                   const int* __restrict__ starts) {
+    const int b = blockIdx.y;
+    const int slot = slots[b];
+    if (slot < 0 || starts[b] != 0) return;
+    uint32_t* row = state + static_cast<size_t>(slot) * words;
+    for (size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < words;
+         i += static_cast<size_t>(gridDim.x) * blockDim.x)
+        row[i] = 0u;
+}
+
 extern "C" {
+
+int mllm_reset_state(void* state, size_t slot_bytes, int n_slots, const int* slots, const int* starts, int B,
+                     hipStream_t stream) {
+    if (B <= 0 || slot_bytes == 0) return 0;
+    if (slot_bytes % 4 != 0 || (reinterpret_cast<uintptr_t>(state) & 3) != 0 || n_slots < 1) return -1;
+    const size_t words = slot_bytes / 4;
+    const unsigned gx = static_cast<unsigned>(std::min<size_t>((words + 255) / 256, 64));
+    reset_state_kernel<<<dim3(gx, B), 256, 0, stream>>>(static_cast<uint32_t*>(state), words, slots, starts);
+    MLLM_LAUNCH_CHECK();
+    return 0;
+}
 
 int mllm_embed(const int* ids, const int* pos, const void* wte, const void* wpe, float* x, int T, int D,
                int dtype, hipStream_t stream) {

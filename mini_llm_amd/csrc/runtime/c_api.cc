@@ -91,6 +91,8 @@ void mllm_sched_commit(void* s) { static_cast<Scheduler*>(s)->commit(); }
 int mllm_sched_on_token(void* s, int64_t id, int is_eos) { return static_cast<Scheduler*>(s)->on_token(id, is_eos != 0); }
 int mllm_sched_abort(void* s, int64_t id) { return static_cast<Scheduler*>(s)->abort(id); }
 int mllm_sched_stop(void* s, int64_t id) { return static_cast<Scheduler*>(s)->stop(id); }
+int mllm_sched_forget(void* s, int64_t id) { return static_cast<Scheduler*>(s)->forget(id); }
+int mllm_sched_n_known(void* s) { return static_cast<Scheduler*>(s)->n_known(); }
 int mllm_sched_has_work(void* s) { return static_cast<Scheduler*>(s)->has_work() ? 1 : 0; }
 int mllm_sched_state(void* s, int64_t id) { return static_cast<int>(static_cast<Scheduler*>(s)->state(id)); }
 int mllm_sched_generated(void* s, int64_t id) { return static_cast<Scheduler*>(s)->generated(id); }

@@ -34,12 +34,15 @@ bool Scheduler::try_plan_tokens(Req& r, int n, int* budget, int* n_seqs) {
 }
 
 // A request is admitted when a state slot is free and the pages for ALL the tokens
-// it has so far are free now (the reference reserves the whole prompt,
-// real_kv_allocator.cu:112-139). The pages themselves are taken portion by portion.
+// it has so far are free now and not promised to a prompt that is under way (the reference
+// reserves the whole prompt, real_kv_allocator.cu:112-139). The pages themselves are taken
+// portion by portion, so what a prompt under way has not taken yet counts as promised.
 bool Scheduler::admit(Req& r) {
     if (cache_->free_state_slots() < 1) return false;
     for (int g = 0; g < cache_->n_groups(); ++g) {
-        if (cache_->pages_needed_fresh(g, r.total_len) > cache_->free_pages(g)) return false;
+        int promised = 0;
+        for (int64_t id : prefill_) promised += cache_->pages_needed(id, g, reqs_.at(id).total_len);
+        if (cache_->pages_needed_fresh(g, r.total_len) + promised > cache_->free_pages(g)) return false;
     }
     if (cache_->add_request(r.id) < 0) return false;
     r.state = RequestState::Prefill;
@@ -231,6 +234,15 @@ int Scheduler::stop(int64_t id) {
     plan_.erase(std::remove_if(plan_.begin(), plan_.end(),
                                [id](const PlanEntry& e) { return e.id == id; }), plan_.end());
     finish(r, RequestState::Finished);
+    return 0;
+}
+
+int Scheduler::forget(int64_t id) {
+    auto it = reqs_.find(id);
+    if (it == reqs_.end()) return -2;
+    RequestState st = it->second.state;
+    if (st != RequestState::Finished && st != RequestState::Failed) return -1;
+    reqs_.erase(it);
     return 0;
 }
 

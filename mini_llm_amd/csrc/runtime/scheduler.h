@@ -79,11 +79,16 @@ public:
     // finished, not failed, and its pages are given back. 0 or -2.
     int stop(int64_t id);
 
+    // Drops the record of a finished or failed request (its id may be used again). 0; -1 if the
+    // request is still live; -2 if unknown.
+    int forget(int64_t id);
+
     bool has_work() const;
     RequestState state(int64_t id) const;
     int generated(int64_t id) const;
     bool pop_event(Event* e);
     const Counters& counters() const { return counters_; }
+    int n_known() const { return static_cast<int>(reqs_.size()); }
     int queue_length(int which) const;   // 0 waiting, 1 deferred_prefill, 2 prefill, 3 decode, 4 deferred_decode
 
 private:

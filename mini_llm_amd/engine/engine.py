@@ -38,8 +38,13 @@ class EngineOptions:
 @dataclass
 class RequestOutput:
     request_id: int
-    token: int
+    token: int                          # -1: no token (the request failed)
     finished: bool
+    error: Optional[str] = None         # why a request failed
+
+
+# A request's record leaves the engine (and the scheduler) with its final output: what a caller
+# wants to keep of it has arrived in the outputs by then, and its id may be used again.
 
 
 @dataclass
@@ -67,9 +72,9 @@ class Engine:
         self.scheduler = Scheduler(self.runner.manager, o.max_batch_num, o.max_tokens_per_step,
                                    o.prefill_chunk, model.max_positions)
         self.eos_token_id = model.config.eos_token_id
-        self.requests: Dict[int, _Request] = {}
+        self.requests: Dict[int, _Request] = {}     # live requests only
         self._next_id = 0
-        self._pending = None            # (PendingTokens, [(request id, finished by that token)]) of the step in flight
+        self._pending = None            # (PendingTokens, [(request, finished by that token)]) of the step in flight
 
     @classmethod
     def from_pretrained(cls, model_dir: str, dtype="bfloat16", device="cuda:0",
@@ -119,10 +124,20 @@ class Engine:
         self.requests[rid] = _Request(rid, ids, len(ids), params)
         return rid
 
-    def abort(self, request_id: int) -> None:
-        self.scheduler.abort(request_id)
+    def abort(self, request_id: int) -> List[int]:
+        """Ends a live request now; a token of it that is still in flight is dropped. Returns the
+        tokens it has generated so far."""
         r = self.requests[request_id]
+        self.scheduler.abort(request_id)
         r.finished, r.failed = True, "aborted"
+        self._drop(r)
+        return r.output
+
+    def _drop(self, r: _Request) -> None:
+        """Forgets a request whose final output is on its way to the caller."""
+        if self.requests.get(r.request_id) is r:
+            del self.requests[r.request_id]
+            self.scheduler.forget(r.request_id)
 
     def has_unfinished(self) -> bool:
         return self.scheduler.has_work() or self._pending is not None
@@ -138,10 +153,10 @@ class Engine:
             return []
         (handle, rows), self._pending = self._pending, None
         outputs = []
-        for (rid, done), tok in zip(rows, handle.result()):
-            r = self.requests.get(rid)
-            if r is None or r.failed or r.ended_early:
-                continue
+        for (r, done), tok in zip(rows, handle.result()):
+            if r.finished or self.requests.get(r.request_id) is not r:
+                continue                      # ended by an earlier token, or aborted
+            rid = r.request_id
             r.tokens.append(tok)
             if not done and self._is_eos(r, tok):
                 # the scheduler has planned on without knowing: take the request out now
@@ -149,6 +164,8 @@ class Engine:
                 r.ended_early = done = True
             r.finished = done
             outputs.append(RequestOutput(rid, tok, done))
+            if done:
+                self._drop(r)
         return outputs
 
     def step(self) -> List[RequestOutput]:
@@ -156,11 +173,12 @@ class Engine:
         outputs: List[RequestOutput] = []
         for rid, kind in self.scheduler.pop_events():
             if kind == "failed":
-                r = self.requests[rid]
-                if r.failed:                   # aborted by the caller, who knows
+                r = self.requests.get(rid)
+                if r is None:                  # aborted by the caller, who knows
                     continue
                 r.finished, r.failed = True, "the page pool cannot hold this request"
-                outputs.append(RequestOutput(rid, -1, True))
+                outputs.append(RequestOutput(rid, -1, True, r.failed))
+                self._drop(r)
         if not plan:
             return outputs + self._collect()
         sampled = [e for e in plan if e.want_last]
@@ -172,7 +190,7 @@ class Engine:
         if not self.options.overlap_decode or unread_portion:
             # the host knows every token it feeds: read what is in flight first
             outputs += self._collect()
-            live = [e for e in plan if not self.requests[e.request_id].finished]
+            live = [e for e in plan if e.request_id in self.requests]
             if len(live) != len(plan):        # ended by a token just read; the scheduler dropped them too
                 plan, sampled = live, [e for e in live if e.want_last]
                 if not plan:
@@ -185,7 +203,7 @@ class Engine:
             r.n_launched += 1
         # A token that the step in flight has sampled and the host has not read is fed on the device:
         # its row among that step's sampled tokens stands in for it.
-        in_flight = {rid: i for i, (rid, _) in enumerate(self._pending[1])} if self._pending else {}
+        in_flight = {r.request_id: i for i, (r, _) in enumerate(self._pending[1])} if self._pending else {}
         if fast:
             # every entry is one decoded token: the whole step runs from static buffers (a HIP graph)
             toks, src = [], []
@@ -212,7 +230,7 @@ class Engine:
             handle = self.runner.launch_step(entries, feed, temps, us)
         self.scheduler.commit()
         # the scheduler moves on as if no token were the end of sequence; `_collect` corrects it
-        rows = [(e.request_id, self.scheduler.on_token(e.request_id, False)) for e in sampled]
+        rows = [(self.requests[e.request_id], self.scheduler.on_token(e.request_id, False)) for e in sampled]
         outputs += self._collect()
         self._pending = (handle, rows) if handle is not None else None
         if not self.options.overlap_decode:
@@ -226,15 +244,20 @@ class Engine:
         if params is None or isinstance(params, SamplingParams):
             params = [params or SamplingParams()] * len(prompts)
         rids = [self.add_request(p, sp) for p, sp in zip(prompts, params)]
+        got: Dict[int, List[int]] = {rid: [] for rid in rids}
+        errors: Dict[int, str] = {}
         while self.has_unfinished():
-            self.step()
-        out = []
+            for o in self.step():
+                if o.request_id not in got:
+                    continue                  # a request the caller added beside these
+                if o.token < 0:
+                    errors[o.request_id] = o.error or "failed"
+                else:
+                    got[o.request_id].append(o.token)
         for rid in rids:
-            r = self.requests.pop(rid)
-            if r.failed:
-                raise RuntimeError(f"request {rid} failed: {r.failed}")
-            out.append(r.output)
-        return out
+            if rid in errors:
+                raise RuntimeError(f"request {rid} failed: {errors[rid]}")
+        return [got[rid] for rid in rids]
 
     def warmup(self, sampling: bool = False) -> List[int]:
         """Captures the decode graphs before the first real request needs them: for every batch size

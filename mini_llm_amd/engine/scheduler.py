@@ -80,6 +80,13 @@ class Scheduler:
         if self._lib.mllm_sched_stop(self._h, rid) != 0:
             raise KeyError(f"request {rid} is unknown")
 
+    def forget(self, rid: int) -> None:
+        """Drops the record of a finished or failed request; its id may then be used again."""
+        self._lib.mllm_sched_forget(self._h, rid)
+
+    def n_known(self) -> int:
+        return self._lib.mllm_sched_n_known(self._h)
+
     def has_work(self) -> bool:
         return bool(self._lib.mllm_sched_has_work(self._h))
 

@@ -44,7 +44,9 @@ class StepContext:
     cu_q: torch.Tensor            # [B+1] row range of each sequence
     ctx_len: torch.Tensor         # [B] tokens cached once this step is done
     starts: torch.Tensor          # [B] tokens cached before this step
-    state_slots: torch.Tensor     # [B] per-request state slot
+    state_slots: torch.Tensor     # [B] per-request state slot; < 0: a padding row, whose state is neither
+                                  #     read nor written (as a token whose page row in ``slots`` is < 0
+                                  #     writes no key or value)
     logit_rows: torch.Tensor      # [n_logits] rows whose logits are wanted
     block_tables: List[torch.Tensor]   # per group [B, max_blocks]
     slots: List[torch.Tensor]          # per group [T] row of the page pool each token writes
@@ -126,6 +128,28 @@ class ModelRunner:
         # plans on the host; on the GPU those steps are captured and replayed as HIP graphs.
         self.fast_decode = bool(getattr(model, "graph_safe", True))
         self.use_graphs = self.device.type == "cuda" and self.fast_decode
+        # Kernel scratch is sized now for the largest decode batch, so that no captured graph is left
+        # with the address of a buffer that a larger batch replaced; should one grow after all (a
+        # step that wants more logits rows than that), the graphs are dropped and captured again.
+        from ..kernels import ops
+        if self.device.type == "cuda":
+            rows = -(-max(max_num_seqs, 1) // 8) * 8
+            n_heads = max((getattr(m, "n_heads", 0) for m in self._mixers()), default=0)
+            head_dim = max((getattr(m, "head_dim", 0) for m in self._mixers()), default=0)
+            ops.reserve_scratch(self.device, rows, model.vocab_size, n_heads, head_dim)
+            ops.on_scratch_growth(self._drop_graphs)
+
+    def _mixers(self):
+        return [getattr(layer, "mixer", None) for layer in getattr(self.model, "layers", [])]
+
+    def _drop_graphs(self) -> None:
+        self._graphs.clear()
+
+    def forward(self, ctx: "StepContext") -> Optional[torch.Tensor]:
+        """The model over one batch: fresh requests (no token cached yet) get their fixed-size state
+        cleared on the device first, then every layer runs."""
+        self.cache.reset_fresh_states(ctx)
+        return self.model.forward(ctx, self.cache)
 
     # -- cache bookkeeping for callers without a scheduler ---------------------------
     def ensure_request(self, rid: int) -> None:
@@ -229,7 +253,7 @@ class ModelRunner:
                     mgr.free_request(rid)
                 raise
         ctx = self.build_context(entries)
-        logits = self.model.forward(ctx, self.cache)
+        logits = self.forward(ctx)
         if manage_cache:
             for e in entries:
                 mgr.commit(e.request_id, mgr.length(e.request_id) + len(e.tokens))
@@ -243,7 +267,7 @@ class ModelRunner:
             grown = torch.zeros(n, dtype=torch.int32, device=self.device)
             if self._tok_out is not None:
                 grown[:self._tok_out.numel()].copy_(self._tok_out)     # tokens a later launch may still take
-                self._graphs.clear()                                   # captured graphs hold the old address
+                self._drop_graphs()                                    # captured graphs hold the old address
             self._tok_out = grown
 
     def launch_step(self, entries: Sequence[StepEntry], feed_rows: Sequence[int],
@@ -270,7 +294,7 @@ class ModelRunner:
             host, buf = self._staging_src.take(ctx.n_tokens)
             host[:] = src
             ops.select_tokens(ctx.token_ids, _Staging.upload(buf, ctx.n_tokens)[:ctx.n_tokens], self._tok_out)
-        logits = self.model.forward(ctx, self.cache)
+        logits = self.forward(ctx)
         if logits is None:
             return None
         n = logits.shape[0]
@@ -338,12 +362,15 @@ class PendingTokens:
 class DecodeGraph:
     """A decode step of fixed batch size on static buffers: embedding, every layer, the head and
     the sampler; on the GPU captured once and replayed as a HIP graph. Per step the host only
-    refreshes the index arrays (one copy) and later reads the sampled tokens, which every graph
-    of a runner leaves in the same device buffer, so that the next step can take its input
-    tokens from there before the host has seen them.
+    refreshes the index arrays (one copy: temperatures and uniform numbers travel in the same
+    buffer) and later reads the sampled tokens, which every graph of a runner leaves in the same
+    device buffer, so that the next step can take its input tokens from there before the host has
+    seen them.
 
-    Rows beyond the live batch repeat row 0 without writing to the cache, so one graph serves
-    every batch size up to its own.
+    Rows beyond the live batch repeat row 0 but write nothing: their page rows and their state
+    slots are -1. So one graph serves every batch size up to its own. The run that precedes the
+    capture (it loads the kernels) is made of such rows only, so a step's effects on keys, values
+    and state happen once, in the replay.
     """
 
     def __init__(self, runner: ModelRunner, batch: int, greedy: bool):
@@ -359,13 +386,13 @@ class DecodeGraph:
         B = batch
         self.offs = _layout(B, B, B, self.max_blocks)
         self.n_ctx_ints = self.offs[-1]
-        self.n_ints = self.n_ctx_ints + B                  # then: the row of the last launch each token comes from
+        # then: the row of the last launch each token comes from, temperatures, uniform numbers
+        self.n_ints = self.n_ctx_ints + 3 * B
         self.dev_ints = torch.zeros(self.n_ints, dtype=torch.int32, device=dev)
-        self.src_rows = self.dev_ints[self.n_ctx_ints:]
+        self.src_rows = self.dev_ints[self.n_ctx_ints:self.n_ctx_ints + B]
+        self.d_float = self.dev_ints[self.n_ctx_ints + B:].view(torch.float32).view(2, B)
         self.ctx = runner._context(self.dev_ints, self.offs, B, B, B, self.max_blocks, 1,
                                    self.max_blocks[0] * runner.page_size if self.max_blocks else 1)
-        self.h_float = torch.zeros((2, B), dtype=torch.float32, pin_memory=on_gpu)
-        self.d_float = torch.zeros((2, B), dtype=torch.float32, device=dev)
         self.out = runner._tok_out[:B]
         # two host buffers in turn: one may still be unread when the next step's copy is queued
         self.h_out = [torch.zeros(B, dtype=torch.int32, pin_memory=on_gpu) for _ in range(2)]
@@ -376,13 +403,14 @@ class DecodeGraph:
 
     def _forward(self) -> None:
         self._ops.select_tokens(self.ctx.token_ids, self.src_rows, self.runner._tok_out)
-        logits = self.runner.model.forward(self.ctx, self.runner.cache)
+        logits = self.runner.forward(self.ctx)
         if self.greedy:
             self._ops.argmax(logits, self.out)
         else:
             self._ops.sample(logits, self.d_float[0], self.d_float[1], self.out)
 
-    def _fill(self, request_ids, tokens, src_rows) -> None:
+    def _fill(self, request_ids, tokens, src_rows, temperatures, uniforms, live: bool = True) -> None:
+        """Refreshes the static buffers for this batch. ``live`` False: every row is a padding row."""
         r, B, n = self.runner, self.batch, len(request_ids)
         ids = np.empty(B, dtype=np.int64)
         ids[:n] = request_ids
@@ -396,48 +424,49 @@ class DecodeGraph:
         if tok.min() < 0 or tok.max() >= r.model.vocab_size:
             raise StepError(f"token ids must lie in [0, {r.model.vocab_size})")
         seg[7][:] = np.arange(B, dtype=np.int32)
+        first_pad = n if live else 0
+        seg[6][first_pad:] = -1                      # padding rows touch no state
         for g in range(len(self.max_blocks)):
-            seg[9 + 2 * g][n:] = -1              # padding rows write nothing to the cache
-        src = host[self.n_ctx_ints:self.n_ints]
+            seg[9 + 2 * g][first_pad:] = -1          # and write nothing to the pages
+        src = host[self.n_ctx_ints:self.n_ctx_ints + B]
         src[:n] = src_rows
         src[n:] = src_rows[0]
-        self.h_cu_q, self.h_starts, self.h_state_slots = seg[3], seg[5], seg[6]
+        fl = host[self.n_ctx_ints + B:self.n_ints].view(np.float32).reshape(2, B)
+        fl[:] = 0.0
+        if not self.greedy:
+            fl[0, :n] = temperatures
+            fl[1, :n] = uniforms
         _Staging.upload(buf, self.n_ints, self.dev_ints)
 
     def launch(self, request_ids, tokens, src_rows, temperatures, uniforms) -> PendingTokens:
         n = len(request_ids)
-        self._fill(request_ids, tokens, src_rows)
-        if not self.greedy:
-            h = self.h_float.numpy()
-            h[0, :n] = temperatures
-            h[1, :n] = uniforms
-            h[0, n:] = 0.0
-            self.d_float.copy_(self.h_float, non_blocking=True)
-        if not self.capture:
+        if self.capture and self.graph is None:
+            # First use: run once eagerly (loads the kernels), with rows that write nothing, then
+            # capture. The run overwrites the sampled tokens that this step may be fed from, so they
+            # are set aside.
+            self._fill(request_ids, tokens, src_rows, temperatures, uniforms, live=False)
+            fed = self.runner._tok_out.clone()
             self._forward()
-        else:
-            if self.graph is None:
-                # First use: run once eagerly (loads the kernels, sizes their scratch), then capture.
-                # The eager run's effects are the step's own (same keys and values written, same
-                # tokens sampled); the fed-back tokens are set aside, since it overwrites them.
-                fed = self.runner._tok_out.clone()
-                self._forward()
-                torch.cuda.synchronize()
-                self.runner._tok_out.copy_(fed)
-                self.graph = torch.cuda.CUDAGraph()
-                # No graph may be destroyed while the stream captures (HIP refuses it and the process
-                # ends), and a dropped engine's graphs may sit in a reference cycle until the collector
-                # runs: so it does not run during the capture. (Running it before every capture instead
-                # costs more than the capture.)
-                gc_was_enabled = gc.isenabled()
-                gc.disable()
-                try:
-                    with torch.cuda.graph(self.graph):
-                        self._forward()
-                finally:
-                    if gc_was_enabled:
-                        gc.enable()
+            torch.cuda.synchronize()
+            self.runner._tok_out.copy_(fed)
+            self.graph = torch.cuda.CUDAGraph()
+            # No graph may be destroyed while the stream captures (HIP refuses it and the process
+            # ends), and a dropped engine's graphs may sit in a reference cycle until the collector
+            # runs: so it does not run during the capture. (Running it before every capture instead
+            # costs more than the capture.)
+            gc_was_enabled = gc.isenabled()
+            gc.disable()
+            try:
+                with torch.cuda.graph(self.graph):
+                    self._forward()
+            finally:
+                if gc_was_enabled:
+                    gc.enable()
+        self._fill(request_ids, tokens, src_rows, temperatures, uniforms)
+        if self.capture:
             self.graph.replay()
+        else:
+            self._forward()
         self._turn ^= 1
         host = self.h_out[self._turn]
         host.copy_(self.out, non_blocking=True)

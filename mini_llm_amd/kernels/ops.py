@@ -115,6 +115,24 @@ def select_tokens(ids: torch.Tensor, src: torch.Tensor, prev: torch.Tensor) -> t
     return ids
 
 
+def reset_state(state: torch.Tensor, slots: torch.Tensor, starts: torch.Tensor) -> None:
+    """Clears row ``slots[b]`` of ``state`` ([n_slots, ...]) for every b with ``starts[b] == 0`` and
+    ``slots[b] >= 0``: the fixed-size state of requests that begin in this step."""
+    _gpu(state, slots, starts)
+    B = slots.numel()
+    _i32(slots, "slots")
+    _i32(starts, "starts", B)
+    if not state.is_contiguous() or state.dim() < 1:
+        raise KernelError("state must be contiguous [n_slots, ...]")
+    slot_bytes = (state.numel() // max(state.shape[0], 1)) * state.element_size()
+    lib = load_library("elementwise")
+    rc = lib.mllm_reset_state(_p(state), ctypes.c_size_t(slot_bytes), state.shape[0], _p(slots), _p(starts), B,
+                              _stream())
+    if rc == -1:
+        raise KernelError(f"reset_state: a slot of {slot_bytes} bytes is no multiple of 4 bytes")
+    _check(rc, "reset_state")
+
+
 def layernorm(x: torch.Tensor, gamma: torch.Tensor, beta: Optional[torch.Tensor], eps: float,
               out: torch.Tensor, rows: Optional[torch.Tensor] = None) -> torch.Tensor:
     """out[i,:] = LayerNorm(x[rows[i] if rows else i,:]); statistics in fp32."""
@@ -137,9 +155,9 @@ def layernorm(x: torch.Tensor, gamma: torch.Tensor, beta: Optional[torch.Tensor]
     return out
 
 
-def linear_scatters_kv(dtype: torch.dtype, rows: int) -> bool:
-    """Whether ``linear(..., kv_scatter=...)`` can write a fused QKV product's keys and values
-    to the pages itself: the many-row bf16 kernel does."""
+def _scatter_is_fused(dtype: torch.dtype, rows: int) -> bool:
+    """Whether the product kernel that runs for these rows writes a fused QKV product's keys and
+    values to the pages in its epilogue: the many-row bf16 kernel does."""
     return dtype == torch.bfloat16 and rows > 64
 
 
@@ -150,9 +168,10 @@ def linear(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], out: 
     epilogue: "store" | "gelu_tanh" | "gelu_erf" (out in a's dtype), "add_residual"
     (out fp32, accumulated in place), "store_f32" (out fp32).
 
-    ``kv_scatter=(slots, k_pages, v_pages, q_cols)`` (only with "store" and where
-    ``linear_scatters_kv`` says so): the columns after the first q_cols are keys, then values, of
-    kv_dim = k_pages.shape[1] columns each, and row m's also go to row slots[m] (>= 0) of the pages.
+    ``kv_scatter=(slots, k_pages, v_pages, q_cols)`` (only with "store"): the columns after the
+    first q_cols are keys, then values, of kv_dim = k_pages.shape[1] columns each, and row m's also
+    go to row slots[m] (>= 0) of the pages: in the product's epilogue where the kernel that runs
+    for these sizes has one, otherwise by a copy kernel after it.
     """
     _gpu(a, w, bias, out)
     _rows2d(a, "a")
@@ -170,8 +189,17 @@ def linear(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], out: 
     if bias is not None and (bias.dtype != torch.float32 or bias.numel() != N or not bias.is_contiguous()):
         raise KernelError(f"bias must be contiguous fp32 [{N}]")
     mode = EPILOGUES[epilogue]
-    if kv_scatter is not None and a.dtype != torch.bfloat16:
-        raise KernelError("linear: the key/value scatter exists for bfloat16 only")
+    if kv_scatter is not None:
+        if epilogue != "store":
+            raise KernelError("linear: the key/value scatter needs the plain store")
+        if not _scatter_is_fused(a.dtype, M):
+            slots, k_pages, v_pages, q_cols = kv_scatter
+            kv_dim = k_pages.shape[1]
+            if N != q_cols + 2 * kv_dim:
+                raise KernelError(f"linear: {N} columns are not {q_cols} + 2 x {kv_dim}")
+            linear(a, w, bias, out, epilogue)
+            kv_append(out, q_cols, q_cols + kv_dim, kv_dim, k_pages, v_pages, slots)
+            return out
     if a.dtype == torch.float32:
         lib = load_library("gemm_f32")
         rc = lib.mllm_gemm_f32(_p(a), a.stride(0), _p(w), w.stride(0), _p(bias), _p(out), out.stride(0),
@@ -182,8 +210,6 @@ def linear(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], out: 
             slots, k_pages, v_pages, q_cols = kv_scatter
             _gpu(slots, k_pages, v_pages)
             kv_dim = k_pages.shape[1]
-            if epilogue != "store" or not linear_scatters_kv(a.dtype, M):
-                raise KernelError("linear: the key/value scatter needs the plain store and more than 64 bf16 rows")
             _i32(slots, "slots", M)
             for name, pg in (("k_pages", k_pages), ("v_pages", v_pages)):
                 if pg.dim() != 2 or pg.shape[1] != kv_dim or not pg.is_contiguous() or pg.dtype != a.dtype:
@@ -381,8 +407,64 @@ def paged_attention(q: torch.Tensor, q_col: int, n_heads: int, n_kv_heads: int, 
     return out
 
 
-_DECODE_WS = {}
 DECODE_SHAPE_OVERRIDE = None      # (nsplit, waves): set by tests of the split path and by tuning scripts
+DECODE_MAX_SPLIT = 8              # most workgroups that share one (token, head) pair's keys
+
+
+# ---------------------------------------------------------------------------------
+# Scratch buffers: device memory that a kernel needs beyond its inputs and outputs
+# (argmax partial results, partial outputs and counters of the split decode attention).
+# One set per device. A captured HIP graph keeps the raw address of the buffer it was
+# captured with, so a buffer is never replaced behind a graph's back: callers that
+# capture graphs reserve room for their largest launch first (``reserve_scratch``),
+# and if a buffer must grow after all, everyone registered with ``on_scratch_growth``
+# is told, and drops the graphs it holds.
+# ---------------------------------------------------------------------------------
+_SCRATCH: dict = {}               # (device, name) -> tensor
+_GROWTH_LISTENERS: list = []      # weak references to bound methods
+
+
+def on_scratch_growth(method) -> None:
+    """Registers a bound method that is called (with no arguments) whenever a scratch buffer has
+    been replaced by a larger one. Held weakly."""
+    import weakref
+    _GROWTH_LISTENERS.append(weakref.WeakMethod(method))
+
+
+def _scratch(device, name: str, numel: int, dtype: torch.dtype, zero: bool = False) -> torch.Tensor:
+    key = (torch.device(device), name)
+    t = _SCRATCH.get(key)
+    if t is not None and t.numel() >= numel:
+        return t
+    grown = (torch.zeros if zero else torch.empty)(numel, dtype=dtype, device=device)
+    _SCRATCH[key] = grown
+    if t is not None:
+        alive = []
+        for ref in _GROWTH_LISTENERS:
+            fn = ref()
+            if fn is not None:
+                fn()
+                alive.append(ref)
+        _GROWTH_LISTENERS[:] = alive
+    return grown
+
+
+def scratch_address(device, name: str) -> int:
+    """Address of a scratch buffer (0 if it does not exist yet): tests check that it stays put."""
+    t = _SCRATCH.get((torch.device(device), name))
+    return 0 if t is None else t.data_ptr()
+
+
+def reserve_scratch(device, rows: int, vocab: int, n_heads: int = 0, head_dim: int = 0) -> None:
+    """Makes the scratch buffers large enough for ``rows`` sampled rows of ``vocab`` logits and for
+    decode attention over ``rows`` tokens of ``n_heads`` heads, so that no later launch up to these
+    sizes replaces them."""
+    if torch.device(device).type != "cuda":
+        return
+    chunks = load_library("sampling").mllm_argmax_chunks(int(vocab))
+    _argmax_scratch(device, rows * chunks)
+    if n_heads and head_dim:
+        _decode_workspace(device, rows * n_heads, DECODE_MAX_SPLIT, head_dim)
 
 
 def _decode_launch_shape(pairs: int, max_ctx_len: int):
@@ -399,19 +481,21 @@ def _decode_launch_shape(pairs: int, max_ctx_len: int):
 
 def _decode_workspace(device, pairs: int, nsplit: int, head_dim: int):
     """Scratch of the split decode attention: partial outputs and a zeroed counter per
-    (token, head). It is kept per device and only ever grows; launches on one stream use it
-    one after the other."""
-    need_f = pairs * nsplit * (head_dim + 2)
-    ws, counters = _DECODE_WS.get(device, (None, None))
-    if ws is None or ws.numel() < need_f:
-        ws = torch.empty(max(need_f, 1 << 16), dtype=torch.float32, device=device)
-    if counters is None or counters.numel() < pairs:
-        counters = torch.zeros(max(pairs, 4096), dtype=torch.int32, device=device)
-    _DECODE_WS[device] = (ws, counters)
+    (token, head) (the kernel leaves the counters at zero). Launches on one stream use it one
+    after the other."""
+    if nsplit <= 1:
+        need_f = 1                      # one workgroup per pair exchanges nothing
+    else:
+        need_f = pairs * nsplit * (head_dim + 2)
+    ws = _scratch(device, "decode_partials", max(need_f, 1 << 16), torch.float32)
+    counters = _scratch(device, "decode_counters", max(pairs, 4096), torch.int32, zero=True)
     return ws, counters
 
 
-_ARGMAX_WS = {}
+def _argmax_scratch(device, n: int):
+    """Partial results of the first stage of argmax: a value and an index per (row, chunk)."""
+    return (_scratch(device, "argmax_values", max(n, 4096), torch.float32),
+            _scratch(device, "argmax_indices", max(n, 4096), torch.int32))
 
 
 def argmax(logits: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
@@ -424,12 +508,7 @@ def argmax(logits: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
     _i32(out, "out", n)
     lib = load_library("sampling")
     chunks = lib.mllm_argmax_chunks(V)
-    key = logits.device
-    pv, pi = _ARGMAX_WS.get(key, (None, None))
-    if pv is None or pv.numel() < n * chunks:
-        pv = torch.empty(max(n * chunks, 4096), dtype=torch.float32, device=logits.device)
-        pi = torch.empty(max(n * chunks, 4096), dtype=torch.int32, device=logits.device)
-        _ARGMAX_WS[key] = (pv, pi)
+    pv, pi = _argmax_scratch(logits.device, n * chunks)
     _check(lib.mllm_argmax(_p(logits), logits.stride(0), n, V, _p(out), _p(pv), _p(pi), _stream()), "argmax")
     return out
 

@@ -72,6 +72,53 @@ class DecoderModel:
             specs += self.head.param_specs(p)
         return specs
 
+    def step_cost(self) -> dict:
+        """What a step costs, read off the parts (for roofline arithmetic, whatever the architecture):
+
+        ``weight_bytes``      bytes of weights that every step reads once whatever its batch (every linear
+                              map's matrix and bias, norm gains and shifts, the head's matrix; embedding
+                              and position tables are gathered by row and not counted);
+        ``flops_per_token``   matrix-product flops of the layers per token (2 x in x out of every linear
+                              map, per call of the execution order);
+        ``flops_per_logits_row``  the head's product for one wanted row;
+        ``attention_flops_per_key``  flops per (token, attended key) summed over the attention calls
+                              (4 x query width: scores and value mix).
+        """
+        from ..parts.linear import Linear
+
+        def linears(part):
+            return [v for v in vars(part).values() if isinstance(v, Linear)] if part is not None else []
+
+        def vectors(part):
+            out = []
+            for v in (vars(part).values() if part is not None else ()):
+                if isinstance(v, torch.Tensor) and v.dim() == 1:
+                    out.append(v)
+                elif isinstance(v, Norm):
+                    out += vectors(v)
+            return out
+
+        nbytes = lambda t: 0 if t is None else t.numel() * t.element_size()
+        weight_bytes = 0
+        for layer in self.layers:
+            for part in (layer, getattr(layer, "mixer", None), getattr(layer, "feed_forward", None)):
+                for lin in linears(part):
+                    weight_bytes += nbytes(lin.weight) + nbytes(lin.bias)
+                weight_bytes += sum(nbytes(v) for v in vectors(part))
+        weight_bytes += sum(nbytes(v) for v in vectors(self.final_norm))
+        head_w = self.embedding.weight if isinstance(self.head, TiedHead) else getattr(self.head, "weight", None)
+        weight_bytes += nbytes(head_w)
+        flops = attn = 0
+        for call in self.order:
+            layer = self.layers[call.layer]
+            for part in (getattr(layer, "mixer", None), getattr(layer, "feed_forward", None)):
+                flops += sum(2 * lin.in_features * lin.out_features for lin in linears(part))
+            q_dim = getattr(getattr(layer, "mixer", None), "q_dim", 0)
+            attn += 4 * q_dim
+        head_flops = 2 * self.embedding.size * self.vocab_size
+        return {"weight_bytes": weight_bytes, "flops_per_token": flops, "flops_per_logits_row": head_flops,
+                "attention_flops_per_key": attn}
+
     def forward(self, ctx, cache) -> Optional[torch.Tensor]:
         """Runs the step's tokens through every call of the execution order and returns
         fp32 logits ``[len(ctx.logit_rows), vocab]`` (None if no logits are wanted)."""

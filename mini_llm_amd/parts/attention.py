@@ -53,10 +53,10 @@ class CausalSelfAttention(Mixer):
         T = h.shape[0]
         g = cache_view.group
         qkv = torch.empty((T, self.q_dim + 2 * self.kv_dim), dtype=self.dtype, device=h.device)
-        # Prompt portions: the product writes the new keys and values to the pages itself, unless a
-        # position encoding still has to turn them. (Single tokens: the attention kernel does.)
-        scatter = (write and self.position is None and ctx.max_q_len > 1
-                   and ops.linear_scatters_kv(self.dtype, T))
+        # Prompt portions: the QKV product is asked to put the new keys and values into the pages
+        # (how is the linear map's business), unless a position encoding still has to turn them.
+        # Single tokens: the attention kernel writes them.
+        scatter = write and self.position is None and ctx.max_q_len > 1
         opts = {"kv_scatter": (ctx.slots[g], cache_view.k_pages, cache_view.v_pages, self.q_dim)} if scatter else {}
         if isinstance(h, NormedInput):
             h.linear(self.qkv, qkv, "store", **opts)

@@ -23,6 +23,30 @@ TINY_B = dict(architectures=["GPT2LMHeadModel"], model_type="gpt2", n_layer=3, n
 TINY = {"a": (TINY_A, 0, 4), "b": (TINY_B, 1, 8)}     # config, seed, page size
 
 
+# The layer sizes of GPT-2 small and GPT-2 XL (width, heads, inner width, vocabulary, positions as in the
+# real models; two layers): the sizes the benchmarks run, where other kernels and tile shapes are chosen
+# than at the tiny sizes.
+REAL_SMALL = dict(architectures=["GPT2LMHeadModel"], model_type="gpt2", n_layer=2, n_embd=768, n_head=12,
+                  n_inner=3072, vocab_size=50257, n_positions=1024, layer_norm_epsilon=1e-5,
+                  activation_function="gelu_new", eos_token_id=50256, bos_token_id=50256)
+REAL_XL = dict(REAL_SMALL, n_embd=1600, n_head=25, n_inner=6400)
+REAL = {"small2": (REAL_SMALL, 2, 16), "xl2": (REAL_XL, 4, 16)}
+CONFIGS = {**TINY, **REAL}
+
+
+@pytest.fixture(scope="session")
+def real_model_dirs(tmp_path_factory):
+    """Model folders at GPT-2 small and XL layer sizes (two layers each), random weights."""
+    from mini_llm_amd.weights.random_init import write_random_model
+    import mini_llm_amd.models  # noqa: F401
+    out = {}
+    for name, (cfg, seed, _) in REAL.items():
+        d = tmp_path_factory.mktemp(f"real_{name}")
+        write_random_model(dict(cfg), str(d), seed)
+        out[name] = str(d)
+    return out
+
+
 @pytest.fixture(scope="session")
 def tiny_model_dirs(tmp_path_factory):
     """Model folders of the two tiny configurations, random weights, made once per session."""

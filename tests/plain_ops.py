@@ -50,12 +50,23 @@ def _gelu_erf(v):
     return 0.5 * v * (1.0 + torch.erf(v / math.sqrt(2.0)))
 
 
-def linear_scatters_kv(dtype, rows):
-    return False
+def reset_state(state, slots, starts):
+    for b in range(slots.numel()):
+        if int(slots[b]) >= 0 and int(starts[b]) == 0:
+            state[int(slots[b])] = 0
+
+
+ROW_BY_ROW = False     # True (set by install()): every output row is a matrix-vector product of its own, so that a
+                       # row's result cannot depend on how many rows share the call (the library may block a
+                       # product differently for different row counts)
 
 
 def linear(a, w, bias, out, epilogue="store", kv_scatter=None):
-    y = a.to(PRECISE) @ w.to(PRECISE).T
+    if ROW_BY_ROW:
+        w64 = w.to(PRECISE)
+        y = torch.stack([w64 @ a[i].to(PRECISE) for i in range(a.shape[0])])
+    else:
+        y = a.to(PRECISE) @ w.to(PRECISE).T
     if bias is not None:
         y = y + bias.to(PRECISE)
     if epilogue == "gelu_tanh":
@@ -132,7 +143,7 @@ def sample(logits, temperature, u, out):
     return out
 
 
-_NAMES = ("embed", "select_tokens", "layernorm", "linear", "linear_scatters_kv", "ln_linear", "kv_append", "paged_attention", "argmax", "sample")
+_NAMES = ("embed", "select_tokens", "reset_state", "layernorm", "linear", "ln_linear", "kv_append", "paged_attention", "argmax", "sample")
 
 
 def install(monkeypatch):
@@ -141,3 +152,5 @@ def install(monkeypatch):
     g = globals()
     for name in _NAMES:
         monkeypatch.setattr(ops, name, g[name])
+    import sys
+    monkeypatch.setattr(sys.modules[__name__], "ROW_BY_ROW", True)

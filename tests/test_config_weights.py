@@ -124,6 +124,92 @@ def test_random_model_folder(tmp_path):
     assert not torch.equal(_tensors(d3)["wpe.weight"], t["wpe.weight"])
 
 
+def test_random_values_follow_the_published_recipe():
+    """The generator is a specification, not a library call: element i of tensor `name` under `seed`
+    is recomputed here with Python integers and math.* only, and a fixed vector pins the constants."""
+    import math
+    from mini_llm_amd.weights.random_init import normal_values
+    M = (1 << 64) - 1
+
+    def mix(x):
+        z = (x + 0x9E3779B97F4A7C15) & M
+        z = ((z ^ (z >> 30)) * 0xBF58476D1CE4E5B9) & M
+        z = ((z ^ (z >> 27)) * 0x94D049BB133111EB) & M
+        return z ^ (z >> 31)
+
+    def fnv(b):
+        h = 0xCBF29CE484222325
+        for c in b:
+            h = ((h ^ c) * 0x100000001B3) & M
+        return h
+
+    def value(seed, name, i, mean, std):
+        key = mix(seed) ^ fnv(name.encode())
+        a, b = mix((key + 2 * i) & M), mix((key + 2 * i + 1) & M)
+        u1, u2 = ((a >> 11) + 1) / 2.0 ** 53, (b >> 11) / 2.0 ** 53
+        return mean + std * math.sqrt(-2.0 * math.log(u1)) * math.cos(2.0 * math.pi * u2)
+
+    assert mix(0) == 0xE220A8397B1DCDAF and fnv(b"wte.weight") == 0x61D3A46D83BC4189
+    got = normal_values(2, "wte.weight", 6, 0.0, 0.02)
+    assert [round(float(v), 9) for v in got[:3]] == [-0.011919891, 0.005637622, -0.020101186]
+    for seed, name, mean, std in ((2, "wte.weight", 0.0, 0.02), (7, "h.3.ln_1.weight", 1.0, 0.1)):
+        v = normal_values(seed, name, 1000, mean, std)
+        for i in (0, 1, 17, 999):
+            assert abs(float(v[i]) - value(seed, name, i, mean, std)) <= 1e-7 * max(1.0, abs(mean))
+    # a value depends on (seed, name, index) only: a window of a tensor equals the same window of the whole
+    whole = normal_values(5, "t", (1 << 18) * 3 + 11, 0.0, 1.0)
+    assert (normal_values(5, "t", 4097, 0.0, 1.0, first=(1 << 18) - 100) == whole[(1 << 18) - 100:(1 << 18) + 3997]).all()
+    assert abs(float(whole.mean())) < 5e-3 and abs(float(whole.std()) - 1.0) < 5e-3
+    assert abs(float((whole ** 4).mean()) - 3.0) < 0.05                                  # normal, not merely unit variance
+    assert not (normal_values(6, "t", 64, 0.0, 1.0) == whole[:64]).any()
+    assert not (normal_values(5, "u", 64, 0.0, 1.0) == whole[:64]).any()
+
+
+def test_a_tensor_keeps_its_values_when_the_model_changes(tmp_path):
+    """Random weights are keyed by tensor name: a model with one more layer has the same first layers."""
+    d2 = write_random_model(dict(TINY_A), str(tmp_path / "l2"), seed=3)
+    d3 = write_random_model(dict(TINY_A, n_layer=3), str(tmp_path / "l3"), seed=3)
+    t2, t3 = _tensors(d2), _tensors(d3)
+    assert set(t2) < set(t3)
+    same = [n for n in t2 if torch.equal(t2[n], t3[n])]
+    # (the residual projections' spread depends on the number of layers, so they differ)
+    assert sorted(set(t2) - set(same)) == sorted(f"h.{i}.{p}.c_proj.weight" for i in range(2) for p in ("attn", "mlp"))
+
+
+def test_loader_reads_shards_and_half_precision(tmp_path):
+    """A checkpoint split over two files named by model.safetensors.index.json, stored in float16."""
+    d = write_random_model(dict(TINY_B), str(tmp_path / "whole"), seed=4, weights_dtype="float16")
+    t = _tensors(d)
+    assert t["wte.weight"].dtype == torch.float16
+    sharded = tmp_path / "sharded"
+    sharded.mkdir()
+    names = sorted(t)
+    parts = {"model-00001-of-00002.safetensors": names[:len(names) // 2],
+             "model-00002-of-00002.safetensors": names[len(names) // 2:]}
+    for fname, ns in parts.items():
+        save_file({n: t[n] for n in ns}, str(sharded / fname))
+    json.dump({"metadata": {}, "weight_map": {n: f for f, ns in parts.items() for n in ns}},
+              open(sharded / "model.safetensors.index.json", "w"))
+    json.dump(json.load(open(os.path.join(d, "config.json"))), open(sharded / "config.json", "w"))
+    for dtype in (torch.float32, torch.bfloat16):
+        a, b = load_model(d, dtype, "cpu"), load_model(str(sharded), dtype, "cpu")
+        for sa, sb in zip(a.param_specs(), b.param_specs()):
+            assert sa.name == sb.name
+        assert torch.equal(a.embedding.weight, b.embedding.weight) and a.embedding.weight.dtype == dtype
+        assert torch.equal(a.embedding.weight, t["wte.weight"].to(dtype))
+        assert torch.equal(a.layers[2].feed_forward.down.weight, b.layers[2].feed_forward.down.weight)
+        assert torch.equal(b.layers[2].feed_forward.down.weight, t["h.2.mlp.c_proj.weight"].t().to(dtype))
+        assert torch.equal(b.layers[1].norm1.gamma, t["h.1.ln_1.weight"])
+    # a tensor in two shards is an error that names it; a shard the index names but that is not there too
+    save_file({names[0]: t[names[0]], **{n: t[n] for n in parts["model-00002-of-00002.safetensors"]}},
+              str(sharded / "model-00002-of-00002.safetensors"))
+    with pytest.raises(WeightsError, match="two files"):
+        load_model(str(sharded), "float32", "cpu")
+    os.remove(sharded / "model-00001-of-00002.safetensors")
+    with pytest.raises((WeightsError, SafetensorsError, OSError)):
+        load_model(str(sharded), "float32", "cpu")
+
+
 def test_loader_places_and_converts(tmp_path):
     d = write_random_model(dict(TINY_A), str(tmp_path / "m"), seed=0, weights_dtype="float32")
     t = _tensors(d)

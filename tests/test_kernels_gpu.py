@@ -163,7 +163,6 @@ def test_linear_bf16_scatters_keys_and_values(ops, M, H, Hkv, dh, K):
     v0 = _rand((rows, kv_dim), torch.bfloat16, g)
     kp, vp = k0.clone().to(DEV), v0.clone().to(DEV)
     out = torch.empty((M, N), dtype=torch.bfloat16, device=DEV)
-    assert ops.linear_scatters_kv(torch.bfloat16, M)
     ops.linear(a.to(DEV), w.to(DEV), bias.to(DEV), out, "store", kv_scatter=(perm.to(DEV), kp, vp, q_cols))
     plain = torch.empty((M, N), dtype=torch.bfloat16, device=DEV)
     ops.linear(a.to(DEV), w.to(DEV), bias.to(DEV), plain, "store")
@@ -176,8 +175,15 @@ def test_linear_bf16_scatters_keys_and_values(ops, M, H, Hkv, dh, K):
     kr, vr = k0.clone(), v0.clone()
     plain_ops.kv_append(out.cpu(), q_cols, q_cols + kv_dim, kv_dim, kr, vr, perm)
     assert torch.equal(kp.cpu(), kr) and torch.equal(vp.cpu(), vr)
+    # few rows: the product's kernel has no such epilogue and a copy kernel follows it; same contract
+    kp8, vp8 = k0.clone().to(DEV), v0.clone().to(DEV)
+    ops.linear(a[:8].to(DEV), w.to(DEV), bias.to(DEV), out[:8], "store", kv_scatter=(perm[:8].to(DEV), kp8, vp8, q_cols))
+    kr, vr = k0.clone(), v0.clone()
+    plain_ops.kv_append(out[:8].cpu(), q_cols, q_cols + kv_dim, kv_dim, kr, vr, perm[:8])
+    assert torch.equal(kp8.cpu(), kr) and torch.equal(vp8.cpu(), vr)
     with pytest.raises(ops.KernelError, match="scatter"):
-        ops.linear(a[:8].to(DEV), w.to(DEV), None, out[:8], "store", kv_scatter=(perm[:8].to(DEV), kp, vp, q_cols))
+        ops.linear(a.to(DEV), w.to(DEV), None, torch.empty((M, N), dtype=torch.float32, device=DEV), "store_f32",
+                   kv_scatter=(perm.to(DEV), kp, vp, q_cols))
 
 
 @pytest.mark.parametrize("M", [1, 8, 16, 17, 48, 64])

@@ -151,8 +151,12 @@ def _define_toy():
 
     @register_mixer("toy_running_mean", replace=True)
     class RunningMean(Mixer):
-        """state <- decay * state + (1 - decay) * h_t, token by token; x_t += gain * state."""
-        graph_safe = False           # it walks the batch on the host
+        """state <- decay * state + (1 - decay) * h_t, token by token; x_t += gain * state.
+
+        All on the device (torch operations over the step's index arrays, nothing read on the
+        host), so decode steps of a model that holds it can be captured as a graph. A request's
+        slot is empty when it begins: the cache storage clears it, not the mixer. Rows whose
+        state slot is < 0 are padding and touch no state."""
 
         def __init__(self, size, decay, dtype, device):
             super().__init__(dtype, device)
@@ -168,15 +172,21 @@ def _define_toy():
             return StateCacheSpec((self.size,), torch.float32)
 
         def forward(self, h, ctx, cache_view, x, write=True):
-            for b in range(ctx.n_seqs):
-                lo, hi = int(ctx.h_cu_q[b]), int(ctx.h_cu_q[b + 1])
-                slot = int(ctx.h_state_slots[b])
-                s = cache_view.slots[slot]
-                if int(ctx.h_starts[b]) == 0:
-                    s.zero_()                      # a new request starts from an empty state
-                for t in range(lo, hi):
-                    s.mul_(self.decay).add_(h[t].float(), alpha=1 - self.decay)
-                    x[t] += self.gain * s
+            state = cache_view.slots                                   # [n_slots, size]
+            n_slots = state.shape[0]
+            lo, hi = ctx.cu_q[:-1].long(), ctx.cu_q[1:].long()
+            slot = ctx.state_slots.long()
+            which = torch.arange(n_slots, device=state.device)
+            for k in range(ctx.max_q_len):                             # the k-th token of every sequence
+                t = lo + k
+                live = (t < hi) & (slot >= 0)
+                t = torch.where(live, t, torch.zeros_like(t))
+                before = state[slot.clamp(min=0)]                      # rows of padding entries are not used
+                s = torch.where(live[:, None], self.decay * before + (1 - self.decay) * h[t].float(),
+                                torch.zeros_like(before))
+                own = ((slot[:, None] == which[None, :]) & live[:, None]).float()      # [B, n_slots], one-hot rows
+                state.copy_(torch.where(own.sum(0)[:, None] > 0, own.T @ s, state))
+                x.index_add_(0, t, self.gain * s)
 
     @dataclasses.dataclass(frozen=True)
     class ToyConfig(ModelConfig):
@@ -293,11 +303,52 @@ def test_toy_architecture_with_a_stateful_mixer(tmp_path, dtype):
         assert fed[r] == len(ids)
         ref = _toy_plain(w, cfg, ids)
         assert (torch.cat(got[r]).double() - ref).abs().max() <= tol, r
-    assert not model.graph_safe and not runner.use_graphs
-    # a slot that is used again starts from an empty state
+    assert model.graph_safe and runner.use_graphs
+    # a slot that is used again starts from an empty state (the storage clears it on the device)
     runner.end_request(3)
+    runner.cache.poison()
     out = runner.step([StepEntry(4, seqs[3], list(range(9)))]).float().cpu()
     assert (out.double() - _toy_plain(w, cfg, seqs[3])).abs().max() <= tol
+
+
+def test_stateful_toy_mixer_decodes_through_captured_graphs(tmp_path):
+    """The toy model's decode steps run as HIP graphs of 16 rows for 9 requests: the 7 padding rows
+    and the run that precedes the capture must leave every request's state alone, a state slot
+    must be empty when its request begins, and tokens must equal greedy decoding of the plain
+    whole-sequence implementation."""
+    from safetensors import safe_open
+    from mini_llm_amd import Engine, EngineOptions, SamplingParams, write_random_model
+    from mini_llm_amd.models import load_model
+    _define_toy()
+    cfg = dict(architectures=["ToyLM"], vocab=203, width=48, heads=3, decay=0.75, eps=1e-5)
+    d = write_random_model(cfg, str(tmp_path / "toy"), seed=5)
+    with safe_open(d + "/model.safetensors", framework="pt") as f:
+        w = {k: f.get_tensor(k).double() for k in f.keys()}
+    g = torch.Generator().manual_seed(1)
+    prompts = [torch.randint(0, 203, (3 + i,), generator=g).tolist() for i in range(9)]
+    new = 7
+
+    def plain_greedy(ids):
+        ids, out = list(ids), []
+        for _ in range(new):
+            logits = _toy_plain(w, cfg, ids)[-1]
+            top = torch.topk(logits, 2).values
+            out.append((int(logits.argmax()), float(top[0] - top[1])))
+            ids.append(out[-1][0])
+        return out
+
+    engine = Engine(load_model(d, "float32", DEV), EngineOptions(kv_block_size=4, total_kv_blocks=64, max_batch_num=12,
+                                                                max_tokens_per_step=64, prefill_chunk=8))
+    engine.runner.cache.poison()
+    assert engine.runner.use_graphs
+    for round_ in range(2):                       # the second round reuses slots that hold old states
+        outs = engine.generate(prompts, SamplingParams(max_new_tokens=new, ignore_eos=True))
+        assert any(k[0] == 16 for k in engine.runner._graphs), "no 16-row decode graph was used"
+        for p, o in zip(prompts, outs):
+            for i, (tok, gap) in enumerate(plain_greedy(p)):
+                assert o[i] == tok or gap < 1e-4, (round_, p, i, o, tok)
+                if o[i] != tok:
+                    break
 
 
 # ---------------------------------------------------------------------------------------------
@@ -463,7 +514,7 @@ def _routed_plain(w, cfg, ids):
 
 ROUTED_CFG = dict(architectures=["ToyRoutedLM"], vocab=157, width=64, heads=4, groups=2, experts=3, window=6,
                   base=50.0, eps=1e-5)
-ROUTED_SEED = 30
+ROUTED_SEED = 35
 
 
 def _routed_sequences():

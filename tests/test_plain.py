@@ -151,6 +151,51 @@ def test_whole_model_against_library_routines(tiny_model_dirs, name):
     assert not torch.allclose(P.forward_logits(cfg, w, [ids[0], ids[0]])[1], mine[0])
 
 
+def test_block_arrangement_is_pinned_by_invariants(tiny_model_dirs):
+    """Where the norms and the residual sums stand, fixed by two cases that need no second arrangement
+    of the whole model to compare with.
+
+    (1) Both residual projections (attention c_proj, MLP c_proj) zero, weights and biases: every layer
+        adds nothing, so logits = ln_f(embedding) wte^T. A model without the final norm, or with a norm
+        ON the stream (post-norm), fails.
+    (2) One layer whose attention c_proj has zero weights and a bias b: the attention sub-layer adds
+        exactly b to every row, so ln_2 must see x + b (pre-norm, sequential), and the result is
+        x + b + MLP(ln_2(x + b)), computed here with library routines. A parallel arrangement
+        (ln_2 sees x) or a post-norm one fails."""
+    cfg, w = P.read_model(tiny_model_dirs["b"])
+    D, eps = cfg["n_embd"], cfg["layer_norm_epsilon"]
+    ids = [7, 7, 900, 41, 3, 512, 88, 7, 19]
+    emb = F.embedding(torch.tensor(ids), w["wte.weight"]) + w["wpe.weight"][:len(ids)]
+    head = lambda x: F.linear(F.layer_norm(x, (D,), w["ln_f.weight"], w["ln_f.bias"], eps), w["wte.weight"])
+
+    w1 = dict(w)
+    for i in range(cfg["n_layer"]):
+        for part in ("attn", "mlp"):
+            w1[f"h.{i}.{part}.c_proj.weight"] = torch.zeros_like(w[f"h.{i}.{part}.c_proj.weight"])
+            w1[f"h.{i}.{part}.c_proj.bias"] = torch.zeros_like(w[f"h.{i}.{part}.c_proj.bias"])
+    assert (P.forward_logits(cfg, w1, ids) - head(emb)).abs().max() <= 1e-12
+    assert (P.forward_logits(cfg, w, ids) - head(emb)).abs().max() > 1e-3       # the layers do count otherwise
+
+    one = dict(cfg, n_layer=1)
+    w2 = dict(w)
+    w2["h.0.attn.c_proj.weight"] = torch.zeros_like(w["h.0.attn.c_proj.weight"])
+    b = 0.1 * torch.sin(torch.arange(D, dtype=D64))                               # a few times the stream
+    w2["h.0.attn.c_proj.bias"] = b
+    x1 = emb + b
+    h = F.layer_norm(x1, (D,), w["h.0.ln_2.weight"], w["h.0.ln_2.bias"], eps)
+    inner = F.gelu(F.linear(h, w["h.0.mlp.c_fc.weight"].T, w["h.0.mlp.c_fc.bias"]))      # config b: the erf form
+    x2 = x1 + F.linear(inner, w["h.0.mlp.c_proj.weight"].T, w["h.0.mlp.c_proj.bias"])
+    got = P.forward_logits(one, w2, ids)
+    assert (got - head(x2)).abs().max() <= 1e-10
+    # what the wrong arrangements would give is far away
+    h_par = F.layer_norm(emb, (D,), w["h.0.ln_2.weight"], w["h.0.ln_2.bias"], eps)
+    par = x1 + F.linear(F.gelu(F.linear(h_par, w["h.0.mlp.c_fc.weight"].T, w["h.0.mlp.c_fc.bias"])),
+                        w["h.0.mlp.c_proj.weight"].T, w["h.0.mlp.c_proj.bias"])
+    assert (got - head(par)).abs().max() > 1e-2, (got - head(par)).abs().max()
+    post = F.layer_norm(x1, (D,), w["h.0.ln_1.weight"], w["h.0.ln_1.bias"], eps)            # a norm on the stream
+    assert (got - head(post + F.linear(inner, w["h.0.mlp.c_proj.weight"].T, w["h.0.mlp.c_proj.bias"]))).abs().max() > 1e-2
+
+
 def test_parts_in_the_wrong_place_are_seen(tiny_model_dirs):
     """Post-norm instead of pre-norm, a missing final norm, an untied or biased head, a wrong
     activation: each moves the logits far beyond any tolerance the engine is held to."""

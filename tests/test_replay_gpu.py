@@ -11,7 +11,7 @@ import torch
 
 import replay_cases as rc
 import replay_util as ru
-from conftest import TINY
+from conftest import CONFIGS, TINY
 
 pytestmark = pytest.mark.gpu
 DTYPES = ["float32", "bfloat16"]
@@ -21,7 +21,7 @@ def _runner(model_dir, name, dtype, n_pages, page=None):
     from mini_llm_amd.engine.step import ModelRunner
     from mini_llm_amd.models import load_model
     model = load_model(model_dir, dtype, "cuda:0")
-    runner = ModelRunner(model, page or TINY[name][2], n_pages, 8)
+    runner = ModelRunner(model, page or CONFIGS[name][2], n_pages, 8)
     runner.cache.poison()          # an unwritten or stale page that is read shows up as NaN
     return runner
 
@@ -36,7 +36,26 @@ def test_schedule_families_match_plain(tiny_model_dirs, name, family, dtype):
     n_pages = ru.peak_tokens(steps) // page
     runner = _runner(tiny_model_dirs[name], name, dtype, n_pages)
     out = ru.run_in_process(runner, steps)
-    rc.check_against_plain(tiny_model_dirs[name], name, reqs, steps, out, dtype)
+    rc.check_against_plain(tiny_model_dirs[name], name, reqs, steps, out, dtype, label=family)
+    assert runner.manager.check() == ""
+    assert runner.manager.free_pages(0) == n_pages and runner.manager.n_requests() == 0
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", ["small2", "xl2"])
+@pytest.mark.parametrize("family", ["whole", "decode_tail", "chunks", "mixed"])
+def test_schedule_families_match_plain_at_real_layer_sizes(real_model_dirs, name, family, dtype):
+    """The same four families at the layer sizes of GPT-2 small and XL (two layers, the real vocabulary):
+    the sizes at which the engine picks the matrix-core attention, the 64-wide decode attention, the
+    two-tile and shared-tile few-row products, the large tiles and the staged head. Requests of the
+    reference's page-edge lengths (5, 15, 16, 17) and of 41, 130 and 300 tokens."""
+    reqs = rc.requests_for(name)
+    steps = rc.families(reqs, large=True)[family]
+    skip = rc.thin(steps)
+    n_pages = ru.peak_tokens(steps) // 16
+    runner = _runner(real_model_dirs[name], name, dtype, n_pages)
+    out = ru.run_in_process(runner, steps)
+    rc.check_against_plain(real_model_dirs[name], name, reqs, steps, out, dtype, skip=skip, label=family)
     assert runner.manager.check() == ""
     assert runner.manager.free_pages(0) == n_pages and runner.manager.n_requests() == 0
 
@@ -49,12 +68,16 @@ def test_schedules_agree_with_each_other(tiny_model_dirs, dtype):
     for fam, steps in rc.families(reqs, seed=5).items():
         runner = _runner(tiny_model_dirs["b"], "b", dtype, 64)
         outs[fam] = ru.collect(steps, ru.run_in_process(runner, steps), 1000)
-    tol = 2e-5 if dtype == "float32" else 4e-2
+    tol = 2e-6 if dtype == "float32" else 8e-3
+    worst = 0.0
     for rid, toks in reqs.items():
         for pos in range(len(toks)):
             base = outs["whole"][rid][pos]
             for fam in ("decode_tail", "chunks", "mixed"):
-                assert np.abs(outs[fam][rid][pos] - base).max() <= tol, (fam, rid, pos)
+                d = np.abs(outs[fam][rid][pos] - base).max()
+                worst = max(worst, d)
+                assert d <= tol, (fam, rid, pos, d)
+    print(f"worst difference between schedules [{dtype}]: {worst:.3e} (allowed {tol:.1e})")
 
 
 @pytest.mark.parametrize("dtype", DTYPES)

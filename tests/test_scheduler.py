@@ -70,6 +70,38 @@ def test_refused_requests():
     assert produced == {1: 1}              # the prompt fills every position: one token, then the length cap
 
 
+def test_pages_promised_to_a_prompt_under_way_are_not_given_to_the_next():
+    """Two prompts of two portions each whose pages fit only one at a time: the second is admitted
+    only when the first has finished, so nobody is preempted and recomputed."""
+    cm, s = make(n_pages=12, page=4, budget=32, chunk=16)
+    s.add_request(1, 32, 2)                # 8 pages for the prompt, 9 with its second token
+    s.add_request(2, 32, 2)
+    p = s.schedule()
+    assert [(e.request_id, e.n_tokens) for e in p] == [(1, 16)]
+    assert s.state(2) == "deferred_prefill"          # 4 pages free are promised to request 1
+    s.commit()
+    produced, plans = drive(s)
+    assert produced == {1: 2, 2: 2}
+    assert s.counters()["preemptions"] == 0
+    assert all(len({e.request_id for e in plan}) == 1 for plan in plans)
+    assert cm.free_pages() == 12 and cm.check() == ""
+
+
+def test_finished_requests_can_be_forgotten():
+    cm, s = make()
+    s.add_request(1, 5, 1)
+    s.add_request(2, 5, 3)
+    s.schedule(); s.commit()
+    assert s.on_token(1, False) and not s.on_token(2, False)
+    assert s.n_known() == 2
+    s.forget(1)
+    s.forget(2)                            # still live: stays
+    assert s.n_known() == 1 and s.state(1) == "unknown" and s.state(2) == "decode_ready"
+    s.add_request(1, 3, 1)                 # the id is free again
+    produced, _ = drive(s)
+    assert produced == {1: 1, 2: 2}
+
+
 def test_prompts_are_cut_under_the_budget_and_decodes_come_first():
     cm, s = make(budget=12, chunk=8)
     s.add_request(1, 20, 3)
@@ -273,9 +305,17 @@ def test_outputs_of_steps_arrive_in_order_and_abort_in_flight(cpu_ops, tiny_mode
             seen[out.request_id].append((out.token, out.finished))
         steps += 1
         if steps == 4:
-            e.abort(b)               # b has a token in flight; it is dropped
-    assert [t for t, _ in seen[a]] == e.requests[a].output and len(seen[a]) == 6
-    assert [f for _, f in seen[a]] == [False] * 5 + [True]
-    assert e.requests[b].failed == "aborted" and len(seen[b]) < 9
-    assert [t for t, _ in seen[b]] == e.requests[b].output
+            b_out = e.abort(b)       # b has a token in flight; it is dropped
+    assert len(seen[a]) == 6 and [f for _, f in seen[a]] == [False] * 5 + [True]
+    ref = _engine(tiny_model_dirs["a"], kv_block_size=4, total_kv_blocks=60, max_batch_num=4)
+    whole = ref.generate([[5, 6, 7, 8], [9, 10, 11]], SamplingParams(max_new_tokens=9, ignore_eos=True))
+    assert [t for t, _ in seen[a]] == whole[0][:6]
+    assert 0 < len(seen[b]) < 9 and [t for t, _ in seen[b]] == b_out == whole[1][:len(b_out)]
     assert e.stats()["free_pages"] == 60 and e.runner.manager.check() == ""
+    # nothing of a finished or aborted request stays behind, and its id can be used again
+    assert e.requests == {} and e.scheduler.n_known() == 0
+    again = e.add_request([5, 6, 7, 8], SamplingParams(max_new_tokens=6, ignore_eos=True), request_id=a)
+    toks = []
+    while e.has_unfinished():
+        toks += [o.token for o in e.step() if o.request_id == again]
+    assert toks == whole[0][:6]

@@ -52,7 +52,7 @@ def test_schedules_agree_bitwise_on_cpu(cpu_ops, tiny_model_dirs):
         for pos in range(len(toks)):
             base = outs["whole"][rid][pos]
             for fam in ("decode_tail", "chunks", "mixed"):
-                np.testing.assert_allclose(outs[fam][rid][pos], base, rtol=0, atol=1e-6)
+                assert np.array_equal(outs[fam][rid][pos], base), (fam, rid, pos)
 
 
 def test_step_errors(cpu_ops, tiny_model_dirs):
