@@ -51,7 +51,8 @@ LIBRARIES: Dict[str, dict] = {
     "attention": {"kind": "hip", "sources": ["kernels/attention.hip"], "headers": ["kernels/common.h"]},
     "attention_decode": {"kind": "hip", "sources": ["kernels/attention_decode.hip"], "headers": ["kernels/common.h"]},
     "attention_prefill": {"kind": "hip", "sources": ["kernels/attention_prefill.hip"], "headers": ["kernels/common.h"]},
-    "sampling": {"kind": "hip", "sources": ["kernels/sampling.hip"], "headers": ["kernels/common.h"]},
+    "sampling": {"kind": "hip", "sources": ["kernels/sampling.hip"],
+                 "headers": ["kernels/common.h", "kernels/noalloc.h"]},
     "peaks": {"kind": "hip", "sources": ["kernels/peaks.hip"], "headers": ["kernels/common.h"]},
 }
 

@@ -1,5 +1,8 @@
 // Token choice on the device: greedy argmax and temperature sampling, fp32 logits.
+#include <mutex>
+
 #include "common.h"
+#include "noalloc.h"
 
 #define SAMPLE_THREADS 256
 
@@ -236,6 +239,53 @@ int mllm_argmax(const float* logits, int ld, int n, int V, int* out, float* part
         MLLM_LAUNCH_CHECK();
     }
     return 0;
+}
+
+}  // extern "C"
+
+// Scratch of the entry point that allocates nothing: the first stage's values, then its indices.
+// In host code this name is only a handle for hipGetSymbolAddress; the array's address on a device is
+// looked up once per device and kept.
+static __device__ __align__(256) unsigned char scratch[MLLM_ARGMAX_NOALLOC_MAX_PAIRS * (sizeof(float) + sizeof(int))];
+
+#define NOALLOC_MAX_DEVICES 64
+static void* g_scratch_ptr[NOALLOC_MAX_DEVICES];     // per device; null until looked up
+static std::mutex g_scratch_mutex;
+
+// The address of `scratch` on the current device (looked up at the first call on that device).
+static hipError_t scratch_on_current_device(void** ptr) {
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return e;
+    if (dev < 0 || dev >= NOALLOC_MAX_DEVICES) return hipErrorInvalidDevice;
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (g_scratch_ptr[dev] == nullptr) {
+        void* p = nullptr;
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess) return e;
+        if (p == nullptr) return hipErrorInvalidSymbol;
+        g_scratch_ptr[dev] = p;
+    }
+    *ptr = g_scratch_ptr[dev];
+    return hipSuccess;
+}
+
+extern "C" {
+
+int mllm_argmax_noalloc_max_pairs(void) { return MLLM_ARGMAX_NOALLOC_MAX_PAIRS; }
+
+int mllm_argmax_noalloc(const float* logits, int ld, int n, int V, int* out, hipStream_t stream) {
+    if (n <= 0) return 0;
+    if (V <= 0) return -1;
+    const int n_chunks = (V + ARGMAX_CHUNK - 1) / ARGMAX_CHUNK;
+    if (static_cast<long long>(n) * n_chunks > MLLM_ARGMAX_NOALLOC_MAX_PAIRS) return -3;
+    void* base = nullptr;
+    const hipError_t e = scratch_on_current_device(&base);
+    if (e != hipSuccess) return static_cast<int>(e);
+    float* part_val = static_cast<float*>(base);
+    int* part_idx = reinterpret_cast<int*>(static_cast<unsigned char*>(base) +
+                                           MLLM_ARGMAX_NOALLOC_MAX_PAIRS * sizeof(float));
+    return mllm_argmax(logits, ld, n, V, out, part_val, part_idx, stream);
 }
 
 int mllm_sample(const float* logits, int ld, int n, int V, const float* temperature, const float* u, int* out,
