@@ -6,9 +6,13 @@
 // the LPK partial dot products are summed with DPP shuffles, and every lane keeps the
 // running maximum, sum and its slice of the output for the keys of its lane group
 // (recurrence of /root/reference/src/kernels/prefill/flashattention.cu:129-178, in base 2).
-// Groups, wavefronts and splits are merged with the same (m, l, o) rule; the last
-// workgroup to finish a (token, head) pair merges the splits, found through an atomic
-// counter (no workgroup ever waits for another).
+// Groups, wavefronts and splits are merged with the same (m, l, o) rule. The splits of a
+// (token, head) pair are merged either by the last workgroup to finish the pair, found through
+// an atomic counter (no workgroup ever waits for another), or, with `partial_out`, not here at
+// all: every workgroup leaves its state (maximum in base 2, sum, unnormalised output, fp32) in the
+// workspace and the kernel that reads the attention output next merges them while it loads its
+// operand (the few-row product of the output projection does), which costs no fence and no second
+// pass here.
 //
 // It stands where the reference has its three-pass decode kernel
 // (/root/reference/src/kernels/decode/paged_attention.cu:58-120); no 1e-6 is added to
@@ -69,7 +73,7 @@ decode_attention_kernel(// the first 16 dwords arrive in registers with the wave
                         float scale_log2e, T* __restrict__ out, int out_stride,
                         float* __restrict__ ws_o, float* __restrict__ ws_ml, int* __restrict__ counters,
                         T* __restrict__ k_pages_w, T* __restrict__ v_pages_w, int k_col, int v_col,
-                        const int* __restrict__ slots) {
+                        const int* __restrict__ slots, int partial_out) {
     constexpr int EPL = Vec16<T>::N;        // elements per lane
     constexpr int DH = LPK * EPL;           // head size
     constexpr int KPW = MLLM_WAVE / LPK;    // keys per wavefront and load instruction
@@ -237,6 +241,16 @@ decode_attention_kernel(// the first 16 dwords arrive in registers with the wave
     };
     block_merge();
     T* op = out + static_cast<size_t>(t) * out_stride + h * DH + c * EPL;
+    if (partial_out) {
+        // the split's state as it is; whoever reads the workspace merges
+        const size_t slot = static_cast<size_t>(pair) * nsplit + split;
+        if (wave == 0 && g == 0) {
+#pragma unroll
+            for (int e = 0; e < EPL; ++e) ws_o[slot * DH + c * EPL + e] = o[e];
+            if (c == 0) { ws_ml[slot * 2] = m; ws_ml[slot * 2 + 1] = l; }
+        }
+        return;
+    }
     if (nsplit == 1) {
         if (wave == 0 && g == 0) {
             const float inv = 1.0f / l;
@@ -297,10 +311,10 @@ static int launch_decode(int lpk, dim3 grid, int waves, hipStream_t stream, cons
                          int max_blocks, const int* token_seq, const int* positions, int n_heads,
                          int n_kv_heads, int page_size, float scale_log2e, int window, int nsplit, T* out,
                          int out_stride, float* ws_o, float* ws_ml, int* counters, T* k_pages_w, T* v_pages_w,
-                         int k_col, int v_col, const int* slots) {
+                         int k_col, int v_col, const int* slots, int partial_out) {
 #define DEC_ARGS token_seq, positions, block_tables, max_blocks, n_heads, n_kv_heads, page_size, window,  \
             nsplit, q, q_stride, q_col, k_pages, v_pages, kv_dim, scale_log2e, out, out_stride,        \
-            ws_o, ws_ml, counters, k_pages_w, v_pages_w, k_col, v_col, slots
+            ws_o, ws_ml, counters, k_pages_w, v_pages_w, k_col, v_col, slots, partial_out
 #define DEC_CASE(L)                                                                                    \
     case L:                                                                                            \
         decode_attention_kernel<T, L, 8><<<grid, waves * MLLM_WAVE, 0, stream>>>(DEC_ARGS);             \
@@ -313,7 +327,50 @@ static int launch_decode(int lpk, dim3 grid, int waves, hipStream_t stream, cons
 #undef DEC_ARGS
 }
 
+// Merges the splits' states that `partial_out` left in the workspace into the attention output:
+// one thread per 4 elements. For readers of the output that do not merge while they load.
+template <typename T>
+__global__ void merge_splits_kernel(const float* __restrict__ ws_o, const float* __restrict__ ws_ml, int nsplit,
+                                    int head_dim, int n_heads, T* __restrict__ out, int out_stride, int total4) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= total4) return;
+    const int per_pair = head_dim / 4;
+    const int pair = i / per_pair, e = (i % per_pair) * 4;
+    float mx = -INFINITY;
+    for (int s = 0; s < nsplit; ++s) mx = fmaxf(mx, ws_ml[(static_cast<size_t>(pair) * nsplit + s) * 2]);
+    float l = 0.f, o[4] = {0.f, 0.f, 0.f, 0.f};
+    for (int s = 0; s < nsplit; ++s) {
+        const size_t slot = static_cast<size_t>(pair) * nsplit + s;
+        const float w = exp2_for<T>(ws_ml[slot * 2] - mx);
+        l += w * ws_ml[slot * 2 + 1];
+        const float4 v = *reinterpret_cast<const float4*>(ws_o + slot * head_dim + e);
+        o[0] += w * v.x; o[1] += w * v.y; o[2] += w * v.z; o[3] += w * v.w;
+    }
+    const float inv = 1.0f / l;
+    T* dst = out + static_cast<size_t>(pair / n_heads) * out_stride + (pair % n_heads) * head_dim + e;
+#pragma unroll
+    for (int k = 0; k < 4; ++k) dst[k] = from_float<T>(o[k] * inv);
+}
+
 extern "C" {
+
+// out[t, h * head_dim + e] from the states of `partial_out` (head_dim % 4 == 0).
+int mllm_merge_attention_splits(const float* ws, int n_q, int n_heads, int head_dim, int nsplit, void* out,
+                                int out_stride, int dtype, hipStream_t stream) {
+    if (n_q <= 0) return 0;
+    if (head_dim % 4 != 0 || nsplit < 1) return -1;
+    const float* ws_o = ws;
+    const float* ws_ml = ws + static_cast<size_t>(n_q) * n_heads * nsplit * head_dim;
+    const int total4 = n_q * n_heads * (head_dim / 4);
+    if (dtype == MLLM_F32)
+        merge_splits_kernel<float><<<(total4 + 255) / 256, 256, 0, stream>>>(ws_o, ws_ml, nsplit, head_dim, n_heads,
+                                                                             static_cast<float*>(out), out_stride, total4);
+    else
+        merge_splits_kernel<bf16_t><<<(total4 + 255) / 256, 256, 0, stream>>>(ws_o, ws_ml, nsplit, head_dim, n_heads,
+                                                                              static_cast<bf16_t*>(out), out_stride, total4);
+    MLLM_LAUNCH_CHECK();
+    return 0;
+}
 
 // Number of floats of workspace (partial outputs and their max/sum) for n_q tokens.
 long mllm_decode_attention_ws_floats(int n_q, int n_heads, int head_dim, int nsplit) {
@@ -325,12 +382,16 @@ long mllm_decode_attention_ws_floats(int n_q, int n_heads, int head_dim, int nsp
 // first launch (the kernel leaves them zero). With `slots` (n_q rows of the page pools, < 0: none) the
 // tokens' own keys/values are taken from columns k_col/v_col of q and written to the pages by this
 // kernel; without, they must be in the pages already.
+// partial_out != 0: nothing is written to `out`; the workspace holds, for pair = token * n_heads + head
+// and split s, the unnormalised output at ws[(pair * nsplit + s) * head_dim ..] and (maximum in base 2,
+// sum) at ws[n_q * n_heads * nsplit * head_dim + (pair * nsplit + s) * 2 ..]; a split without keys has
+// sum 0 and a large negative maximum.
 int mllm_decode_attention(const void* q, int q_stride, int q_col, const void* k_pages, const void* v_pages,
                           int kv_dim, const int* block_tables, int max_blocks, const int* token_seq,
                           const int* positions, int n_q, int n_heads, int n_kv_heads, int head_dim,
                           int page_size, float scale, int window, int nsplit, int waves, void* out,
                           int out_stride, float* ws, int* counters, int k_col, int v_col, const int* slots,
-                          int dtype, hipStream_t stream) {
+                          int partial_out, int dtype, hipStream_t stream) {
     if (n_q <= 0) return 0;
     const int esz = dtype == MLLM_F32 ? 4 : 2;
     const int lpk = head_dim * esz / 16;
@@ -346,12 +407,12 @@ int mllm_decode_attention(const void* q, int q_stride, int q_col, const void* k_
         rc = launch_decode<float>(lpk, grid, waves, stream, (const float*)q, q_stride, q_col, (const float*)k_pages,
                                   (const float*)v_pages, kv_dim, block_tables, max_blocks, token_seq, positions,
                                   n_heads, n_kv_heads, page_size, sl2, window, nsplit, (float*)out, out_stride,
-                                  ws_o, ws_ml, counters, (float*)k_pages, (float*)v_pages, k_col, v_col, slots);
+                                  ws_o, ws_ml, counters, (float*)k_pages, (float*)v_pages, k_col, v_col, slots, partial_out);
     else
         rc = launch_decode<bf16_t>(lpk, grid, waves, stream, (const bf16_t*)q, q_stride, q_col, (const bf16_t*)k_pages,
                                    (const bf16_t*)v_pages, kv_dim, block_tables, max_blocks, token_seq, positions,
                                    n_heads, n_kv_heads, page_size, sl2, window, nsplit, (bf16_t*)out, out_stride,
-                                   ws_o, ws_ml, counters, (bf16_t*)k_pages, (bf16_t*)v_pages, k_col, v_col, slots);
+                                   ws_o, ws_ml, counters, (bf16_t*)k_pages, (bf16_t*)v_pages, k_col, v_col, slots, partial_out);
     if (rc != 0) return rc;
     MLLM_LAUNCH_CHECK();
     return 0;

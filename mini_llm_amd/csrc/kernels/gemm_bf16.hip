@@ -385,13 +385,25 @@ static void launch_tiled(const bf16_t* a, int lda, const bf16_t* w, int ldw, con
 // from L2), are copied into LDS once per workgroup (A_STAGED: wide products), or are normalised
 // from the fp32 stream into LDS first (A_NORMED): LayerNorm
 // (/root/reference/src/kernels/layernorm.cu:32-49) fused into the product that follows it.
+// A_MERGED: A is the output of decode attention that split every (token, head) pair's keys over
+// several workgroups and left their states in a workspace (attention_decode.hip, partial_out): a lane
+// that would load 8 elements of a row loads those elements of every split's unnormalised output and
+// the splits' maxima and sums instead, and merges them in registers. The attention kernel then
+// needs no pass that waits for its last workgroup, and more workgroups stream the keys.
 // ---------------------------------------------------------------------------------------------
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 
-enum { A_GLOBAL = 0, A_NORMED = 1, A_STAGED = 2 };
+enum { A_GLOBAL = 0, A_NORMED = 1, A_STAGED = 2, A_MERGED = 3 };
+#define MERGE_MAX_SPLITS 4      // splits of a pair that the merging load takes (registers: 10 per split and load)
+
+// The states of up to MERGE_MAX_SPLITS splits for 8 consecutive elements of one head of one token.
+struct SplitStates {
+    float2 ml[MERGE_MAX_SPLITS];          // maximum (base 2), sum
+    float4 o[MERGE_MAX_SPLITS][2];        // 8 elements of the unnormalised output
+};
 
 template <int MT, int ASRC, bool SPLIT_K, int U, bool A_TWO = true, int NT = 1>
-__global__ void __launch_bounds__(ASRC == A_NORMED ? 512 : (ASRC == A_GLOBAL ? 768 : 1024))
+__global__ void __launch_bounds__(ASRC == A_NORMED ? 512 : (ASRC == A_GLOBAL || ASRC == A_MERGED ? 768 : 1024))
 gemm_bf16_skinny(// the first 16 dwords arrive in registers with the wavefront: what the first loads need
                  const bf16_t* __restrict__ W, int ldw, int N, int K, int M, int col_blocks, int row_blocks,
                  int cols_per_wg, int k_parts, const void* __restrict__ Ain, int lda, int mode,
@@ -399,7 +411,11 @@ gemm_bf16_skinny(// the first 16 dwords arrive in registers with the wavefront: 
                  // the rest is loaded by the kernel and needed later
                  void* __restrict__ C, int ldc, const float* __restrict__ gamma, const float* __restrict__ beta,
                  float eps, const int* __restrict__ rows, float* __restrict__ part_sums,
-                 int* __restrict__ part_counters) {
+                 int* __restrict__ part_counters,
+                 // A_MERGED: the attention splits' states (layout: attention_decode.hip), their number,
+                 // heads per token and head size (K = heads x head size)
+                 const float* __restrict__ split_o = nullptr, const float* __restrict__ split_ml = nullptr,
+                 int n_splits = 1, int a_heads = 1, int a_head_dim = 8) {
     // NT > 1 (SPLIT_K, MT == 1): the workgroup owns cols_per_wg <= 16 NT columns, NT tiles that share
     // the rows of A, the last one possibly narrower: for products with more than 256 tiles, whose
     // columns are dealt out evenly to 256 workgroups (one per compute unit; a kernel of this size
@@ -409,7 +425,8 @@ gemm_bf16_skinny(// the first 16 dwords arrive in registers with the wavefront: 
     extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
     __shared__ int sm_last;
     constexpr bool LN_FUSED = ASRC == A_NORMED;
-    constexpr bool IN_LDS = ASRC != A_GLOBAL;
+    constexpr bool IN_LDS = ASRC == A_NORMED || ASRC == A_STAGED;
+    constexpr bool A_REGS = !IN_LDS;      // the rows of A travel through registers and the wavefront's LDS region
     // The wavefront's index as a scalar: what depends on it alone (its k blocks, whether it has a
     // whole chunk, whether it owns outputs) then branches for real. Derived from threadIdx it would
     // count as divergent, both sides of every such condition would run one after the other under
@@ -433,8 +450,8 @@ gemm_bf16_skinny(// the first 16 dwords arrive in registers with the wavefront: 
     const int k_stride = SPLIT_K ? nw * k_parts * 64 : 64;         // distance between its k blocks
     const size_t red_bytes = SPLIT_K ? static_cast<size_t>(nw) * T * 256 * sizeof(float) : 0;
     // per wavefront: SB k blocks at a time change lanes through LDS, each NT weight tiles (+ the A block)
-    constexpr int SB = (ASRC == A_STAGED || (ASRC == A_GLOBAL && NT > 1) || U < 4) ? 1 : 2;
-    constexpr int STAGE_BYTES = SB * (NT * 2048 + (ASRC == A_GLOBAL ? 2048 : 0));
+    constexpr int SB = (ASRC == A_STAGED || (A_REGS && NT > 1) || U < 4) ? 1 : 2;
+    constexpr int STAGE_BYTES = SB * (NT * 2048 + (A_REGS ? 2048 : 0));
     float* red = reinterpret_cast<float*>(smem_raw);                       // [nw][T][256]
     bf16x8* stage_w = reinterpret_cast<bf16x8*>(smem_raw + red_bytes + static_cast<size_t>(wave) * STAGE_BYTES);
     bf16x8* stage_a = stage_w + SB * NT * 128;                             // (A_GLOBAL only)
@@ -501,17 +518,69 @@ gemm_bf16_skinny(// the first 16 dwords arrive in registers with the wavefront: 
     // A_GLOBAL: the rows of A travel like the weights (rows beyond M: the last one, never stored);
     // a workgroup with at most 8 rows needs one load per k block
     const bf16_t* arow[2] = {A, A};
+    int arow_idx[2] = {0, 0};
     // (A_TWO false: the launcher knows that M <= 8, and the chunks keep half the registers for A)
     const bool a_two = A_TWO && M - m_base > 8;
-    if (ASRC == A_GLOBAL) {
+    if (A_REGS) {
 #pragma unroll
-        for (int j = 0; j < 2; ++j) arow[j] = A + static_cast<size_t>(min(m_base + lr + 8 * j, M - 1)) * lda;
+        for (int j = 0; j < 2; ++j) {
+            arow_idx[j] = min(m_base + lr + 8 * j, M - 1);
+            arow[j] = A + static_cast<size_t>(arow_idx[j]) * lda;
+        }
     }
+    // A_MERGED: requests the splits' states for the 8 elements from k on of row `row` (all loads together;
+    // splits beyond n_splits take the last one again and get no weight), and merges them later
+    auto fetch_splits = [&](SplitStates& st, int row, int k) {
+        const int h = k / a_head_dim, e = k - h * a_head_dim;
+        const size_t pair = static_cast<size_t>(row) * a_heads + h;
+#pragma unroll
+        for (int sidx = 0; sidx < MERGE_MAX_SPLITS; ++sidx) {
+            const size_t slot = pair * n_splits + min(sidx, n_splits - 1);
+            st.ml[sidx] = *reinterpret_cast<const float2*>(split_ml + slot * 2);
+            const float4* src = reinterpret_cast<const float4*>(split_o + slot * a_head_dim + e);
+            st.o[sidx][0] = src[0];
+            st.o[sidx][1] = src[1];
+        }
+    };
+    auto merge_splits = [&](const SplitStates& st) -> bf16x8 {
+        float mx = st.ml[0].x;
+#pragma unroll
+        for (int sidx = 1; sidx < MERGE_MAX_SPLITS; ++sidx) mx = fmaxf(mx, sidx < n_splits ? st.ml[sidx].x : mx);
+        float l = 0.f, o[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int sidx = 0; sidx < MERGE_MAX_SPLITS; ++sidx) {
+            const float w = sidx < n_splits ? fast_exp2(st.ml[sidx].x - mx) : 0.f;
+            l = fmaf(w, st.ml[sidx].y, l);
+            o[0] = fmaf(w, st.o[sidx][0].x, o[0]); o[1] = fmaf(w, st.o[sidx][0].y, o[1]);
+            o[2] = fmaf(w, st.o[sidx][0].z, o[2]); o[3] = fmaf(w, st.o[sidx][0].w, o[3]);
+            o[4] = fmaf(w, st.o[sidx][1].x, o[4]); o[5] = fmaf(w, st.o[sidx][1].y, o[5]);
+            o[6] = fmaf(w, st.o[sidx][1].z, o[6]); o[7] = fmaf(w, st.o[sidx][1].w, o[7]);
+        }
+        const float inv = 1.0f / l;
+        union { uint32_t w[4]; bf16x8 v; } pk;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) pk.w[i] = pack_bf16x2(o[2 * i] * inv, o[2 * i + 1] * inv);
+        return pk.v;
+    };
     const int n_blocks = k_first < K ? (K - k_first + k_stride - 1) / k_stride : 0;   // of this wavefront
     const int n_chunks = n_blocks / H;
     struct Chunk {
         bf16x8 b[NT][U];
-        bf16x8 a[ASRC == A_GLOBAL ? (A_TWO ? U : U / 2) : 1];
+        bf16x8 a[A_REGS ? (A_TWO ? U : U / 2) : 1];
+    };
+    // (A_MERGED) the states requested for a chunk's blocks, rows 0..7 and 8..15
+    SplitStates pending[ASRC == A_MERGED ? U / 2 : 1][ASRC == A_MERGED && A_TWO ? 2 : 1];
+    auto fetch_block_splits = [&](int h, int k0) {
+        if (ASRC != A_MERGED) return;
+#pragma unroll
+        for (int j = 0; j < (A_TWO ? 2 : 1); ++j)
+            if (j == 0 || a_two) fetch_splits(pending[h][j], arow_idx[j], min(k0 + 8 * piece[j], K - 8));
+    };
+    auto merge_block_splits = [&](Chunk& c, int h) {
+        if (ASRC != A_MERGED) return;
+#pragma unroll
+        for (int j = 0; j < (A_TWO ? 2 : 1); ++j)
+            if (j == 0 || a_two) c.a[A_TWO ? 2 * h + j : h] = merge_splits(pending[h][j]);
     };
     auto load_steps = [&](Chunk& c, int u0, int k0) {      // the k block at k0 (rows 0..7, rows 8..15) into slots u0, u0+1
 #pragma unroll
@@ -529,6 +598,7 @@ gemm_bf16_skinny(// the first 16 dwords arrive in registers with the wavefront: 
                 c.b[t][u0 + j] = STREAM ? __builtin_nontemporal_load(src) : *src;
             }
             if (ASRC == A_GLOBAL && (j == 0 || a_two)) c.a[A_TWO ? u0 + j : u0 / 2] = *reinterpret_cast<const bf16x8*>(arow[j] + k);
+            // (A_MERGED: the splits' states were requested before the weights and are merged after them)
         }
     };
     auto wave_lds_order = [&]() {       // orders the wavefront's own LDS writes and reads (no instruction)
@@ -543,7 +613,7 @@ gemm_bf16_skinny(// the first 16 dwords arrive in registers with the wavefront: 
         static_assert(CNT <= SB, "staging room");
 #pragma unroll
         for (int i = 0; i < CNT; ++i) {
-            if (ASRC == A_GLOBAL) {
+            if (A_REGS) {
                 stage_a[i * 128 + lane] = c.a[A_TWO ? u0 + 2 * i : (u0 + 2 * i) / 2];
                 if (a_two) stage_a[i * 128 + 64 + lane] = c.a[A_TWO ? u0 + 2 * i + 1 : 0];
             }
@@ -560,7 +630,7 @@ gemm_bf16_skinny(// the first 16 dwords arrive in registers with the wavefront: 
 #pragma unroll
             for (int half = 0; half < 2; ++half) {
                 const int slot = row16 * 8 + ((2 * kq + half) ^ rd_swz);
-                if (ASRC == A_GLOBAL) af[i][half] = stage_a[i * 128 + slot];
+                if (A_REGS) af[i][half] = stage_a[i * 128 + slot];
 #pragma unroll
                 for (int t = 0; t < NT; ++t) bf[i][t][half] = stage_w[(i * NT + t) * 128 + slot];
             }
@@ -596,11 +666,20 @@ gemm_bf16_skinny(// the first 16 dwords arrive in registers with the wavefront: 
         }
     };
     auto load_chunk = [&](Chunk& c, int chunk) {            // chunk index within this wavefront's blocks
+        if (ASRC == A_MERGED) {
+#pragma unroll
+            for (int h = 0; h < H; ++h) fetch_block_splits(h, k_first + (chunk * H + h) * k_stride);
+            __builtin_amdgcn_sched_barrier(0);
+        }
 #pragma unroll
         for (int h = 0; h < H; ++h) load_steps(c, 2 * h, k_first + (chunk * H + h) * k_stride);
         // the instruction scheduler must not sink these loads towards their uses: they are issued
         // here to be in flight together
         __builtin_amdgcn_sched_barrier(0);
+        if (ASRC == A_MERGED) {
+#pragma unroll
+            for (int h = 0; h < H; ++h) merge_block_splits(c, h);
+        }
     };
     auto mma_chunk = [&](const Chunk& c, int chunk) { mma_some(c, H, k_first + chunk * H * k_stride); };
     // rows of the fp32 stream that this wavefront normalises (read before the weights are
@@ -616,10 +695,21 @@ gemm_bf16_skinny(// the first 16 dwords arrive in registers with the wavefront: 
     Chunk c0, c1;
     auto load_left = [&]() {                                // the blocks after the last whole chunk
         const int first = n_chunks * H, left = n_blocks - first;
+        if (ASRC == A_MERGED) {
+#pragma unroll
+            for (int h = 0; h < H - 1; ++h)
+                if (h < left) fetch_block_splits(h, k_first + (first + h) * k_stride);
+            __builtin_amdgcn_sched_barrier(0);
+        }
 #pragma unroll
         for (int h = 0; h < H - 1; ++h)
             if (h < left) load_steps(c1, 2 * h, k_first + (first + h) * k_stride);
         __builtin_amdgcn_sched_barrier(0);
+        if (ASRC == A_MERGED) {
+#pragma unroll
+            for (int h = 0; h < H - 1; ++h)
+                if (h < left) merge_block_splits(c1, h);
+        }
     };
     // The first loads are one whole chunk for every wavefront, without a condition: a wavefront
     // with fewer blocks than a chunk takes its last block again (its own line, requested a moment
@@ -628,9 +718,18 @@ gemm_bf16_skinny(// the first 16 dwords arrive in registers with the wavefront: 
     // wait for the weights.)
     const int last_block = n_blocks > 0 ? n_blocks - 1 : 0;
     auto first_loads = [&]() {
+        if (ASRC == A_MERGED) {
+#pragma unroll
+            for (int h = 0; h < H; ++h) fetch_block_splits(h, k_first + min(h, last_block) * k_stride);
+            __builtin_amdgcn_sched_barrier(0);
+        }
 #pragma unroll
         for (int h = 0; h < H; ++h) load_steps(c0, 2 * h, k_first + min(h, last_block) * k_stride);
         __builtin_amdgcn_sched_barrier(0);
+        if (ASRC == A_MERGED) {
+#pragma unroll
+            for (int h = 0; h < H; ++h) merge_block_splits(c0, h);
+        }
     };
     // The fused norm's operands are requested before the weights: loads return in the order of
     // their requests, so the norm (whose rows come from L2) can be computed while the weights are
@@ -840,10 +939,18 @@ constexpr int SPLIT_MAX_PARTS = 8;
 constexpr int SPLIT_MIN_K_BLOCKS = 12;    // k blocks of 64 elements that every part keeps at least
 constexpr int SPLIT_FROM_K_BLOCKS = 80;   // shorter K: the fences cost more than the parallelism gains (measured)
 
-template <bool LN_FUSED>
+struct MergedA {        // A_MERGED: where the attention splits' states lie
+    const float* split_o = nullptr;
+    const float* split_ml = nullptr;
+    int n_splits = 1, heads = 1, head_dim = 8;
+};
+
+template <bool LN_FUSED, bool MERGED = false>
 static int launch_skinny(const void* A, int lda, const bf16_t* W, int ldw, const float* bias, void* C, int ldc,
                          int M, int N, int K, int mode, const float* gamma, const float* beta, float eps,
-                         const int* rows, hipStream_t stream, void* workspace = nullptr, size_t workspace_bytes = 0) {
+                         const int* rows, hipStream_t stream, void* workspace = nullptr, size_t workspace_bytes = 0,
+                         MergedA merged = MergedA{}) {
+    static_assert(!(LN_FUSED && MERGED), "one source of A");
     const int tiles = (N + 15) / 16;
     const bool split_k = tiles < 1024;
     // Narrow products: 16 rows per workgroup and one workgroup per 16 rows (more workgroups, each
@@ -872,7 +979,10 @@ static int launch_skinny(const void* A, int lda, const bf16_t* W, int ldw, const
     // SPLIT_MIN_K_BLOCKS k blocks. Needs the workspace: SPLIT_COUNTERS counters, then 256 floats
     // per tile and part.
     int k_parts = 1;
-    if (split_k && !LN_FUSED && workspace != nullptr && k_blocks >= SPLIT_FROM_K_BLOCKS) {
+    if (MERGED && (!split_k || M > 16 || merged.n_splits < 1 || merged.n_splits > MERGE_MAX_SPLITS ||
+                   merged.head_dim % 8 != 0 || merged.heads * merged.head_dim != K))
+        return -2;
+    if (split_k && !LN_FUSED && !MERGED && workspace != nullptr && k_blocks >= SPLIT_FROM_K_BLOCKS) {
         const int wgs = tiles * row_blocks;
         k_parts = std::min(std::min(256 / std::max(wgs, 1), k_blocks / SPLIT_MIN_K_BLOCKS), SPLIT_MAX_PARTS);
         if (k_parts < 2 || wgs > SPLIT_COUNTERS ||
@@ -900,13 +1010,13 @@ static int launch_skinny(const void* A, int lda, const bf16_t* W, int ldw, const
     // More than 256 tiles (and one row block): two tiles per workgroup, the columns dealt out evenly
     // to 256 workgroups.
     int cols_per_wg = 16;
-    const bool two_tiles = split_k && row_blocks == 1 && k_parts == 1 && tiles > 256 && tiles <= 512 &&
+    const bool two_tiles = !MERGED && split_k && row_blocks == 1 && k_parts == 1 && tiles > 256 && tiles <= 512 &&
                            (LN_FUSED || M <= 8);
     if (two_tiles) cols_per_wg = (N + 255) / 256;
     // Fewer than 256 tiles, one row block and a long K (the second product of the feed-forward):
     // narrower tiles, down to 4 columns, so that more compute units share the weights. (Short K, or
     // the fused norm: the kernel's time is latency, not bytes, and nothing is gained; measured.)
-    if (split_k && !LN_FUSED && row_blocks == 1 && k_parts == 1 && tiles < 256 && k_blocks >= 48)
+    if (split_k && !LN_FUSED && !MERGED && row_blocks == 1 && k_parts == 1 && tiles < 256 && k_blocks >= 48)
         cols_per_wg = std::min(16, std::max((N + 255) / 256, 4));
     const int col_blocks = split_k ? (N + cols_per_wg - 1) / cols_per_wg : (tiles + nw - 1) / nw;
     const dim3 grid((col_blocks + N_XCD - 1) / N_XCD * N_XCD * row_blocks, k_parts), block(nw * 64);
@@ -923,7 +1033,8 @@ static int launch_skinny(const void* A, int lda, const bf16_t* W, int ldw, const
                                            static_cast<int>(staged_bytes));                            \
         if (e != hipSuccess) return static_cast<int>(e);                                               \
         kernel<<<grid, block, staged_bytes, stream>>>(W, ldw, N, K, M, col_blocks, row_blocks, 16, 1, A, lda, mode, \
-                                                      bias, C, ldc, gamma, beta, eps, rows, nullptr, nullptr); \
+                                                      bias, C, ldc, gamma, beta, eps, rows, nullptr, nullptr, \
+                                                      nullptr, nullptr, 1, 1, 8);                      \
         break;                                                                                         \
     }
         switch (mt) {
@@ -940,7 +1051,7 @@ static int launch_skinny(const void* A, int lda, const bf16_t* W, int ldw, const
             return -2;
     }
     if (smem > MAX_DYNAMIC_LDS) return -2;
-    constexpr int ASRC = LN_FUSED ? A_NORMED : A_GLOBAL;
+    constexpr int ASRC = LN_FUSED ? A_NORMED : (MERGED ? A_MERGED : A_GLOBAL);
 #define SKINNY_LAUNCH(SPLIT, UV, A2, NTV)                                                              \
     do {                                                                                               \
         auto kernel = gemm_bf16_skinny<1, ASRC, SPLIT, UV, A2, NTV>;                                   \
@@ -953,7 +1064,8 @@ static int launch_skinny(const void* A, int lda, const bf16_t* W, int ldw, const
         }                                                                                              \
         kernel<<<grid, block, smem, stream>>>(W, ldw, N, K, M, col_blocks, row_blocks, cols_per_wg, k_parts, A, lda, \
                                               mode, bias, C, ldc, gamma, beta, eps, rows, part_sums,      \
-                                              part_counters);                                          \
+                                              part_counters, merged.split_o, merged.split_ml, merged.n_splits, \
+                                              merged.heads, merged.head_dim);                          \
     } while (0)
     if (split_k) {
         // a chunk holds all k blocks of a wavefront when they are at most 3 (4 without the fused
@@ -970,6 +1082,23 @@ static int launch_skinny(const void* A, int lda, const bf16_t* W, int ldw, const
                 case 1: SKINNY_LAUNCH(true, 2, false, 1); break;
                 case 2: SKINNY_LAUNCH(true, 4, false, 1); break;
                 default: SKINNY_LAUNCH(true, 6, false, 1); break;
+            }
+        } else if (MERGED) {
+            // the splits' states of a whole chunk are in flight together: one chunk holds all of a
+            // wavefront's k blocks, at most 3
+            if (per_wave > 3) return -2;
+            if (M <= 8) {
+                switch (per_wave) {
+                    case 1: SKINNY_LAUNCH(true, 2, false, 1); break;
+                    case 2: SKINNY_LAUNCH(true, 4, false, 1); break;
+                    default: SKINNY_LAUNCH(true, 6, false, 1); break;
+                }
+            } else {
+                switch (per_wave) {
+                    case 1: SKINNY_LAUNCH(true, 2, true, 1); break;
+                    case 2: SKINNY_LAUNCH(true, 4, true, 1); break;
+                    default: SKINNY_LAUNCH(true, 6, true, 1); break;
+                }
             }
         } else if (M <= 8) {
             switch (std::min(per_wave, 4)) {
@@ -1091,6 +1220,28 @@ int mllm_gemm_bf16_kv(const void* A, int lda, const void* W, int ldw, const floa
         return -1;
     KvScatter kv{slots, static_cast<bf16_t*>(k_pages), static_cast<bf16_t*>(v_pages), q_cols, kv_dim};
     return gemm_bf16_dispatch(A, lda, W, ldw, bias, C, ldc, M, N, K, EPI_STORE, stream, kv);
+}
+
+// The product whose A is the output of split decode attention, merged from the splits' states while it
+// is loaded: C = epilogue(merge(states) W^T + bias) with A[m, h * head_dim + e] = sum_s w_s o_s[e] /
+// sum_s w_s l_s, w_s = 2^(m_s - max m). M <= 16 tokens, n_splits <= 4, head_dim % 8 == 0, K = n_heads *
+// head_dim <= 2304 or so. Returns 0, a HIP error code, -1 for misaligned operands, or -2 when the sizes
+// are not ones this kernel takes (the caller then merges with mllm_merge_attention_splits and runs the
+// ordinary product).
+int mllm_gemm_bf16_merged(const float* split_o, const float* split_ml, int n_splits, int n_heads, int head_dim,
+                          const void* W, int ldw, const float* bias, void* C, int ldc, int M, int N, int mode,
+                          hipStream_t stream) {
+    const int K = n_heads * head_dim;
+    if (M <= 0 || N <= 0) return 0;
+    if (K % 8 != 0 || ldw % 8 != 0 || (reinterpret_cast<uintptr_t>(W) & 15) ||
+        (reinterpret_cast<uintptr_t>(split_o) & 15) || (reinterpret_cast<uintptr_t>(split_ml) & 7))
+        return -1;
+    MergedA merged{split_o, split_ml, n_splits, n_heads, head_dim};
+    int rc = launch_skinny<false, true>(nullptr, K, static_cast<const bf16_t*>(W), ldw, bias, C, ldc, M, N, K, mode,
+                                        nullptr, nullptr, 0.f, nullptr, stream, nullptr, 0, merged);
+    if (rc != 0) return rc;
+    MLLM_LAUNCH_CHECK();
+    return 0;
 }
 
 // LayerNorm of the fp32 rows x[M,K] (row m taken from x[rows[m]] when `rows` is given) fused into the

@@ -52,6 +52,8 @@ class StepContext:
     slots: List[torch.Tensor]          # per group [T] row of the page pool each token writes
     max_q_len: int
     max_ctx_len: int
+    n_single: int = 0             # the first n_single sequences bring one token each (decoded tokens stand
+                                  #     first in a scheduler's mixed step); kernels may treat them apart
     # host copies, for parts that plan on the host
     h_cu_q: np.ndarray = None
     h_starts: np.ndarray = None
@@ -169,7 +171,7 @@ class ModelRunner:
         return seg
 
     def _context(self, dev: torch.Tensor, offs, T, B, n_logits, max_blocks, max_q_len, max_ctx_len,
-                 seg=None, request_ids=()) -> StepContext:
+                 seg=None, request_ids=(), n_single=0) -> StepContext:
         d = [dev[offs[i]:offs[i + 1]] for i in range(len(offs) - 1)]
         G = len(max_blocks)
         return StepContext(
@@ -178,7 +180,7 @@ class ModelRunner:
             state_slots=d[6], logit_rows=d[7][:n_logits],
             block_tables=[d[8 + 2 * g].view(B, max_blocks[g]) for g in range(G)],
             slots=[d[9 + 2 * g] for g in range(G)],
-            max_q_len=max_q_len, max_ctx_len=max_ctx_len,
+            max_q_len=max_q_len, max_ctx_len=max_ctx_len, n_single=n_single,
             h_cu_q=None if seg is None else seg[3].copy(),
             h_starts=None if seg is None else seg[5].copy(),
             h_state_slots=None if seg is None else seg[6].copy(),
@@ -230,8 +232,10 @@ class ModelRunner:
         if tok.min() < 0 or tok.max() >= vocab:
             raise StepError(f"token ids must lie in [0, {vocab})")
         dev = self._staging.upload(buf, offs[-1])
+        many = np.flatnonzero(n_tok != 1)
+        n_single = int(many[0]) if many.size else B
         return self._context(dev, offs, T, B, n_logits, max_blocks, int(n_tok.max()), int(ctx.max()), seg,
-                             ids.tolist())
+                             ids.tolist(), n_single)
 
     def step(self, entries: Sequence[StepEntry], manage_cache: bool = True) -> Optional[torch.Tensor]:
         """Runs one batch. With ``manage_cache`` the runner registers new requests, takes
@@ -392,7 +396,7 @@ class DecodeGraph:
         self.src_rows = self.dev_ints[self.n_ctx_ints:self.n_ctx_ints + B]
         self.d_float = self.dev_ints[self.n_ctx_ints + B:].view(torch.float32).view(2, B)
         self.ctx = runner._context(self.dev_ints, self.offs, B, B, B, self.max_blocks, 1,
-                                   self.max_blocks[0] * runner.page_size if self.max_blocks else 1)
+                                   self.max_blocks[0] * runner.page_size if self.max_blocks else 1, n_single=B)
         self.out = runner._tok_out[:B]
         # two host buffers in turn: one may still be unread when the next step's copy is queued
         self.h_out = [torch.zeros(B, dtype=torch.int32, pin_memory=on_gpu) for _ in range(2)]

@@ -161,9 +161,48 @@ def _scatter_is_fused(dtype: torch.dtype, rows: int) -> bool:
     return dtype == torch.bfloat16 and rows > 64
 
 
+class AttentionSplits:
+    """The output of decode attention that has not been merged yet: every (token, head) pair's keys
+    were split over ``nsplit`` workgroups, whose states (running maximum, sum, unnormalised output)
+    lie in the attention scratch. ``linear`` takes it in place of a tensor and merges while it loads
+    (``tensor()`` merges into an ordinary activation). Valid until the next attention launch."""
+
+    def __init__(self, ws: torch.Tensor, n_tokens: int, n_heads: int, head_dim: int, nsplit: int, dtype):
+        self.ws, self.n_tokens, self.n_heads, self.head_dim, self.nsplit = ws, n_tokens, n_heads, head_dim, nsplit
+        self.dtype, self.device = dtype, ws.device
+        self.shape = (n_tokens, n_heads * head_dim)
+
+    def tensor(self, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+        if out is None:
+            out = torch.empty(self.shape, dtype=self.dtype, device=self.device)
+        lib = load_library("attention_decode")
+        _check(lib.mllm_merge_attention_splits(_p(self.ws), self.n_tokens, self.n_heads, self.head_dim, self.nsplit,
+                                               _p(out), out.stride(0), _DT[self.dtype], _stream()), "merge_splits")
+        return out
+
+
+MERGE_MAX_ROWS = 16        # tokens whose attention splits a product merges while loading (one row block)
+MERGE_MAX_SPLITS = 4       # and the most splits per (token, head) pair it takes
+
+
+def _linear_from_splits(a: AttentionSplits, w, bias, out, epilogue: str) -> Optional[torch.Tensor]:
+    """The product fed by unmerged attention splits, or None if its kernel does not take these sizes."""
+    M, K = a.shape
+    N = w.shape[0]
+    lib = load_library("gemm_bf16")
+    ml = a.ws[M * a.n_heads * a.nsplit * a.head_dim:]
+    rc = lib.mllm_gemm_bf16_merged(_p(a.ws), _p(ml), a.nsplit, a.n_heads, a.head_dim, _p(w), w.stride(0), _p(bias),
+                                   _p(out), out.stride(0), M, N, EPILOGUES[epilogue], _stream())
+    if rc == -2:
+        return None
+    _check(rc, "linear (merging attention splits)")
+    return out
+
+
 def linear(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], out: torch.Tensor,
            epilogue: str = "store", kv_scatter: Optional[tuple] = None) -> torch.Tensor:
-    """out = epilogue(a @ w.T + bias). a: [M,K], w: [N,K] (same dtype), bias: fp32 [N].
+    """out = epilogue(a @ w.T + bias). a: [M,K] (or the unmerged ``AttentionSplits`` of decode attention),
+    w: [N,K] (same dtype), bias: fp32 [N].
 
     epilogue: "store" | "gelu_tanh" | "gelu_erf" (out in a's dtype), "add_residual"
     (out fp32, accumulated in place), "store_f32" (out fp32).
@@ -173,8 +212,10 @@ def linear(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], out: 
     go to row slots[m] (>= 0) of the pages: in the product's epilogue where the kernel that runs
     for these sizes has one, otherwise by a copy kernel after it.
     """
-    _gpu(a, w, bias, out)
-    _rows2d(a, "a")
+    splits = a if isinstance(a, AttentionSplits) else None
+    _gpu(None if splits else a, w, bias, out)
+    if splits is None:
+        _rows2d(a, "a")
     _rows2d(w, "w")
     _rows2d(out, "out")
     M, K = a.shape
@@ -183,6 +224,14 @@ def linear(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], out: 
         raise KernelError(f"linear: a is {tuple(a.shape)} {a.dtype}, w is {tuple(w.shape)} {w.dtype}")
     if epilogue not in EPILOGUES:
         raise KernelError(f"unknown epilogue '{epilogue}'")
+    if splits is not None:
+        want = torch.float32 if epilogue in ("add_residual", "store_f32") else a.dtype
+        ok = (kv_scatter is None and a.dtype == torch.bfloat16 and out.shape == (M, N) and out.dtype == want
+              and (bias is None or (bias.dtype == torch.float32 and bias.numel() == N and bias.is_contiguous()))
+              and w.stride(0) % 8 == 0 and w.data_ptr() % 16 == 0)
+        if ok and _linear_from_splits(a, w, bias, out, epilogue) is not None:
+            return out
+        a = splits.tensor()
     want = torch.float32 if epilogue in ("add_residual", "store_f32") else a.dtype
     if out.shape != (M, N) or out.dtype != want:
         raise KernelError(f"linear({epilogue}): out must be [{M}, {N}] {want}, got {tuple(out.shape)} {out.dtype}")
@@ -319,7 +368,7 @@ def paged_attention(q: torch.Tensor, q_col: int, n_heads: int, n_kv_heads: int, 
                     block_tables: torch.Tensor, token_seq: torch.Tensor, positions: torch.Tensor,
                     scale: float, window: int, out: torch.Tensor, *, cu_q: Optional[torch.Tensor] = None,
                     ctx_len: Optional[torch.Tensor] = None, max_q_len: int = 0, max_ctx_len: int = 0,
-                    append: Optional[tuple] = None) -> torch.Tensor:
+                    append: Optional[tuple] = None, n_single: int = 0, may_split: bool = False):
     """Causal attention of the step's queries over the pages.
 
     q: [T, >= q_col + n_heads*head_dim] (queries of token t start at column q_col);
@@ -330,6 +379,14 @@ def paged_attention(q: torch.Tensor, q_col: int, n_heads: int, n_kv_heads: int, 
     ``append=(k_col, v_col, slots)``: the step's own keys and values are still in q's rows
     (columns k_col, v_col) and this op writes them to row ``slots[t]`` of the pages first
     (fused into the decode kernel where that runs); without it they are in the pages already.
+
+    ``n_single``: the first n_single sequences of the batch bring one token each (decoded tokens stand
+    first in a mixed step). They then go to the single-query kernel and only the portions behind them
+    to the 64-query tiles of the matrix cores, where a lone query would leave 63 of 64 lanes idle.
+
+    ``may_split``: the caller hands the result to ``linear`` next and accepts an ``AttentionSplits``
+    in place of ``out`` (returned when a few single tokens' keys were split over several workgroups
+    each; ``out`` is then left unwritten).
     """
     _gpu(q, k_pages, v_pages, block_tables, token_seq, positions, out)
     _rows2d(q, "q")
@@ -370,23 +427,50 @@ def paged_attention(q: torch.Tensor, q_col: int, n_heads: int, n_kv_heads: int, 
             _i32(slots, "slots", T)
             if max(k_col, v_col) + kv_dim > q.shape[1] or min(k_col, v_col) < 0 or (k_col * esz) % 16 or (v_col * esz) % 16:
                 raise KernelError("key/value columns lie outside q's rows or are not 16-byte aligned")
+    tiles_ok = (q.dtype == torch.bfloat16 and head_dim in (32, 64, 128) and max_q_len > 1
+                and cu_q is not None and ctx_len is not None
+                and page_size & (page_size - 1) == 0 and page_size >= head_dim // 16
+                and block_tables.shape[1] <= 2048)
+    if (tiles_ok and 0 < n_single < block_tables.shape[0] and lpk >= 2 and (lpk & (lpk - 1)) == 0
+            and block_tables.shape[1] <= 4096):
+        # a mixed step: the leading single tokens, then the portions, two launches over disjoint rows
+        # (every row's keys and values are in the pages by now)
+        paged_attention(q[:n_single], q_col, n_heads, n_kv_heads, head_dim, k_pages, v_pages, page_size,
+                        block_tables[:n_single], token_seq[:n_single], positions[:n_single], scale, window,
+                        out[:n_single], max_q_len=1, max_ctx_len=max_ctx_len)
+        B = block_tables.shape[0] - n_single
+        _i32(cu_q, "cu_q", block_tables.shape[0] + 1)
+        _i32(ctx_len, "ctx_len", block_tables.shape[0])
+        if out.data_ptr() % 16 or (out.stride(0) * esz) % 8:
+            raise KernelError("attention output rows must be 8-byte aligned")
+        lib = load_library("attention_prefill")
+        # (row numbers in cu_q are absolute, so q and out are passed whole and the per-sequence arrays from
+        # the first portion on)
+        _check(lib.mllm_prefill_attention_bf16(
+            _p(q), q.stride(0), q_col, _p(k_pages), _p(v_pages), kv_dim, _p(block_tables[n_single:]),
+            block_tables.shape[1], _p(cu_q[n_single:]), _p(ctx_len[n_single:]), B, (T - n_single) // 64 + B,
+            n_heads, n_kv_heads, head_dim, page_size, ctypes.c_float(scale), int(window or 0), _p(out),
+            out.stride(0), _stream()), "prefill_attention")
+        return out
     if decode:
         # every query is a single decoded token: split its keys over workgroups
         pairs = T * n_heads
-        nsplit, waves = _decode_launch_shape(pairs, max_ctx_len)
+        unmerged = (may_split and q.dtype == torch.bfloat16 and T <= MERGE_MAX_ROWS and head_dim % 8 == 0
+                    and DECODE_SHAPE_OVERRIDE is None)
+        nsplit, waves = _decode_launch_shape(pairs, max_ctx_len, unmerged)
+        unmerged = unmerged and nsplit > 1
         ws, counters = _decode_workspace(q.device, pairs, nsplit, head_dim)
         lib = load_library("attention_decode")
         _check(lib.mllm_decode_attention(
             _p(q), q.stride(0), q_col, _p(k_pages), _p(v_pages), kv_dim, _p(block_tables), block_tables.shape[1],
             _p(token_seq), _p(positions), T, n_heads, n_kv_heads, head_dim, page_size, ctypes.c_float(scale),
             int(window or 0), nsplit, waves, _p(out), out.stride(0), _p(ws), _p(counters), k_col, v_col, _p(slots),
-            _dt(q), _stream()),
+            1 if unmerged else 0, _dt(q), _stream()),
             "decode_attention")
+        if unmerged:
+            return AttentionSplits(ws, T, n_heads, head_dim, nsplit, q.dtype)
         return out
-    if (q.dtype == torch.bfloat16 and head_dim in (32, 64, 128) and max_q_len > 1
-            and cu_q is not None and ctx_len is not None
-            and page_size & (page_size - 1) == 0 and page_size >= head_dim // 16
-            and block_tables.shape[1] <= 2048):
+    if tiles_ok:
         # prompt portions: tiles of 64 queries on the matrix cores
         B = block_tables.shape[0]
         _i32(cu_q, "cu_q", B + 1)
@@ -467,10 +551,23 @@ def reserve_scratch(device, rows: int, vocab: int, n_heads: int = 0, head_dim: i
         _decode_workspace(device, rows * n_heads, DECODE_MAX_SPLIT, head_dim)
 
 
-def _decode_launch_shape(pairs: int, max_ctx_len: int):
+DECODE_UNMERGED_SHAPE = None     # (nsplit, waves) for splits that the next product merges: tuning scripts
+
+
+def _decode_launch_shape(pairs: int, max_ctx_len: int, unmerged: bool = False):
     """How many workgroups share one (token, head) pair's keys, and wavefronts per workgroup."""
     if DECODE_SHAPE_OVERRIDE is not None:
         return DECODE_SHAPE_OVERRIDE
+    if unmerged:
+        # The splits cost nothing to merge here (the next product does it while it loads), so few pairs
+        # are spread over the compute units: a unit streams keys at 35 to 90 GB/s, and a pair's keys
+        # and values at 768 tokens are 200 KB. Every split keeps at least 128 keys.
+        if DECODE_UNMERGED_SHAPE is not None:
+            return DECODE_UNMERGED_SHAPE
+        nsplit = max(1, min(MERGE_MAX_SPLITS, 384 // max(pairs, 1), max_ctx_len // 128))
+        if nsplit > 1:
+            keys = -(-max_ctx_len // nsplit)
+            return nsplit, max(2, min(12, -(-keys // 64)))
     # One workgroup per pair: merging splits (fences, a second merge) costs about 3 us, more than
     # the parallelism gains below about 2,000 keys (measured at 12 to 96 pairs). Few pairs get more
     # wavefronts each instead (measured: 12 are 1 to 3 % of a decode step faster than 8 up to 200

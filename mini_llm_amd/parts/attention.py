@@ -66,9 +66,12 @@ class CausalSelfAttention(Mixer):
             self.position.in_mixer(qkv, self, ctx)
         append = (self.q_dim, self.q_dim + self.kv_dim, ctx.slots[g]) if write and not scatter else None
         attn = torch.empty((T, self.q_dim), dtype=self.dtype, device=h.device)
-        ops.paged_attention(qkv, 0, self.n_heads, self.n_kv_heads, self.head_dim,
-                            cache_view.k_pages, cache_view.v_pages, cache_view.page_size,
-                            ctx.block_tables[g], ctx.token_seq, ctx.positions, self.scale, self.window, attn,
-                            cu_q=ctx.cu_q, ctx_len=ctx.ctx_len, max_q_len=ctx.max_q_len,
-                            max_ctx_len=ctx.max_ctx_len, append=append)
+        # (the result may come back unmerged, as the states of several workgroups per token and head:
+        # the output projection takes either)
+        attn = ops.paged_attention(qkv, 0, self.n_heads, self.n_kv_heads, self.head_dim,
+                                   cache_view.k_pages, cache_view.v_pages, cache_view.page_size,
+                                   ctx.block_tables[g], ctx.token_seq, ctx.positions, self.scale, self.window, attn,
+                                   cu_q=ctx.cu_q, ctx_len=ctx.ctx_len, max_q_len=ctx.max_q_len,
+                                   max_ctx_len=ctx.max_ctx_len, append=append, n_single=ctx.n_single,
+                                   may_split=True)
         self.out(attn, x, "add_residual")

@@ -99,6 +99,7 @@ def kv_append(src, k_col, v_col, kv_dim, k_pages, v_pages, slots):
 
 def paged_attention(q, q_col, n_heads, n_kv_heads, head_dim, k_pages, v_pages, page_size, block_tables,
                     token_seq, positions, scale, window, out, append=None, **_):
+    # (the hints n_single and may_split change nothing here: the result is always merged into `out`)
     T = q.shape[0]
     if append is not None:
         kv_append(q, append[0], append[1], n_kv_heads * head_dim, k_pages, v_pages, append[2])

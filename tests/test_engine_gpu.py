@@ -132,6 +132,48 @@ def test_graph_decode_matches_eager_steps(tiny_model_dirs, dtype):
     assert all(len(o) == 20 for o in outs["graph"])
 
 
+def test_scratch_stays_put_while_decode_graphs_of_growing_batches_are_captured(tmp_path):
+    """A vocabulary of 50,257 (25 argmax chunks a row) and up to 176 requests, no warm-up: a batch of 8
+    captures its graph first, then 176 requests capture the larger ones, then 8 again replay the first
+    graph. The kernels' scratch is sized for the largest batch when the runner is built, so its
+    addresses never change and the early graph still writes where its replays read; tokens equal those
+    of general steps that wait for every token."""
+    from mini_llm_amd import Engine, EngineOptions, SamplingParams, write_random_model
+    from mini_llm_amd.kernels import ops
+    cfg = dict(architectures=["GPT2LMHeadModel"], model_type="gpt2", n_layer=2, n_embd=64, n_head=2, n_inner=128,
+               vocab_size=50257, n_positions=48, layer_norm_epsilon=1e-5, activation_function="gelu_new",
+               eos_token_id=50256, bos_token_id=50256)
+    d = write_random_model(cfg, str(tmp_path / "wide"), seed=6)
+    g = torch.Generator().manual_seed(3)
+    few = [torch.randint(0, 50256, (3 + i,), generator=g).tolist() for i in range(8)]
+    many = [torch.randint(0, 50256, (2 + i % 7,), generator=g).tolist() for i in range(176)]
+    sp = SamplingParams(max_new_tokens=5, ignore_eos=True)
+    names = ("argmax_values", "argmax_indices", "decode_partials", "decode_counters")
+
+    def run(graphs: bool):
+        e = Engine.from_pretrained(d, dtype="float32", options=EngineOptions(
+            kv_block_size=4, total_kv_blocks=176 * 4 + 8, max_batch_num=176, max_tokens_per_step=1024,
+            prefill_chunk=16, overlap_decode=graphs))
+        if not graphs:
+            e.runner.fast_decode = False
+        before = [ops.scratch_address("cuda:0", n) for n in names]
+        assert all(before), "the runner reserves the scratch when it is built"
+        outs = [e.generate(few, sp)]
+        first = dict(e.runner._graphs)
+        outs.append(e.generate(many, sp))
+        outs.append(e.generate(few, sp))
+        if graphs:
+            assert first and all(e.runner._graphs.get(k) is v for k, v in first.items()), "an early graph was dropped"
+            assert any(k[0] == 176 for k in e.runner._graphs)
+            assert [ops.scratch_address("cuda:0", n) for n in names] == before
+        assert e.stats()["free_pages"] == 176 * 4 + 8
+        return outs
+
+    with_graphs, general = run(True), run(False)
+    assert with_graphs[0] == with_graphs[2]
+    assert with_graphs == general
+
+
 def test_command_line(tiny_model_dirs, tmp_path):
     cfg, w = plain_gpt2.read_model(tiny_model_dirs["a"])
     prompts = _prompts("a", (5, 17), 1)

@@ -358,7 +358,7 @@ def test_kv_append_reference_vector(ops, dtype):
     assert (kp.cpu()[untouched] == -1).all() and (vp.cpu()[untouched] == -1).all()
 
 
-def _attention_case(ops, dtype, H, Hkv, dh, page, seqs, window, gen, boost=None):
+def _attention_case(ops, dtype, H, Hkv, dh, page, seqs, window, gen, boost=None, n_single=0):
     """seqs: list of (start, q_len). Builds pages in scrambled order, garbage elsewhere."""
     B = len(seqs)
     ctx = [s + n for s, n in seqs]
@@ -398,7 +398,7 @@ def _attention_case(ops, dtype, H, Hkv, dh, page, seqs, window, gen, boost=None)
     ops.paged_attention(q.to(DEV), 8, H, Hkv, dh, kp.to(DEV), vp.to(DEV), page, tables.to(DEV),
                         token_seq.to(DEV), positions.to(DEV), scale, window, out,
                         cu_q=cu.to(DEV), ctx_len=torch.tensor(ctx, dtype=torch.int32).to(DEV),
-                        max_q_len=max(n for _, n in seqs), max_ctx_len=max(ctx))
+                        max_q_len=max(n for _, n in seqs), max_ctx_len=max(ctx), n_single=n_single)
     ref = torch.zeros(T, H * dh, dtype=torch.float64)
     plain_ops.paged_attention(q, 8, H, Hkv, dh, kp, vp, page, tables, token_seq, positions, scale, window, ref)
     return out.cpu().double(), ref
@@ -496,6 +496,90 @@ def test_paged_attention_prefill_tiles(ops, H, Hkv, dh, page, window):
     out, ref = _attention_case(ops, torch.bfloat16, H, Hkv, dh, page, seqs, window, g)
     assert torch.isfinite(out).all()
     assert (out - ref).abs().max() <= _tol(torch.bfloat16, 2)
+
+
+@pytest.mark.parametrize("T", [1, 8, 16])
+@pytest.mark.parametrize("H,Hkv,dh,page,N", [(12, 12, 64, 16, 768), (25, 25, 64, 16, 1600), (3, 3, 32, 8, 96),
+                                             (4, 2, 128, 16, 200), (16, 16, 64, 16, 1024)])
+@pytest.mark.parametrize("shape", [(2, 4), (3, 2), (4, 12), None])
+def test_decode_attention_splits_merged_by_the_next_product(ops, T, H, Hkv, dh, page, N, shape):
+    """Single tokens whose keys are split over several workgroups per (token, head): the attention op
+    hands back the splits unmerged and the product that follows merges them while it loads. Equal to
+    attention followed by the product on merged rows; contexts from one key (most splits empty) to
+    several hundred; the tokens' own keys come from their qkv rows and reach the pages."""
+    g = torch.Generator().manual_seed(T * 31 + H + dh)
+    ctx = [1, 700, 130, 2, 64, 65, 300, 17, 1000, 5, 129, 511, 33, 256, 90, 3][:T]
+    nblk = [-(-c // page) for c in ctx]
+    n_pages = sum(nblk) + 2
+    perm = torch.randperm(n_pages, generator=g).tolist()
+    kv_dim, D = Hkv * dh, H * dh
+    kp = torch.full((n_pages * page, kv_dim), float("nan"), dtype=torch.bfloat16)
+    vp = torch.full((n_pages * page, kv_dim), float("nan"), dtype=torch.bfloat16)
+    tables = torch.zeros(T, max(nblk), dtype=torch.int32)
+    qkv = _rand((T, D + 2 * kv_dim), torch.bfloat16, g)
+    slots = torch.zeros(T, dtype=torch.int32)
+    used = 0
+    for b in range(T):
+        for j in range(nblk[b]):
+            tables[b, j] = perm[used]
+            used += 1
+        js = torch.arange(ctx[b] - 1)                   # the last key is the token's own, not in the pages yet
+        rows = tables[b].long()[js // page] * page + js % page
+        kp[rows] = _rand((ctx[b] - 1, kv_dim), torch.bfloat16, g)
+        vp[rows] = _rand((ctx[b] - 1, kv_dim), torch.bfloat16, g)
+        slots[b] = int(tables[b, (ctx[b] - 1) // page]) * page + (ctx[b] - 1) % page
+    token_seq = torch.arange(T, dtype=torch.int32)
+    positions = torch.tensor([c - 1 for c in ctx], dtype=torch.int32)
+    w = _rand((N, D), torch.bfloat16, g, std=1.0 / math.sqrt(D))
+    bias = 0.5 * _rand((N,), torch.float32, g)
+    x0 = _rand((T, N), torch.float32, g)
+    # reference: append, attention, product, all plain
+    rk, rv = kp.clone(), vp.clone()
+    att = torch.zeros(T, D, dtype=torch.float64)
+    plain_ops.paged_attention(qkv, 0, H, Hkv, dh, rk, rv, page, tables, token_seq, positions, dh ** -0.5, 0, att,
+                              append=(D, D + kv_dim, slots))
+    ref = plain_ops.linear(att, w.double(), bias, x0.double().clone(), "add_residual")
+    kd, vd = kp.to(DEV), vp.to(DEV)
+    out = torch.empty(T, D, dtype=torch.bfloat16, device=DEV)
+    ops.DECODE_UNMERGED_SHAPE = shape
+    try:
+        a = ops.paged_attention(qkv.to(DEV), 0, H, Hkv, dh, kd, vd, page, tables.to(DEV), token_seq.to(DEV),
+                                positions.to(DEV), dh ** -0.5, 0, out, max_q_len=1, max_ctx_len=max(ctx),
+                                append=(D, D + kv_dim, slots.to(DEV)), may_split=True)
+    finally:
+        ops.DECODE_UNMERGED_SHAPE = None
+    if shape is not None or (max(ctx) >= 256 and T * H <= 192):
+        assert isinstance(a, ops.AttentionSplits) and a.nsplit == (shape[0] if shape else a.nsplit) and a.nsplit > 1
+    x = x0.clone().to(DEV)
+    ops.linear(a, w.to(DEV), bias.to(DEV), x, "add_residual")
+    assert torch.isfinite(x).all()
+    assert (x.cpu().double() - ref).abs().max() <= 3e-2
+    written = slots.long()
+    assert torch.equal(kd.cpu()[written], rk[written]) and torch.equal(vd.cpu()[written], rv[written])
+    if isinstance(a, ops.AttentionSplits):
+        # merged into an ordinary activation by the kernel of its own: the same rows
+        merged = a.tensor()
+        assert (merged.cpu().double() - att).abs().max() <= 2e-2
+        y = torch.empty(T, N, dtype=torch.bfloat16, device=DEV)
+        ops.linear(a, w.to(DEV), bias.to(DEV), y, "gelu_tanh")
+        ref_y = plain_ops.linear(att, w.double(), bias, torch.empty(T, N, dtype=torch.float64), "gelu_tanh")
+        assert (y.cpu().double() - ref_y).abs().max() <= 3e-2
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("H,Hkv,dh,page,window", [(12, 12, 64, 16, 0), (3, 3, 32, 8, 0), (4, 1, 128, 16, 40), (4, 4, 16, 4, 0)])
+def test_paged_attention_single_tokens_before_portions(ops, dtype, H, Hkv, dh, page, window):
+    """A scheduler's mixed step: decoded tokens first, then prompt portions. The leading single tokens
+    (`n_single` of them) go to the single-query kernel and the rest to the query tiles; a single token
+    that stands among the portions stays with them. Same result as without the hint."""
+    g = torch.Generator().manual_seed(H + dh)
+    seqs = [(130, 1), (0, 1), (299, 1), (64, 1), (0, 37), (17, 1), (5, 70), (100, 130)]
+    out, ref = _attention_case(ops, dtype, H, Hkv, dh, page, seqs, window, g, n_single=4)
+    assert torch.isfinite(out).all()
+    assert (out - ref).abs().max() <= _tol(dtype, 2)
+    g = torch.Generator().manual_seed(H + dh)
+    plain, _ = _attention_case(ops, dtype, H, Hkv, dh, page, seqs, window, g)
+    assert (out - plain).abs().max() <= _tol(dtype, 2)
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
