@@ -88,7 +88,17 @@ decode_attention_kernel(// the first 16 dwords arrive in registers with the wave
     const int hk = h / (n_heads / n_kv_heads);
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / MLLM_WAVE), lane = threadIdx.x % MLLM_WAVE;
     const int c = lane % LPK, g = lane / LPK;
-    const int b = token_seq[t], p = positions[t];
+    // (token_seq == nullptr: every sequence brings one token, token t belongs to sequence t; the block
+    // table can then be requested at once, beside the position, instead of after a load of its own)
+    const int b = token_seq != nullptr ? token_seq[t] : t;
+    const int* gtable_row = block_tables + static_cast<size_t>(b) * max_blocks;
+    // Without a window the keys start at block 0 whatever the position is, and rows of the table are
+    // filled to their end (zeros behind a sequence's last block): the whole row goes to LDS without
+    // waiting for the position.
+    const bool whole_row = window <= 0 && max_blocks <= DEC_TABLE_LDS;
+    if (whole_row)
+        for (int i = threadIdx.x; i < max_blocks; i += blockDim.x) sm_table[i] = gtable_row[i];
+    const int p = positions[t];
     const int lo = (window > 0 && p - window + 1 > 0) ? p - window + 1 : 0;
     const int n_keys = p - lo + 1;
     const int per = (n_keys + nsplit - 1) / nsplit;
@@ -105,10 +115,10 @@ decode_attention_kernel(// the first 16 dwords arrive in registers with the wave
 
     // The block table entries of this workgroup's keys go to LDS first, so that no key load waits
     // for a table load.
-    const int first_blk = kb >> shift;
+    const int first_blk = whole_row ? 0 : kb >> shift;
     const int n_blk = ke_pages > kb ? ((ke_pages - 1) >> shift) - first_blk + 1 : 0;
-    {
-        const int* gtable = block_tables + static_cast<size_t>(b) * max_blocks + first_blk;
+    if (!whole_row) {
+        const int* gtable = gtable_row + first_blk;
         for (int i = threadIdx.x; i < n_blk; i += blockDim.x) sm_table[i] = gtable[i];
     }
 

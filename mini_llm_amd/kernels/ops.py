@@ -437,7 +437,7 @@ def paged_attention(q: torch.Tensor, q_col: int, n_heads: int, n_kv_heads: int, 
         # (every row's keys and values are in the pages by now)
         paged_attention(q[:n_single], q_col, n_heads, n_kv_heads, head_dim, k_pages, v_pages, page_size,
                         block_tables[:n_single], token_seq[:n_single], positions[:n_single], scale, window,
-                        out[:n_single], max_q_len=1, max_ctx_len=max_ctx_len)
+                        out[:n_single], max_q_len=1, max_ctx_len=max_ctx_len, n_single=n_single)
         B = block_tables.shape[0] - n_single
         _i32(cu_q, "cu_q", block_tables.shape[0] + 1)
         _i32(ctx_len, "ctx_len", block_tables.shape[0])
@@ -461,9 +461,12 @@ def paged_attention(q: torch.Tensor, q_col: int, n_heads: int, n_kv_heads: int, 
         unmerged = unmerged and nsplit > 1
         ws, counters = _decode_workspace(q.device, pairs, nsplit, head_dim)
         lib = load_library("attention_decode")
+        # every sequence of the batch brings one token (the caller says so): token t is sequence t, and the
+        # kernel need not load that
+        seq_of_token = None if n_single == T == block_tables.shape[0] else token_seq
         _check(lib.mllm_decode_attention(
             _p(q), q.stride(0), q_col, _p(k_pages), _p(v_pages), kv_dim, _p(block_tables), block_tables.shape[1],
-            _p(token_seq), _p(positions), T, n_heads, n_kv_heads, head_dim, page_size, ctypes.c_float(scale),
+            _p(seq_of_token), _p(positions), T, n_heads, n_kv_heads, head_dim, page_size, ctypes.c_float(scale),
             int(window or 0), nsplit, waves, _p(out), out.stride(0), _p(ws), _p(counters), k_col, v_col, _p(slots),
             1 if unmerged else 0, _dt(q), _stream()),
             "decode_attention")
@@ -564,7 +567,9 @@ def _decode_launch_shape(pairs: int, max_ctx_len: int, unmerged: bool = False):
         # and values at 768 tokens are 200 KB. Every split keeps at least 128 keys.
         if DECODE_UNMERGED_SHAPE is not None:
             return DECODE_UNMERGED_SHAPE
-        nsplit = max(1, min(MERGE_MAX_SPLITS, 384 // max(pairs, 1), max_ctx_len // 128))
+        # (measured at GPT-2 small sizes, 768 keys: 12 pairs x 4 splits of 4 wavefronts and 96 pairs x 2 splits
+        # of 8 wavefronts are the fastest shapes; more workgroups than compute units lose again)
+        nsplit = max(1, min(MERGE_MAX_SPLITS, 256 // max(pairs, 1), max_ctx_len // 128))
         if nsplit > 1:
             keys = -(-max_ctx_len // nsplit)
             return nsplit, max(2, min(12, -(-keys // 64)))
