@@ -37,6 +37,9 @@ HIPCC_FLAGS = [
     "-Wno-unused-command-line-argument", "-Wno-unknown-warning-option",
 ]
 CXX_FLAGS = ["-O2", "-std=c++17", "-fPIC", "-shared", "-Wall"]
+# host code that uses the HIP runtime (streams, memory) and the kernel libraries' entry points
+HIPHOST_FLAGS = ["-O2", "-std=c++17", "-fPIC", "-shared", "-Wall", "-x", "c++", "-D__HIP_PLATFORM_AMD__",
+                 "-I/opt/rocm/include"]
 
 # library name -> (compiler kind, sources relative to csrc, headers that also enter the hash)
 LIBRARIES: Dict[str, dict] = {
@@ -54,6 +57,15 @@ LIBRARIES: Dict[str, dict] = {
     "sampling": {"kind": "hip", "sources": ["kernels/sampling.hip"],
                  "headers": ["kernels/common.h", "kernels/noalloc.h"]},
     "peaks": {"kind": "hip", "sources": ["kernels/peaks.hip"], "headers": ["kernels/common.h"]},
+    # the native engine: checked dispatch over the kernels, the parts, the model's step function
+    # (host code only; it calls the kernel libraries' entry points)
+    "engine": {
+        "kind": "hiphost",
+        "sources": ["engine/ops.cc", "engine/parts.cc", "engine/engine_api.cc"],
+        "headers": ["engine/ops.h", "engine/parts.h", "engine/kernels.h"],
+        "needs": ["elementwise", "gemm_f32", "gemm_bf16", "attention", "attention_decode", "attention_prefill",
+                  "sampling"],
+    },
 }
 
 _loaded: Dict[str, ctypes.CDLL] = {}
@@ -78,7 +90,7 @@ def _paths(name: str):
 def _source_hash(name: str) -> str:
     spec, srcs, hdrs = _paths(name)
     h = hashlib.sha256()
-    flags = HIPCC_FLAGS if spec["kind"] == "hip" else CXX_FLAGS
+    flags = {"hip": HIPCC_FLAGS, "cxx": CXX_FLAGS, "hiphost": HIPHOST_FLAGS}[spec["kind"]]
     h.update(" ".join(flags).encode())
     for p in srcs + hdrs:
         with open(p, "rb") as f:
@@ -115,16 +127,26 @@ def build_library(name: str, verbose: bool = True) -> str:
     spec, srcs, _ = _paths(name)
     os.makedirs(LIB_DIR, exist_ok=True)
     so = lib_path(name)
+    link: List[str] = []
     if spec["kind"] == "hip":
         cc = _find("hipcc", ["/opt/rocm/bin"])
         cmd = [cc] + HIPCC_FLAGS
+    elif spec["kind"] == "hiphost":
+        for dep in spec.get("needs", []):          # link against the kernel libraries beside it
+            if not is_current(dep):
+                build_library(dep, verbose)
+        cc = _find("g++", ["/usr/bin"])
+        cmd = [cc] + HIPHOST_FLAGS
+        link = [f"-L{LIB_DIR}"] + [f"-lmllm_{d}" for d in spec.get("needs", [])] + \
+               ["-L/opt/rocm/lib", "-lamdhip64", "-Wl,-rpath,$ORIGIN", "-Wl,-rpath,/opt/rocm/lib"]
     else:
         cc = _find("g++", ["/usr/bin"])
         cmd = [cc] + CXX_FLAGS
     # Compile to a private name, then rename: a concurrent process never sees a half-written file.
     fd, tmp = tempfile.mkstemp(prefix=f".{name}.", suffix=".so", dir=LIB_DIR)
     os.close(fd)
-    cmd = cmd + [f"-I{os.path.join(CSRC, 'kernels')}", f"-I{os.path.join(CSRC, 'runtime')}"] + srcs + ["-o", tmp]
+    cmd = cmd + [f"-I{os.path.join(CSRC, 'kernels')}", f"-I{os.path.join(CSRC, 'runtime')}",
+                 f"-I{os.path.join(CSRC, 'engine')}"] + srcs + ["-o", tmp] + link
     env = dict(os.environ)
     env.setdefault("TMPDIR", tempfile.gettempdir())
     if not env.get("HOME") or not os.access(env["HOME"], os.W_OK):
@@ -164,8 +186,12 @@ def build_library(name: str, verbose: bool = True) -> str:
 def build_all(verbose: bool = True, jobs: int = 4) -> None:
     """Compiles every library, whatever is there already."""
     from concurrent.futures import ThreadPoolExecutor
+    first = [n for n in LIBRARIES if not LIBRARIES[n].get("needs")]
     with ThreadPoolExecutor(max_workers=jobs) as ex:
-        list(ex.map(lambda n: build_library(n, verbose), LIBRARIES))
+        list(ex.map(lambda n: build_library(n, verbose), first))
+    for n in LIBRARIES:                     # then those that link against others
+        if n not in first:
+            build_library(n, verbose)
     with _lock:
         _loaded.clear()
 

@@ -1,0 +1,195 @@
+// The parts a model is put together from, natively: mixer, feed-forward, norm, block arrangement,
+// and the model that runs them in the order its configuration gives.
+//
+// A part knows its own sizes and constants (parameters) and the tensors it owns; it does not know
+// which model it is in. Parts are built by kind name through registries, from a bag of parameters
+// (numbers, strings, device tensors), so that another kind of part is one class and one
+// registration, and a configuration chooses layer by layer.
+//
+// Interfaces (`x` is the fp32 residual stream [T, hidden]; `h` a normalised activation in the
+// compute dtype; `step` the batch's index arrays; `arena` memory for the step's temporaries):
+//   Norm::forward(x, rows, n) -> h            Norm::linear(x, lin, out, epilogue, rows)
+//   Mixer::forward(h, step, cache, x, write)  adds the mixer's output into x
+//   FeedForward::forward(h, step, x)          adds its output into x
+//   Block::forward(x, step, cache, write)     runs one layer on the stream
+//
+// The reference's model has these pieces fixed in one class
+// (/root/reference/src/model/gpt2_model.cu:275-363 block_prefill, :404-428 the head).
+#pragma once
+
+#include <functional>
+#include <map>
+#include <memory>
+#include <string>
+#include <vector>
+
+#include "ops.h"
+
+namespace minillm {
+
+// Memory for a step's temporaries: a bump allocator over one device buffer that the caller owns.
+class Arena {
+public:
+    Arena(void* base, size_t bytes) : base_(static_cast<char*>(base)), capacity_(bytes) {}
+    void* take(size_t bytes);
+    Tensor2 tensor(int dtype, int64_t rows, int64_t cols) {
+        return Tensor2(take(static_cast<size_t>(rows) * cols * dtype_size(dtype)), dtype, rows, cols);
+    }
+    size_t mark() const { return used_; }
+    void release(size_t mark) { used_ = mark; }
+    size_t peak() const { return peak_; }
+
+private:
+    char* base_;
+    size_t capacity_, used_ = 0, peak_ = 0;
+};
+
+// The step's batch: sizes known to the host and device arrays (int32).
+struct StepView {
+    int n_tokens = 0, n_seqs = 0, n_logits = 0, max_q_len = 0, max_ctx_len = 0, n_single = 0;
+    const int* token_ids = nullptr;    // [T]
+    const int* positions = nullptr;    // [T]
+    const int* token_seq = nullptr;    // [T]
+    const int* cu_q = nullptr;         // [B+1]
+    const int* ctx_len = nullptr;      // [B]
+    const int* starts = nullptr;       // [B]
+    const int* state_slots = nullptr;  // [B]
+    const int* logit_rows = nullptr;   // [n_logits]
+    int n_groups = 0;
+    const int* const* block_tables = nullptr;   // per group [B, max_blocks[g]]
+    const int* max_blocks = nullptr;            // per group
+    const int* const* slots = nullptr;          // per group [T]
+};
+
+// What a call of the execution order sees of its cache.
+struct CacheView {
+    int kind = 0;                  // 0 none, 1 pages of keys and values, 2 fixed-size state slots
+    Tensor2 k_pages, v_pages;      // [n_pages * page_size, kv_dim]
+    int group = 0, page_size = 0, window = 0;
+    void* state = nullptr;         // [n_slots, slot_bytes]
+    size_t slot_bytes = 0;
+    int n_slots = 0;
+};
+
+// A bag of parameters a part is built from.
+struct Params {
+    std::map<std::string, double> num;
+    std::map<std::string, std::string> str;
+    std::map<std::string, Tensor2> tensor;
+
+    double number(const std::string& key) const;
+    double number(const std::string& key, double fallback) const;
+    int integer(const std::string& key) const { return static_cast<int>(number(key)); }
+    const std::string& string(const std::string& key) const;
+    const Tensor2& weights(const std::string& key) const;          // must be there
+    const Tensor2* weights_or_null(const std::string& key) const;
+};
+
+class Linear {
+public:
+    Linear() = default;
+    // weight [out, in] in the compute dtype (k contiguous: the layout the matrix kernels read), bias fp32 [out] or none
+    Linear(const Tensor2& weight, const Tensor2* bias);
+    void operator()(const Tensor2& a, const Tensor2& out, int epilogue, const KvScatter* kv, hipStream_t s) const {
+        linear(a, weight, bias, out, epilogue, kv, s);
+    }
+    Tensor2 weight;
+    const float* bias = nullptr;
+    int in_features() const { return static_cast<int>(weight.cols); }
+    int out_features() const { return static_cast<int>(weight.rows); }
+};
+
+class Norm {
+public:
+    virtual ~Norm() = default;
+    // h[i,:] = norm(x[rows ? rows[i] : i, :]), n rows, from the arena
+    virtual Tensor2 forward(const Tensor2& x, const int* rows, int n, Arena& arena, hipStream_t s) const = 0;
+    // out = epilogue(lin(norm(x[rows]))); a norm with a fused kernel overrides this
+    virtual void linear(const Tensor2& x, const Linear& lin, const Tensor2& out, int epilogue, const int* rows,
+                        Arena& arena, hipStream_t s) const;
+    virtual size_t workspace_bytes(int rows) const = 0;
+    int dtype = BF16;
+};
+
+// The input of a sub-layer as (stream, norm), not yet normalised: a part's first linear map may
+// absorb the norm.
+class NormedInput {
+public:
+    NormedInput(const Norm& norm, const Tensor2& x) : norm_(norm), x_(x) {}
+    const Tensor2& tensor(Arena& arena, hipStream_t s);
+    void linear(const Linear& lin, const Tensor2& out, int epilogue, const KvScatter* kv, Arena& arena, hipStream_t s);
+    int64_t rows() const { return x_.rows; }
+
+private:
+    const Norm& norm_;
+    Tensor2 x_, h_;
+    bool have_ = false;
+};
+
+class Mixer {
+public:
+    virtual ~Mixer() = default;
+    virtual void forward(NormedInput& h, const StepView& step, const CacheView& cache, const Tensor2& x, bool write,
+                         Arena& arena, hipStream_t s) const = 0;
+    virtual size_t workspace_bytes(int tokens) const = 0;
+};
+
+class FeedForward {
+public:
+    virtual ~FeedForward() = default;
+    virtual void forward(NormedInput& h, const StepView& step, const Tensor2& x, Arena& arena, hipStream_t s) const = 0;
+    virtual size_t workspace_bytes(int tokens) const = 0;
+};
+
+class Block {
+public:
+    virtual ~Block() = default;
+    virtual void forward(const Tensor2& x, const StepView& step, const CacheView& cache, bool write, Arena& arena,
+                         hipStream_t s) const = 0;
+    virtual size_t workspace_bytes(int tokens) const = 0;
+};
+
+// -- registries: kind name -> factory ---------------------------------------------------------------
+using NormFactory = std::function<std::unique_ptr<Norm>(const Params&)>;
+using MixerFactory = std::function<std::unique_ptr<Mixer>(const Params&)>;
+using FeedForwardFactory = std::function<std::unique_ptr<FeedForward>(const Params&)>;
+using BlockFactory = std::function<std::unique_ptr<Block>(std::unique_ptr<Mixer>, std::unique_ptr<FeedForward>,
+                                                         std::vector<std::unique_ptr<Norm>>)>;
+void register_norm(const std::string& kind, NormFactory f);
+void register_mixer(const std::string& kind, MixerFactory f);
+void register_feed_forward(const std::string& kind, FeedForwardFactory f);
+void register_block(const std::string& kind, BlockFactory f);
+bool has_part(const std::string& category, const std::string& kind);     // category: norm | mixer | feed_forward | block
+std::unique_ptr<Norm> build_norm(const std::string& kind, const Params& p);
+std::unique_ptr<Mixer> build_mixer(const std::string& kind, const Params& p);
+std::unique_ptr<FeedForward> build_feed_forward(const std::string& kind, const Params& p);
+std::unique_ptr<Block> build_block(const std::string& kind, std::unique_ptr<Mixer> m, std::unique_ptr<FeedForward> f,
+                                   std::vector<std::unique_ptr<Norm>> norms);
+
+// One entry of the execution order: which layer runs, on which cache, and whether it writes it.
+struct LayerCall {
+    int layer = 0, cache = 0;
+    bool write = true;
+};
+
+// A decoder-only model: embedding (+ learned position table), the calls of the execution order, the
+// final norm and the head (tied to the embedding) on the wanted rows only.
+class DecoderModel {
+public:
+    Tensor2 wte;                   // [V, D]
+    Tensor2 wpe;                   // [P, D] or empty
+    std::vector<std::unique_ptr<Block>> layers;
+    std::vector<LayerCall> order;
+    std::unique_ptr<Norm> final_norm;
+    int dtype = BF16;
+
+    int vocab_size() const { return static_cast<int>(wte.rows); }
+    int hidden_size() const { return static_cast<int>(wte.cols); }
+    // Bytes of arena that a step of `tokens` tokens and `n_logits` wanted rows needs at most.
+    size_t workspace_bytes(int tokens, int n_logits) const;
+    // Runs the step; fp32 logits [n_logits, V] into `logits` (untouched if no logits are wanted).
+    void forward(const StepView& step, const std::vector<CacheView>& caches, Arena& arena, const Tensor2& logits,
+                 hipStream_t s) const;
+};
+
+}  // namespace minillm

@@ -54,6 +54,8 @@ class StepContext:
     max_ctx_len: int
     n_single: int = 0             # the first n_single sequences bring one token each (decoded tokens stand
                                   #     first in a scheduler's mixed step); kernels may treat them apart
+    static_buffers: bool = False  # the step runs from buffers whose addresses never change (a captured
+                                  #     graph replays it): its temporaries must stay where they are too
     # host copies, for parts that plan on the host
     h_cu_q: np.ndarray = None
     h_starts: np.ndarray = None
@@ -140,6 +142,10 @@ class ModelRunner:
             head_dim = max((getattr(m, "head_dim", 0) for m in self._mixers()), default=0)
             ops.reserve_scratch(self.device, rows, model.vocab_size, n_heads, head_dim)
             ops.on_scratch_growth(self._drop_graphs)
+            native = model.native() if getattr(model, "use_native", False) and hasattr(model, "native") else None
+            if native is not None:
+                native.reserve_static(rows)
+                native.on_static_arena_replaced = weakref.WeakMethod(self._drop_graphs)
 
     def _mixers(self):
         return [getattr(layer, "mixer", None) for layer in getattr(self.model, "layers", [])]
@@ -336,6 +342,9 @@ class ModelRunner:
         greedy = temperatures is None or all(t <= 0 for t in temperatures)
         bucket = B if B <= 8 else -(-B // 8) * 8
         self._room_for_tokens(bucket)
+        if self.use_graphs:
+            from ..kernels import ops
+            ops.notify_scratch_growth()           # a scratch buffer replaced since the last step: graphs are dropped
         key = (bucket, greedy)
         g = self._graphs.get(key)
         if g is None:
@@ -397,6 +406,7 @@ class DecodeGraph:
         self.d_float = self.dev_ints[self.n_ctx_ints + B:].view(torch.float32).view(2, B)
         self.ctx = runner._context(self.dev_ints, self.offs, B, B, B, self.max_blocks, 1,
                                    self.max_blocks[0] * runner.page_size if self.max_blocks else 1, n_single=B)
+        self.ctx.static_buffers = True
         self.out = runner._tok_out[:B]
         # two host buffers in turn: one may still be unread when the next step's copy is queued
         self.h_out = [torch.zeros(B, dtype=torch.int32, pin_memory=on_gpu) for _ in range(2)]

@@ -1,16 +1,16 @@
-"""The engine's device operations: thin, checked wrappers over the HIP kernels.
+"""The engine's device operations, seen from Python: a thin face over the native ops
+(csrc/engine/ops.cc), which check shapes, strides and dtypes, choose among the kernels of an
+operation by size and launch on the current HIP stream (so the calls can be captured in a HIP
+graph). The native parts call the same functions directly; this face serves the tests and parts
+written in Python.
 
-Every op takes torch tensors that live on the GPU, checks on the host that shapes,
-strides and dtypes match what the kernel and its grid assume, and launches on the
-current HIP stream (so the calls can be captured in a HIP graph). There is no CPU
-path: a tensor that is not on the GPU, or a kernel library that cannot be built and
-loaded, raises.
-
-Parts look ops up as ``ops.<name>`` at call time.
+There is no CPU path: a tensor that is not on the GPU, or a library that cannot be built and
+loaded, raises. Parts look ops up as ``ops.<name>`` at call time.
 """
 from __future__ import annotations
 
 import ctypes
+import weakref
 from typing import Optional
 
 import torch
@@ -19,16 +19,78 @@ from ..build import load_library
 
 EPILOGUES = {"store": 0, "gelu_tanh": 1, "gelu_erf": 2, "add_residual": 3, "store_f32": 4}
 _DT = {torch.float32: 0, torch.bfloat16: 1}
+_DT_BACK = {0: torch.float32, 1: torch.bfloat16}
 
 
 class KernelError(RuntimeError):
     pass
 
 
-def _dt(t: torch.Tensor) -> int:
-    if t.dtype not in _DT:
-        raise KernelError(f"unsupported dtype {t.dtype} (float32 or bfloat16)")
-    return _DT[t.dtype]
+# -- the native structures (csrc/engine/ops.h) ---------------------------------------------------
+_vp, _i, _i64, _f = ctypes.c_void_p, ctypes.c_int, ctypes.c_int64, ctypes.c_float
+
+
+class Tensor2(ctypes.Structure):
+    _fields_ = [("data", _vp), ("dtype", _i), ("rows", _i64), ("cols", _i64), ("stride", _i64)]
+
+
+class KvScatterC(ctypes.Structure):
+    _fields_ = [("slots", _vp), ("k_pages", Tensor2), ("v_pages", Tensor2), ("q_cols", _i)]
+
+
+class AttentionSplitsC(ctypes.Structure):
+    _fields_ = [("ws", _vp), ("n_tokens", _i), ("n_heads", _i), ("head_dim", _i), ("nsplit", _i), ("dtype", _i)]
+
+
+class AttentionArgsC(ctypes.Structure):
+    _fields_ = [("q", Tensor2), ("q_col", _i), ("n_heads", _i), ("n_kv_heads", _i), ("head_dim", _i),
+                ("k_pages", Tensor2), ("v_pages", Tensor2), ("page_size", _i), ("block_tables", _vp),
+                ("n_seqs", _i), ("max_blocks", _i), ("token_seq", _vp), ("positions", _vp), ("scale", _f),
+                ("window", _i), ("out", Tensor2), ("cu_q", _vp), ("ctx_len", _vp), ("max_q_len", _i),
+                ("max_ctx_len", _i), ("append", _i), ("k_col", _i), ("v_col", _i), ("slots", _vp),
+                ("n_single", _i), ("may_split", _i)]
+
+
+_lib = None
+
+
+def engine_library():
+    """The native engine library, with its functions' types declared."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    lib = load_library("engine")
+    T2p, sz = ctypes.POINTER(Tensor2), ctypes.c_size_t
+    sigs = {
+        "mllm_last_error": (ctypes.c_char_p, []),
+        "mllm_reserve_scratch": (_i, [_i, _i, _i, _i]),
+        "mllm_scratch_generation": (ctypes.c_ulonglong, []),
+        "mllm_scratch_address": (_vp, [ctypes.c_char_p]),
+        "mllm_set_tuning": (_i, [ctypes.c_char_p, _i, _i]),
+        "mllm_op_embed": (_i, [_vp, _vp, T2p, T2p, T2p, _vp]),
+        "mllm_op_select_tokens": (_i, [_vp, _vp, _vp, _i, _i, _vp]),
+        "mllm_op_reset_state": (_i, [_vp, sz, _i, _vp, _vp, _i, _vp]),
+        "mllm_op_layernorm": (_i, [T2p, _vp, _vp, _f, T2p, _vp, _vp]),
+        "mllm_op_kv_append": (_i, [T2p, _i, _i, T2p, T2p, _vp, _vp]),
+        "mllm_op_linear": (_i, [T2p, T2p, _vp, T2p, _i, ctypes.POINTER(KvScatterC), _vp]),
+        "mllm_op_linear_from_splits": (_i, [ctypes.POINTER(AttentionSplitsC), T2p, _vp, T2p, _i, _vp, _vp]),
+        "mllm_op_merge_splits": (_i, [ctypes.POINTER(AttentionSplitsC), T2p, _vp]),
+        "mllm_op_ln_linear": (_i, [T2p, _vp, _vp, _f, T2p, _vp, T2p, _i, _vp, _vp, _vp]),
+        "mllm_op_paged_attention": (_i, [ctypes.POINTER(AttentionArgsC), ctypes.POINTER(AttentionSplitsC),
+                                         ctypes.POINTER(_i), _vp]),
+        "mllm_op_argmax": (_i, [T2p, _vp, _vp]),
+        "mllm_op_sample": (_i, [T2p, _vp, _vp, _vp, _vp]),
+    }
+    for name, (res, args) in sigs.items():
+        fn = getattr(lib, name)
+        fn.restype, fn.argtypes = res, args
+    _lib = lib
+    return lib
+
+
+def _ok(rc: int) -> None:
+    if rc != 0:
+        raise KernelError(engine_library().mllm_last_error().decode("utf-8", "replace"))
 
 
 def _gpu(*tensors: Optional[torch.Tensor]) -> None:
@@ -54,18 +116,23 @@ def _p(t: Optional[torch.Tensor]) -> ctypes.c_void_p:
     return ctypes.c_void_p(0 if t is None else t.data_ptr())
 
 
-def _check(rc: int, what: str) -> None:
-    if rc == 0:
-        return
-    if rc < 0:
-        raise KernelError(f"{what}: the kernel refuses these sizes (code {rc})")
-    raise KernelError(f"{what}: HIP error {rc} at launch")
+def _dt(t: torch.Tensor) -> int:
+    if t.dtype not in _DT:
+        raise KernelError(f"unsupported dtype {t.dtype} (float32 or bfloat16)")
+    return _DT[t.dtype]
 
 
-def _rows2d(t: torch.Tensor, name: str) -> None:
-    if t.dim() != 2 or t.stride(1) != 1:
+def t2(t: Optional[torch.Tensor], name: str = "tensor") -> Tensor2:
+    """A 2-D native view of a tensor (a 1-D tensor is one row)."""
+    if t is None:
+        return Tensor2(None, 0, 0, 0, 0)
+    if t.dim() == 1:
+        t = t.view(1, -1)
+    if t.dim() != 2 or (t.shape[1] > 1 and t.stride(1) != 1):
         raise KernelError(f"{name} must be 2-D with a contiguous last dimension, got shape "
                           f"{tuple(t.shape)} strides {t.stride()}")
+    stride = t.stride(0) if t.shape[0] > 1 else max(t.stride(0), t.shape[1])
+    return Tensor2(t.data_ptr(), _dt(t), t.shape[0], t.shape[1], stride)
 
 
 def _i32(t: torch.Tensor, name: str, n: Optional[int] = None) -> None:
@@ -75,7 +142,89 @@ def _i32(t: torch.Tensor, name: str, n: Optional[int] = None) -> None:
         raise KernelError(f"{name} has {t.numel()} entries, {n} needed")
 
 
-# ---------------------------------------------------------------------------------
+def _f32vec(t: Optional[torch.Tensor], name: str, n: int) -> None:
+    if t is not None and (t.dtype != torch.float32 or t.numel() != n or not t.is_contiguous()):
+        raise KernelError(f"{name} must be contiguous fp32 [{n}]")
+
+
+# -- scratch and tuning -----------------------------------------------------------------------------
+# Scratch buffers: device memory that a kernel needs beyond its inputs and outputs (argmax partial
+# results, the states of split decode attention, shared-tile sums). One set per device, owned by the
+# native side. A captured HIP graph keeps the raw address of the buffer it was captured with, so a
+# buffer is never replaced behind a graph's back: callers that capture graphs reserve room for their
+# largest launch first (``reserve_scratch``), and if a buffer must grow after all, everyone registered
+# with ``on_scratch_growth`` is told at the next ``notify_scratch_growth()``, and drops its graphs.
+_GROWTH_LISTENERS: list = []
+_seen_generation = 0
+
+
+def on_scratch_growth(method) -> None:
+    """Registers a bound method that is called (with no arguments) when a scratch buffer has been
+    replaced by a larger one (noticed by ``notify_scratch_growth``). Held weakly."""
+    _GROWTH_LISTENERS.append(weakref.WeakMethod(method))
+
+
+def notify_scratch_growth() -> bool:
+    """Tells the listeners if a scratch buffer has been replaced since the last call. Whoever replays
+    graphs calls this first."""
+    global _seen_generation
+    gen = engine_library().mllm_scratch_generation()
+    if gen == _seen_generation:
+        return False
+    _seen_generation = gen
+    alive = []
+    for ref in _GROWTH_LISTENERS:
+        fn = ref()
+        if fn is not None:
+            fn()
+            alive.append(ref)
+    _GROWTH_LISTENERS[:] = alive
+    return True
+
+
+def scratch_address(device, name: str) -> int:
+    """Address of a scratch buffer (0 if it does not exist yet): tests check that it stays put."""
+    with torch.cuda.device(torch.device(device)):
+        return engine_library().mllm_scratch_address(name.encode()) or 0
+
+
+def reserve_scratch(device, rows: int, vocab: int, n_heads: int = 0, head_dim: int = 0) -> None:
+    """Makes the scratch buffers large enough for ``rows`` sampled rows of ``vocab`` logits and for
+    decode attention over ``rows`` tokens of ``n_heads`` heads, so that no later launch up to these
+    sizes replaces them."""
+    if torch.device(device).type != "cuda":
+        return
+    with torch.cuda.device(torch.device(device)):
+        _ok(engine_library().mllm_reserve_scratch(int(rows), int(vocab), int(n_heads), int(head_dim)))
+
+
+# Tuning hooks: tests and tuning scripts set these module attributes; they reach the native side at the
+# next op that they concern.
+DECODE_SHAPE_OVERRIDE = None      # (nsplit, waves): forced launch shape of decode attention merged in its kernel
+DECODE_UNMERGED_SHAPE = None      # (nsplit, waves): forced shape of splits that the next product merges
+MERGE_MAX_ROWS = 16               # tokens whose attention splits a product merges while loading (one row block)
+LN_FUSE_MAX_ROWS = 32             # above this many rows the norm is faster as a kernel of its own (measured: 1-2 % of a
+                                  # decode step gained at 24 and 32 rows, 3 % lost at 64)
+_pushed_tuning = None
+
+
+def push_tuning() -> None:
+    """Hands the module's tuning values to the native side if they have changed."""
+    global _pushed_tuning
+    now = (DECODE_SHAPE_OVERRIDE, DECODE_UNMERGED_SHAPE, MERGE_MAX_ROWS, LN_FUSE_MAX_ROWS)
+    if now == _pushed_tuning:
+        return
+    lib = engine_library()
+    a, b = DECODE_SHAPE_OVERRIDE or (0, 0)
+    _ok(lib.mllm_set_tuning(b"decode_shape", int(a), int(b)))
+    a, b = DECODE_UNMERGED_SHAPE or (0, 0)
+    _ok(lib.mllm_set_tuning(b"unmerged_shape", int(a), int(b)))
+    _ok(lib.mllm_set_tuning(b"merge_max_rows", int(MERGE_MAX_ROWS), 0))
+    _ok(lib.mllm_set_tuning(b"ln_fuse_max_rows", int(LN_FUSE_MAX_ROWS), 0))
+    _pushed_tuning = now
+
+
+# -- the ops -----------------------------------------------------------------------------------------
 
 def embed(ids: torch.Tensor, positions: Optional[torch.Tensor], wte: torch.Tensor,
           wpe: Optional[torch.Tensor], out: torch.Tensor) -> torch.Tensor:
@@ -83,22 +232,16 @@ def embed(ids: torch.Tensor, positions: Optional[torch.Tensor], wte: torch.Tenso
     (the caller checks them on the host)."""
     _gpu(ids, positions, wte, wpe, out)
     T = ids.numel()
-    _rows2d(wte, "wte")
-    D = wte.shape[1]
     _i32(ids, "ids")
-    if not wte.is_contiguous():
-        raise KernelError("wte must be contiguous")
     if wpe is not None:
         if positions is None:
             raise KernelError("positions are needed with a position table")
         _i32(positions, "positions", T)
-        if wpe.dtype != wte.dtype or wpe.dim() != 2 or wpe.shape[1] != D or not wpe.is_contiguous():
-            raise KernelError("wpe must be contiguous [P, D] in wte's dtype")
-    if out.dtype != torch.float32 or out.shape != (T, D) or not out.is_contiguous():
-        raise KernelError(f"out must be contiguous fp32 [{T}, {D}]")
-    lib = load_library("elementwise")
-    _check(lib.mllm_embed(_p(ids), _p(positions if wpe is not None else None), _p(wte), _p(wpe), _p(out),
-                          T, D, _dt(wte), _stream()), "embed")
+    if out.dim() != 2 or out.shape[0] != T:
+        raise KernelError(f"out must be contiguous fp32 [{T}, {wte.shape[1]}]")
+    _ok(engine_library().mllm_op_embed(_p(ids), _p(positions), ctypes.byref(t2(wte, "wte")),
+                                       ctypes.byref(t2(wpe, "wpe")) if wpe is not None else None,
+                                       ctypes.byref(t2(out, "out")), _stream()))
     return out
 
 
@@ -110,8 +253,7 @@ def select_tokens(ids: torch.Tensor, src: torch.Tensor, prev: torch.Tensor) -> t
     _i32(ids, "ids")
     _i32(src, "src", n)
     _i32(prev, "prev")
-    lib = load_library("elementwise")
-    _check(lib.mllm_select_tokens(_p(ids), _p(src), _p(prev), n, prev.numel(), _stream()), "select_tokens")
+    _ok(engine_library().mllm_op_select_tokens(_p(ids), _p(src), _p(prev), n, prev.numel(), _stream()))
     return ids
 
 
@@ -125,40 +267,27 @@ def reset_state(state: torch.Tensor, slots: torch.Tensor, starts: torch.Tensor) 
     if not state.is_contiguous() or state.dim() < 1:
         raise KernelError("state must be contiguous [n_slots, ...]")
     slot_bytes = (state.numel() // max(state.shape[0], 1)) * state.element_size()
-    lib = load_library("elementwise")
-    rc = lib.mllm_reset_state(_p(state), ctypes.c_size_t(slot_bytes), state.shape[0], _p(slots), _p(starts), B,
-                              _stream())
-    if rc == -1:
-        raise KernelError(f"reset_state: a slot of {slot_bytes} bytes is no multiple of 4 bytes")
-    _check(rc, "reset_state")
+    _ok(engine_library().mllm_op_reset_state(_p(state), slot_bytes, state.shape[0], _p(slots), _p(starts), B,
+                                             _stream()))
 
 
 def layernorm(x: torch.Tensor, gamma: torch.Tensor, beta: Optional[torch.Tensor], eps: float,
               out: torch.Tensor, rows: Optional[torch.Tensor] = None) -> torch.Tensor:
     """out[i,:] = LayerNorm(x[rows[i] if rows else i,:]); statistics in fp32."""
     _gpu(x, gamma, beta, out, rows)
-    if x.dtype != torch.float32 or x.dim() != 2 or not x.is_contiguous():
+    if x.dim() != 2:
         raise KernelError("layernorm input must be contiguous fp32 [rows, D]")
     D = x.shape[1]
     n = rows.numel() if rows is not None else x.shape[0]
     if rows is not None:
         _i32(rows, "rows")
-    if gamma.dtype != torch.float32 or gamma.numel() != D or not gamma.is_contiguous():
-        raise KernelError(f"gamma must be fp32 [{D}]")
-    if beta is not None and (beta.dtype != torch.float32 or beta.numel() != D or not beta.is_contiguous()):
-        raise KernelError(f"beta must be fp32 [{D}]")
-    if out.shape != (n, D) or not out.is_contiguous():
+    _f32vec(gamma, "gamma", D)
+    _f32vec(beta, "beta", D)
+    if out.shape != (n, D):
         raise KernelError(f"out must be contiguous [{n}, {D}]")
-    lib = load_library("elementwise")
-    _check(lib.mllm_layernorm(_p(x), _p(rows), _p(gamma), _p(beta), _p(out), n, D, ctypes.c_float(eps),
-                              _dt(out), _stream()), "layernorm")
+    _ok(engine_library().mllm_op_layernorm(ctypes.byref(t2(x, "x")), _p(gamma), _p(beta), eps,
+                                           ctypes.byref(t2(out, "out")), _p(rows), _stream()))
     return out
-
-
-def _scatter_is_fused(dtype: torch.dtype, rows: int) -> bool:
-    """Whether the product kernel that runs for these rows writes a fused QKV product's keys and
-    values to the pages in its epilogue: the many-row bf16 kernel does."""
-    return dtype == torch.bfloat16 and rows > 64
 
 
 class AttentionSplits:
@@ -167,39 +296,20 @@ class AttentionSplits:
     lie in the attention scratch. ``linear`` takes it in place of a tensor and merges while it loads
     (``tensor()`` merges into an ordinary activation). Valid until the next attention launch."""
 
-    def __init__(self, ws: torch.Tensor, n_tokens: int, n_heads: int, head_dim: int, nsplit: int, dtype):
-        self.ws, self.n_tokens, self.n_heads, self.head_dim, self.nsplit = ws, n_tokens, n_heads, head_dim, nsplit
-        self.dtype, self.device = dtype, ws.device
-        self.shape = (n_tokens, n_heads * head_dim)
+    def __init__(self, c: AttentionSplitsC, device):
+        self.c = c
+        self.n_tokens, self.n_heads, self.head_dim, self.nsplit = c.n_tokens, c.n_heads, c.head_dim, c.nsplit
+        self.dtype, self.device = _DT_BACK[c.dtype], device
+        self.shape = (c.n_tokens, c.n_heads * c.head_dim)
 
     def tensor(self, out: Optional[torch.Tensor] = None) -> torch.Tensor:
         if out is None:
             out = torch.empty(self.shape, dtype=self.dtype, device=self.device)
-        lib = load_library("attention_decode")
-        _check(lib.mllm_merge_attention_splits(_p(self.ws), self.n_tokens, self.n_heads, self.head_dim, self.nsplit,
-                                               _p(out), out.stride(0), _DT[self.dtype], _stream()), "merge_splits")
+        _ok(engine_library().mllm_op_merge_splits(ctypes.byref(self.c), ctypes.byref(t2(out, "out")), _stream()))
         return out
 
 
-MERGE_MAX_ROWS = 16        # tokens whose attention splits a product merges while loading (one row block)
-MERGE_MAX_SPLITS = 4       # and the most splits per (token, head) pair it takes
-
-
-def _linear_from_splits(a: AttentionSplits, w, bias, out, epilogue: str) -> Optional[torch.Tensor]:
-    """The product fed by unmerged attention splits, or None if its kernel does not take these sizes."""
-    M, K = a.shape
-    N = w.shape[0]
-    lib = load_library("gemm_bf16")
-    ml = a.ws[M * a.n_heads * a.nsplit * a.head_dim:]
-    rc = lib.mllm_gemm_bf16_merged(_p(a.ws), _p(ml), a.nsplit, a.n_heads, a.head_dim, _p(w), w.stride(0), _p(bias),
-                                   _p(out), out.stride(0), M, N, EPILOGUES[epilogue], _stream())
-    if rc == -2:
-        return None
-    _check(rc, "linear (merging attention splits)")
-    return out
-
-
-def linear(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], out: torch.Tensor,
+def linear(a, w: torch.Tensor, bias: Optional[torch.Tensor], out: torch.Tensor,
            epilogue: str = "store", kv_scatter: Optional[tuple] = None) -> torch.Tensor:
     """out = epilogue(a @ w.T + bias). a: [M,K] (or the unmerged ``AttentionSplits`` of decode attention),
     w: [N,K] (same dtype), bias: fp32 [N].
@@ -214,90 +324,26 @@ def linear(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], out: 
     """
     splits = a if isinstance(a, AttentionSplits) else None
     _gpu(None if splits else a, w, bias, out)
-    if splits is None:
-        _rows2d(a, "a")
-    _rows2d(w, "w")
-    _rows2d(out, "out")
-    M, K = a.shape
-    N = w.shape[0]
-    if w.shape[1] != K or w.dtype != a.dtype:
-        raise KernelError(f"linear: a is {tuple(a.shape)} {a.dtype}, w is {tuple(w.shape)} {w.dtype}")
     if epilogue not in EPILOGUES:
         raise KernelError(f"unknown epilogue '{epilogue}'")
+    _f32vec(bias, "bias", w.shape[0])
+    lib = engine_library()
     if splits is not None:
-        want = torch.float32 if epilogue in ("add_residual", "store_f32") else a.dtype
-        ok = (kv_scatter is None and a.dtype == torch.bfloat16 and out.shape == (M, N) and out.dtype == want
-              and (bias is None or (bias.dtype == torch.float32 and bias.numel() == N and bias.is_contiguous()))
-              and w.stride(0) % 8 == 0 and w.data_ptr() % 16 == 0)
-        if ok and _linear_from_splits(a, w, bias, out, epilogue) is not None:
-            return out
-        a = splits.tensor()
-    want = torch.float32 if epilogue in ("add_residual", "store_f32") else a.dtype
-    if out.shape != (M, N) or out.dtype != want:
-        raise KernelError(f"linear({epilogue}): out must be [{M}, {N}] {want}, got {tuple(out.shape)} {out.dtype}")
-    if bias is not None and (bias.dtype != torch.float32 or bias.numel() != N or not bias.is_contiguous()):
-        raise KernelError(f"bias must be contiguous fp32 [{N}]")
-    mode = EPILOGUES[epilogue]
-    if kv_scatter is not None:
-        if epilogue != "store":
-            raise KernelError("linear: the key/value scatter needs the plain store")
-        if not _scatter_is_fused(a.dtype, M):
-            slots, k_pages, v_pages, q_cols = kv_scatter
-            kv_dim = k_pages.shape[1]
-            if N != q_cols + 2 * kv_dim:
-                raise KernelError(f"linear: {N} columns are not {q_cols} + 2 x {kv_dim}")
-            linear(a, w, bias, out, epilogue)
-            kv_append(out, q_cols, q_cols + kv_dim, kv_dim, k_pages, v_pages, slots)
-            return out
-    if a.dtype == torch.float32:
-        lib = load_library("gemm_f32")
-        rc = lib.mllm_gemm_f32(_p(a), a.stride(0), _p(w), w.stride(0), _p(bias), _p(out), out.stride(0),
-                               M, N, K, mode, _stream())
-    elif a.dtype == torch.bfloat16:
-        lib = load_library("gemm_bf16")
         if kv_scatter is not None:
-            slots, k_pages, v_pages, q_cols = kv_scatter
-            _gpu(slots, k_pages, v_pages)
-            kv_dim = k_pages.shape[1]
-            _i32(slots, "slots", M)
-            for name, pg in (("k_pages", k_pages), ("v_pages", v_pages)):
-                if pg.dim() != 2 or pg.shape[1] != kv_dim or not pg.is_contiguous() or pg.dtype != a.dtype:
-                    raise KernelError(f"{name} must be contiguous [rows, {kv_dim}] {a.dtype}")
-            if q_cols % 4 or kv_dim % 4 or N != q_cols + 2 * kv_dim:
-                raise KernelError(f"linear: {N} columns are not {q_cols} + 2 x {kv_dim} (multiples of 4)")
-            rc = lib.mllm_gemm_bf16_kv(_p(a), a.stride(0), _p(w), w.stride(0), _p(bias), _p(out), out.stride(0),
-                                       M, N, K, _p(slots), _p(k_pages), _p(v_pages), int(q_cols), int(kv_dim),
-                                       _stream())
-        else:
-            ws = _gemm_workspace(a.device) if M <= 256 else None
-            rc = lib.mllm_gemm_bf16(_p(a), a.stride(0), _p(w), w.stride(0), _p(bias), _p(out), out.stride(0),
-                                    M, N, K, mode, _p(ws), ctypes.c_size_t(GEMM_WORKSPACE_BYTES if M <= 256 else 0),
-                                    _stream())
-        if rc == -1:
-            raise KernelError(
-                f"linear(bf16): K={K} and the row strides ({a.stride(0)}, {w.stride(0)}) must be multiples "
-                "of 8 elements and the operands 16-byte aligned")
-    else:
-        raise KernelError(f"linear: unsupported dtype {a.dtype}")
-    _check(rc, "linear")
+            raise KernelError("linear: attention splits and a key/value scatter do not go together")
+        tmp = torch.empty(splits.shape, dtype=splits.dtype, device=splits.device)
+        _ok(lib.mllm_op_linear_from_splits(ctypes.byref(splits.c), ctypes.byref(t2(w, "w")), _p(bias),
+                                           ctypes.byref(t2(out, "out")), EPILOGUES[epilogue], _p(tmp), _stream()))
+        return out
+    kv = None
+    if kv_scatter is not None:
+        slots, k_pages, v_pages, q_cols = kv_scatter
+        _gpu(slots, k_pages, v_pages)
+        _i32(slots, "slots", a.shape[0])
+        kv = ctypes.byref(KvScatterC(slots.data_ptr(), t2(k_pages, "k_pages"), t2(v_pages, "v_pages"), int(q_cols)))
+    _ok(lib.mllm_op_linear(ctypes.byref(t2(a, "a")), ctypes.byref(t2(w, "w")), _p(bias), ctypes.byref(t2(out, "out")),
+                           EPILOGUES[epilogue], kv, _stream()))
     return out
-
-
-GEMM_WORKSPACE_BYTES = 16 * 1024 + 256 * 1024     # counters, then 1 KB per workgroup of a shared-tile launch
-_GEMM_WS = {}
-
-
-def _gemm_workspace(device) -> torch.Tensor:
-    """Scratch of the few-row products that share a tile among workgroups: zeroed once per device
-    (the kernel leaves its counters at zero); launches on one stream use it one after the other."""
-    ws = _GEMM_WS.get(device)
-    if ws is None:
-        ws = _GEMM_WS[device] = torch.zeros(GEMM_WORKSPACE_BYTES // 4, dtype=torch.int32, device=device)
-    return ws
-
-
-LN_FUSE_MAX_ROWS = 32      # above this many rows the norm is faster as a kernel of its own (measured: 1-2 % of a
-                           # decode step gained at 24 and 32 rows, 3 % lost at 64)
 
 
 def ln_linear(x: torch.Tensor, gamma: torch.Tensor, beta: Optional[torch.Tensor], eps: float,
@@ -307,42 +353,28 @@ def ln_linear(x: torch.Tensor, gamma: torch.Tensor, beta: Optional[torch.Tensor]
     ``rows`` (int32 [M]) row m of the input is x[rows[m]].
 
     For bfloat16 weights, at most 32 rows and fewer than 16384 columns the norm is fused into the
-    product (one kernel);
-    otherwise the norm and the product run one after the other. Same numerics either way:
-    statistics in fp32, the normalised rows rounded to w's dtype before the product.
+    product (one kernel); otherwise the norm and the product run one after the other. Same numerics
+    either way: statistics in fp32, the normalised rows rounded to w's dtype before the product.
     """
     _gpu(x, gamma, beta, w, bias, out, rows)
+    if epilogue not in EPILOGUES:
+        raise KernelError(f"unknown epilogue '{epilogue}'")
     K = x.shape[1]
     M = x.shape[0] if rows is None else rows.numel()
-    N = w.shape[0]
     if rows is not None:
         _i32(rows, "rows")
-    if (w.dtype == torch.bfloat16 and M <= LN_FUSE_MAX_ROWS and x.dtype == torch.float32 and x.is_contiguous()
-            and gamma.data_ptr() % 16 == 0 and (beta is None or beta.data_ptr() % 16 == 0)):
-        _rows2d(w, "w")
-        _rows2d(out, "out")
-        if w.shape[1] != K or gamma.numel() != K or gamma.dtype != torch.float32:
-            raise KernelError(f"ln_linear: x is {tuple(x.shape)}, w is {tuple(w.shape)}, gamma {tuple(gamma.shape)}")
-        if beta is not None and (beta.numel() != K or beta.dtype != torch.float32):
-            raise KernelError("ln_linear: beta must be fp32 [K]")
-        if epilogue not in EPILOGUES:
-            raise KernelError(f"unknown epilogue '{epilogue}'")
-        want = torch.float32 if epilogue in ("add_residual", "store_f32") else w.dtype
-        if out.shape != (M, N) or out.dtype != want:
-            raise KernelError(f"ln_linear({epilogue}): out must be [{M}, {N}] {want}")
-        if bias is not None and (bias.dtype != torch.float32 or bias.numel() != N or not bias.is_contiguous()):
-            raise KernelError(f"bias must be contiguous fp32 [{N}]")
-        lib = load_library("gemm_bf16")
-        rc = lib.mllm_ln_gemm_bf16(_p(x), x.stride(0), _p(rows), _p(gamma), _p(beta), ctypes.c_float(eps), _p(w),
-                                   w.stride(0), _p(bias), _p(out), out.stride(0), M, N, K, EPILOGUES[epilogue],
-                                   _stream())
-        if rc == 0:
-            return out
-        if rc != -2:
-            _check(rc, "ln_linear")
-    h = torch.empty((M, K), dtype=w.dtype, device=x.device)
-    layernorm(x, gamma, beta, eps, h, rows)
-    return linear(h, w, bias, out, epilogue)
+    _f32vec(gamma, "gamma", K)
+    _f32vec(beta, "beta", K)
+    _f32vec(bias, "bias", w.shape[0])
+    if out.shape[0] != M:
+        raise KernelError(f"ln_linear({epilogue}): out must have {M} rows")
+    push_tuning()
+    # (room for the normalised rows, used when the fused kernel does not take these sizes)
+    tmp = torch.empty((M, K), dtype=w.dtype, device=x.device)
+    _ok(engine_library().mllm_op_ln_linear(ctypes.byref(t2(x, "x")), _p(gamma), _p(beta), eps, ctypes.byref(t2(w, "w")),
+                                           _p(bias), ctypes.byref(t2(out, "out")), EPILOGUES[epilogue], _p(rows),
+                                           _p(tmp), _stream()))
+    return out
 
 
 def kv_append(src: torch.Tensor, k_col: int, v_col: int, kv_dim: int, k_pages: torch.Tensor,
@@ -350,17 +382,12 @@ def kv_append(src: torch.Tensor, k_col: int, v_col: int, kv_dim: int, k_pages: t
     """Copies columns [k_col, k_col+kv_dim) and [v_col, v_col+kv_dim) of each row of ``src``
     into row ``slots[t]`` of the key and value pages (slot < 0: skipped)."""
     _gpu(src, k_pages, v_pages, slots)
-    _rows2d(src, "src")
-    T = src.shape[0]
-    _i32(slots, "slots", T)
-    for name, pg in (("k_pages", k_pages), ("v_pages", v_pages)):
-        if pg.dim() != 2 or pg.shape[1] != kv_dim or not pg.is_contiguous() or pg.dtype != src.dtype:
-            raise KernelError(f"{name} must be contiguous [rows, {kv_dim}] {src.dtype}")
-    if max(k_col, v_col) + kv_dim > src.shape[1] or min(k_col, v_col) < 0:
-        raise KernelError("key/value columns lie outside the source rows")
-    lib = load_library("elementwise")
-    _check(lib.mllm_kv_append(_p(src), src.stride(0), k_col, v_col, _p(k_pages), _p(v_pages), kv_dim,
-                              _p(slots), T, _dt(src), _stream()), "kv_append")
+    _i32(slots, "slots", src.shape[0])
+    if k_pages.dim() != 2 or k_pages.shape[1] != kv_dim:
+        raise KernelError(f"k_pages must be contiguous [rows, {kv_dim}] {src.dtype}")
+    _ok(engine_library().mllm_op_kv_append(ctypes.byref(t2(src, "src")), int(k_col), int(v_col),
+                                           ctypes.byref(t2(k_pages, "k_pages")), ctypes.byref(t2(v_pages, "v_pages")),
+                                           _p(slots), _stream()))
 
 
 def paged_attention(q: torch.Tensor, q_col: int, n_heads: int, n_kv_heads: int, head_dim: int,
@@ -388,230 +415,45 @@ def paged_attention(q: torch.Tensor, q_col: int, n_heads: int, n_kv_heads: int, 
     in place of ``out`` (returned when a few single tokens' keys were split over several workgroups
     each; ``out`` is then left unwritten).
     """
-    _gpu(q, k_pages, v_pages, block_tables, token_seq, positions, out)
-    _rows2d(q, "q")
-    _rows2d(out, "out")
+    _gpu(q, k_pages, v_pages, block_tables, token_seq, positions, out, cu_q, ctx_len)
     T = q.shape[0]
-    kv_dim = n_kv_heads * head_dim
-    if q_col < 0 or q_col + n_heads * head_dim > q.shape[1]:
-        raise KernelError("query columns lie outside q's rows")
-    if out.shape[0] != T or out.shape[1] != n_heads * head_dim or out.dtype != q.dtype:
-        raise KernelError(f"out must be [{T}, {n_heads * head_dim}] {q.dtype}")
-    for name, pg in (("k_pages", k_pages), ("v_pages", v_pages)):
-        if pg.dim() != 2 or pg.shape[1] != kv_dim or not pg.is_contiguous() or pg.dtype != q.dtype:
-            raise KernelError(f"{name} must be contiguous [rows, {kv_dim}] {q.dtype}")
-    if k_pages.shape[0] % page_size != 0:
-        raise KernelError("the page pool is not a whole number of pages")
     if block_tables.dim() != 2 or block_tables.dtype != torch.int32 or not block_tables.is_contiguous():
         raise KernelError("block_tables must be contiguous int32 [B, max_blocks]")
+    B = block_tables.shape[0]
     _i32(token_seq, "token_seq", T)
     _i32(positions, "positions", T)
-    if head_dim % 8 != 0 or head_dim > 256:
-        raise KernelError(f"head_dim={head_dim} is not supported (multiples of 8 up to 256)")
-    if n_heads % n_kv_heads != 0:
-        raise KernelError(f"n_heads={n_heads} is not a multiple of n_kv_heads={n_kv_heads}")
-    esz = q.element_size()
-    if (q.stride(0) * esz) % 16 or (q_col * esz) % 16 or (head_dim * esz) % 16 or q.data_ptr() % 16:
-        raise KernelError("query rows and heads must be 16-byte aligned")
-    lpk = head_dim * esz // 16
-    decode = (max_q_len == 1 and lpk >= 2 and (lpk & (lpk - 1)) == 0
-              and page_size & (page_size - 1) == 0 and block_tables.shape[1] <= 4096)
-    k_col = v_col = 0
-    slots = None
+    if cu_q is not None:
+        _i32(cu_q, "cu_q", B + 1)
+    if ctx_len is not None:
+        _i32(ctx_len, "ctx_len", B)
+    a = AttentionArgsC()
+    a.q, a.q_col, a.n_heads, a.n_kv_heads, a.head_dim = t2(q, "q"), int(q_col), int(n_heads), int(n_kv_heads), int(head_dim)
+    a.k_pages, a.v_pages, a.page_size = t2(k_pages, "k_pages"), t2(v_pages, "v_pages"), int(page_size)
+    a.block_tables, a.n_seqs, a.max_blocks = block_tables.data_ptr(), B, block_tables.shape[1]
+    a.token_seq, a.positions, a.scale, a.window = token_seq.data_ptr(), positions.data_ptr(), float(scale), int(window or 0)
+    a.out = t2(out, "out")
+    a.cu_q = cu_q.data_ptr() if cu_q is not None else None
+    a.ctx_len = ctx_len.data_ptr() if ctx_len is not None else None
+    a.max_q_len, a.max_ctx_len = int(max_q_len), int(max_ctx_len)
     if append is not None:
         k_col, v_col, slots = append
-        if not decode:
-            kv_append(q, k_col, v_col, kv_dim, k_pages, v_pages, slots)
-            slots = None
-        else:
-            _i32(slots, "slots", T)
-            if max(k_col, v_col) + kv_dim > q.shape[1] or min(k_col, v_col) < 0 or (k_col * esz) % 16 or (v_col * esz) % 16:
-                raise KernelError("key/value columns lie outside q's rows or are not 16-byte aligned")
-    tiles_ok = (q.dtype == torch.bfloat16 and head_dim in (32, 64, 128) and max_q_len > 1
-                and cu_q is not None and ctx_len is not None
-                and page_size & (page_size - 1) == 0 and page_size >= head_dim // 16
-                and block_tables.shape[1] <= 2048)
-    if (tiles_ok and 0 < n_single < block_tables.shape[0] and lpk >= 2 and (lpk & (lpk - 1)) == 0
-            and block_tables.shape[1] <= 4096):
-        # a mixed step: the leading single tokens, then the portions, two launches over disjoint rows
-        # (every row's keys and values are in the pages by now)
-        paged_attention(q[:n_single], q_col, n_heads, n_kv_heads, head_dim, k_pages, v_pages, page_size,
-                        block_tables[:n_single], token_seq[:n_single], positions[:n_single], scale, window,
-                        out[:n_single], max_q_len=1, max_ctx_len=max_ctx_len, n_single=n_single)
-        B = block_tables.shape[0] - n_single
-        _i32(cu_q, "cu_q", block_tables.shape[0] + 1)
-        _i32(ctx_len, "ctx_len", block_tables.shape[0])
-        if out.data_ptr() % 16 or (out.stride(0) * esz) % 8:
-            raise KernelError("attention output rows must be 8-byte aligned")
-        lib = load_library("attention_prefill")
-        # (row numbers in cu_q are absolute, so q and out are passed whole and the per-sequence arrays from
-        # the first portion on)
-        _check(lib.mllm_prefill_attention_bf16(
-            _p(q), q.stride(0), q_col, _p(k_pages), _p(v_pages), kv_dim, _p(block_tables[n_single:]),
-            block_tables.shape[1], _p(cu_q[n_single:]), _p(ctx_len[n_single:]), B, (T - n_single) // 64 + B,
-            n_heads, n_kv_heads, head_dim, page_size, ctypes.c_float(scale), int(window or 0), _p(out),
-            out.stride(0), _stream()), "prefill_attention")
-        return out
-    if decode:
-        # every query is a single decoded token: split its keys over workgroups
-        pairs = T * n_heads
-        unmerged = (may_split and q.dtype == torch.bfloat16 and T <= MERGE_MAX_ROWS and head_dim % 8 == 0
-                    and DECODE_SHAPE_OVERRIDE is None)
-        nsplit, waves = _decode_launch_shape(pairs, max_ctx_len, unmerged)
-        unmerged = unmerged and nsplit > 1
-        ws, counters = _decode_workspace(q.device, pairs, nsplit, head_dim)
-        lib = load_library("attention_decode")
-        # every sequence of the batch brings one token (the caller says so): token t is sequence t, and the
-        # kernel need not load that
-        seq_of_token = None if n_single == T == block_tables.shape[0] else token_seq
-        _check(lib.mllm_decode_attention(
-            _p(q), q.stride(0), q_col, _p(k_pages), _p(v_pages), kv_dim, _p(block_tables), block_tables.shape[1],
-            _p(seq_of_token), _p(positions), T, n_heads, n_kv_heads, head_dim, page_size, ctypes.c_float(scale),
-            int(window or 0), nsplit, waves, _p(out), out.stride(0), _p(ws), _p(counters), k_col, v_col, _p(slots),
-            1 if unmerged else 0, _dt(q), _stream()),
-            "decode_attention")
-        if unmerged:
-            return AttentionSplits(ws, T, n_heads, head_dim, nsplit, q.dtype)
-        return out
-    if tiles_ok:
-        # prompt portions: tiles of 64 queries on the matrix cores
-        B = block_tables.shape[0]
-        _i32(cu_q, "cu_q", B + 1)
-        _i32(ctx_len, "ctx_len", B)
-        if out.data_ptr() % 16 or (out.stride(0) * esz) % 8:
-            raise KernelError("attention output rows must be 8-byte aligned")
-        lib = load_library("attention_prefill")
-        _check(lib.mllm_prefill_attention_bf16(
-            _p(q), q.stride(0), q_col, _p(k_pages), _p(v_pages), kv_dim, _p(block_tables), block_tables.shape[1],
-            _p(cu_q), _p(ctx_len), B, T // 64 + B, n_heads, n_kv_heads, head_dim, page_size,
-            ctypes.c_float(scale), int(window or 0), _p(out), out.stride(0), _stream()), "prefill_attention")
-        return out
-    lib = load_library("attention")
-    _check(lib.mllm_paged_attention_generic(
-        _p(q), q.stride(0), q_col, _p(k_pages), _p(v_pages), kv_dim, _p(block_tables), block_tables.shape[1],
-        _p(token_seq), _p(positions), T, n_heads, n_kv_heads, head_dim, page_size, ctypes.c_float(scale),
-        int(window or 0), _p(out), out.stride(0), _dt(q), _stream()), "paged_attention")
+        _gpu(slots)
+        _i32(slots, "slots", T)
+        a.append, a.k_col, a.v_col, a.slots = 1, int(k_col), int(v_col), slots.data_ptr()
+    a.n_single, a.may_split = int(n_single), 1 if may_split else 0
+    push_tuning()
+    splits, unmerged = AttentionSplitsC(), _i(0)
+    _ok(engine_library().mllm_op_paged_attention(ctypes.byref(a), ctypes.byref(splits), ctypes.byref(unmerged), _stream()))
+    if unmerged.value:
+        return AttentionSplits(splits, q.device)
     return out
-
-
-DECODE_SHAPE_OVERRIDE = None      # (nsplit, waves): set by tests of the split path and by tuning scripts
-DECODE_MAX_SPLIT = 8              # most workgroups that share one (token, head) pair's keys
-
-
-# ---------------------------------------------------------------------------------
-# Scratch buffers: device memory that a kernel needs beyond its inputs and outputs
-# (argmax partial results, partial outputs and counters of the split decode attention).
-# One set per device. A captured HIP graph keeps the raw address of the buffer it was
-# captured with, so a buffer is never replaced behind a graph's back: callers that
-# capture graphs reserve room for their largest launch first (``reserve_scratch``),
-# and if a buffer must grow after all, everyone registered with ``on_scratch_growth``
-# is told, and drops the graphs it holds.
-# ---------------------------------------------------------------------------------
-_SCRATCH: dict = {}               # (device, name) -> tensor
-_GROWTH_LISTENERS: list = []      # weak references to bound methods
-
-
-def on_scratch_growth(method) -> None:
-    """Registers a bound method that is called (with no arguments) whenever a scratch buffer has
-    been replaced by a larger one. Held weakly."""
-    import weakref
-    _GROWTH_LISTENERS.append(weakref.WeakMethod(method))
-
-
-def _scratch(device, name: str, numel: int, dtype: torch.dtype, zero: bool = False) -> torch.Tensor:
-    key = (torch.device(device), name)
-    t = _SCRATCH.get(key)
-    if t is not None and t.numel() >= numel:
-        return t
-    grown = (torch.zeros if zero else torch.empty)(numel, dtype=dtype, device=device)
-    _SCRATCH[key] = grown
-    if t is not None:
-        alive = []
-        for ref in _GROWTH_LISTENERS:
-            fn = ref()
-            if fn is not None:
-                fn()
-                alive.append(ref)
-        _GROWTH_LISTENERS[:] = alive
-    return grown
-
-
-def scratch_address(device, name: str) -> int:
-    """Address of a scratch buffer (0 if it does not exist yet): tests check that it stays put."""
-    t = _SCRATCH.get((torch.device(device), name))
-    return 0 if t is None else t.data_ptr()
-
-
-def reserve_scratch(device, rows: int, vocab: int, n_heads: int = 0, head_dim: int = 0) -> None:
-    """Makes the scratch buffers large enough for ``rows`` sampled rows of ``vocab`` logits and for
-    decode attention over ``rows`` tokens of ``n_heads`` heads, so that no later launch up to these
-    sizes replaces them."""
-    if torch.device(device).type != "cuda":
-        return
-    chunks = load_library("sampling").mllm_argmax_chunks(int(vocab))
-    _argmax_scratch(device, rows * chunks)
-    if n_heads and head_dim:
-        _decode_workspace(device, rows * n_heads, DECODE_MAX_SPLIT, head_dim)
-
-
-DECODE_UNMERGED_SHAPE = None     # (nsplit, waves) for splits that the next product merges: tuning scripts
-
-
-def _decode_launch_shape(pairs: int, max_ctx_len: int, unmerged: bool = False):
-    """How many workgroups share one (token, head) pair's keys, and wavefronts per workgroup."""
-    if DECODE_SHAPE_OVERRIDE is not None:
-        return DECODE_SHAPE_OVERRIDE
-    if unmerged:
-        # The splits cost nothing to merge here (the next product does it while it loads), so few pairs
-        # are spread over the compute units: a unit streams keys at 35 to 90 GB/s, and a pair's keys
-        # and values at 768 tokens are 200 KB. Every split keeps at least 128 keys.
-        if DECODE_UNMERGED_SHAPE is not None:
-            return DECODE_UNMERGED_SHAPE
-        # (measured at GPT-2 small sizes, 768 keys: 12 pairs x 4 splits of 4 wavefronts and 96 pairs x 2 splits
-        # of 8 wavefronts are the fastest shapes; more workgroups than compute units lose again)
-        nsplit = max(1, min(MERGE_MAX_SPLITS, 256 // max(pairs, 1), max_ctx_len // 128))
-        if nsplit > 1:
-            keys = -(-max_ctx_len // nsplit)
-            return nsplit, max(2, min(12, -(-keys // 64)))
-    # One workgroup per pair: merging splits (fences, a second merge) costs about 3 us, more than
-    # the parallelism gains below about 2,000 keys (measured at 12 to 96 pairs). Few pairs get more
-    # wavefronts each instead (measured: 12 are 1 to 3 % of a decode step faster than 8 up to 200
-    # pairs at GPT-2 small to XL sizes, 3 % slower from 384 pairs).
-    return 1, (4 if pairs >= 512 else 6 if pairs > 256 else 12)
-
-
-
-def _decode_workspace(device, pairs: int, nsplit: int, head_dim: int):
-    """Scratch of the split decode attention: partial outputs and a zeroed counter per
-    (token, head) (the kernel leaves the counters at zero). Launches on one stream use it one
-    after the other."""
-    if nsplit <= 1:
-        need_f = 1                      # one workgroup per pair exchanges nothing
-    else:
-        need_f = pairs * nsplit * (head_dim + 2)
-    ws = _scratch(device, "decode_partials", max(need_f, 1 << 16), torch.float32)
-    counters = _scratch(device, "decode_counters", max(pairs, 4096), torch.int32, zero=True)
-    return ws, counters
-
-
-def _argmax_scratch(device, n: int):
-    """Partial results of the first stage of argmax: a value and an index per (row, chunk)."""
-    return (_scratch(device, "argmax_values", max(n, 4096), torch.float32),
-            _scratch(device, "argmax_indices", max(n, 4096), torch.int32))
 
 
 def argmax(logits: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
     """out[i] = index of the largest logits[i,:], the lowest index on ties."""
     _gpu(logits, out)
-    _rows2d(logits, "logits")
-    if logits.dtype != torch.float32:
-        raise KernelError("logits must be fp32")
-    n, V = logits.shape
-    _i32(out, "out", n)
-    lib = load_library("sampling")
-    chunks = lib.mllm_argmax_chunks(V)
-    pv, pi = _argmax_scratch(logits.device, n * chunks)
-    _check(lib.mllm_argmax(_p(logits), logits.stride(0), n, V, _p(out), _p(pv), _p(pi), _stream()), "argmax")
+    _i32(out, "out", logits.shape[0])
+    _ok(engine_library().mllm_op_argmax(ctypes.byref(t2(logits, "logits")), _p(out), _stream()))
     return out
 
 
@@ -619,15 +461,10 @@ def sample(logits: torch.Tensor, temperature: torch.Tensor, u: torch.Tensor, out
     """Row i: temperature[i] <= 0 takes the argmax; otherwise draws from
     softmax(logits[i]/temperature[i]) by inverse CDF at u[i] in [0,1)."""
     _gpu(logits, temperature, u, out)
-    _rows2d(logits, "logits")
-    if logits.dtype != torch.float32:
-        raise KernelError("logits must be fp32")
-    n, V = logits.shape
+    n = logits.shape[0]
     for name, t in (("temperature", temperature), ("u", u)):
         if t.dtype != torch.float32 or t.numel() < n or not t.is_contiguous():
             raise KernelError(f"{name} must be contiguous fp32 [{n}]")
     _i32(out, "out", n)
-    lib = load_library("sampling")
-    _check(lib.mllm_sample(_p(logits), logits.stride(0), n, V, _p(temperature), _p(u), _p(out), _stream()),
-           "sample")
+    _ok(engine_library().mllm_op_sample(ctypes.byref(t2(logits, "logits")), _p(temperature), _p(u), _p(out), _stream()))
     return out

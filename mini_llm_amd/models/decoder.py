@@ -119,9 +119,24 @@ class DecoderModel:
         return {"weight_bytes": weight_bytes, "flops_per_token": flops, "flops_per_logits_row": head_flops,
                 "attention_flops_per_key": attn}
 
+    use_native = True        # False: always run through the parts' Python forward methods (tests compare the two)
+
+    def native(self):
+        """The native twin of this model (built at first use, once the weights are loaded), or None when
+        a part has no native kind or the model is not on the GPU."""
+        if not hasattr(self, "_native"):
+            from .native import NativeModel
+            self._native = NativeModel.build(self)
+        return self._native
+
     def forward(self, ctx, cache) -> Optional[torch.Tensor]:
         """Runs the step's tokens through every call of the execution order and returns
-        fp32 logits ``[len(ctx.logit_rows), vocab]`` (None if no logits are wanted)."""
+        fp32 logits ``[len(ctx.logit_rows), vocab]`` (None if no logits are wanted). A model whose
+        parts are all native runs the whole step in one native call; otherwise the parts' Python
+        ``forward`` methods run one after the other (the same kernels either way)."""
+        native = self.native() if self.use_native else None
+        if native is not None:
+            return native.forward(ctx, cache)
         x = self.embedding.forward(ctx, self.position)
         for call in self.order:
             self.layers[call.layer].forward(x, ctx, cache.view(call.cache), call.write)

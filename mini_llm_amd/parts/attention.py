@@ -24,6 +24,13 @@ class CausalSelfAttention(Mixer):
     """
 
     accepts_normed_input = True
+    native_kind = "causal_attention"
+
+    def native_params(self):
+        return {"n_heads": self.n_heads, "n_kv_heads": self.n_kv_heads, "head_dim": self.head_dim,
+                "scale": self.scale, "window": self.window, "dtype": ops._DT[self.dtype],
+                "qkv.weight": self.qkv.weight, "qkv.bias": self.qkv.bias,
+                "out.weight": self.out.weight, "out.bias": self.out.bias}
 
     def __init__(self, hidden_size: int, n_heads: int, n_kv_heads: int, head_dim: int, scale: float,
                  window: Optional[int], bias: bool, weight_layout: str, names: Dict[str, str],

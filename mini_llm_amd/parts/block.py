@@ -12,6 +12,10 @@ class PreNormBlock(Block):
     sub-layer, on the residual stream (/root/reference/src/model/gpt2_model.cu:279-363)."""
 
     n_norms = 2
+    native_kind = "pre_norm"
+
+    def native_norms(self):
+        return [self.norm1, self.norm2]
 
     def __init__(self, mixer: Mixer, feed_forward: FeedForward, norms: Sequence[Norm],
                  norm_names: Sequence[str], dtype, device):

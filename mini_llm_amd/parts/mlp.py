@@ -19,6 +19,13 @@ class DenseMLP(FeedForward):
     (/root/reference/src/kernels/gelu.cu:7-9) and exact erf-GELU."""
 
     accepts_normed_input = True
+    native_kind = "dense_mlp"
+
+    def native_params(self):
+        from ..kernels import ops
+        return {"activation": self.activation, "dtype": ops._DT[self.dtype],
+                "up.weight": self.up.weight, "up.bias": self.up.bias,
+                "down.weight": self.down.weight, "down.bias": self.down.bias}
 
     def __init__(self, hidden_size: int, inner_size: int, activation: str, bias: bool, weight_layout: str,
                  names: Dict[str, str], dtype, device, init_std: float = 0.02, out_init_std: float = 0.02):

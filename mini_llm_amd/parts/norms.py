@@ -15,6 +15,8 @@ class LayerNorm(Norm):
     variance, statistics in fp32 (/root/reference/src/kernels/layernorm.cu:32-49).
     Input: the fp32 stream. Output: the compute dtype."""
 
+    native_kind = "layernorm"
+
     def __init__(self, size: int, eps: float, dtype, device, bias: bool = True):
         super().__init__(dtype, device)
         self.size, self.eps, self.has_bias = int(size), float(eps), bool(bias)
@@ -26,6 +28,9 @@ class LayerNorm(Norm):
         if self.has_bias:
             specs.append(ParamSpec(prefix + ".bias", (self.size,), "vector", self._set_beta, (0.0, 0.02)))
         return specs
+
+    def native_params(self):
+        return {"size": self.size, "eps": self.eps, "dtype": ops._DT[self.dtype], "gamma": self.gamma, "beta": self.beta}
 
     def _set_gamma(self, t):
         self.gamma = t

@@ -548,7 +548,7 @@ def test_decode_attention_splits_merged_by_the_next_product(ops, T, H, Hkv, dh, 
                                 append=(D, D + kv_dim, slots.to(DEV)), may_split=True)
     finally:
         ops.DECODE_UNMERGED_SHAPE = None
-    if shape is not None or (max(ctx) >= 256 and T * H <= 192):
+    if shape is not None or (max(ctx) >= 256 and T * H <= 128):
         assert isinstance(a, ops.AttentionSplits) and a.nsplit == (shape[0] if shape else a.nsplit) and a.nsplit > 1
     x = x0.clone().to(DEV)
     ops.linear(a, w.to(DEV), bias.to(DEV), x, "add_residual")

@@ -61,6 +61,25 @@ def test_schedule_families_match_plain_at_real_layer_sizes(real_model_dirs, name
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+def test_native_step_equals_the_parts_python_forward(tiny_model_dirs, dtype):
+    """A model whose parts are all native runs its step in one native call; with `use_native` off the
+    parts' Python forward methods run instead. Same kernels, same arguments: the logits are equal
+    bit for bit, and both match the plain implementation."""
+    reqs = rc.requests_for("b", seed=3, lengths=[40, 9, 100, 70])
+    steps, _ = ru.trace_mixed(reqs, seed=3)
+    outs = []
+    for native in (True, False):
+        runner = _runner(tiny_model_dirs["b"], "b", dtype, ru.peak_tokens(steps) // 8)
+        runner.model.use_native = native
+        assert (runner.model.native() is not None)
+        outs.append(ru.run_in_process(runner, steps))
+    assert outs[0].keys() == outs[1].keys()
+    for k in outs[0]:
+        assert np.array_equal(outs[0][k], outs[1][k]), k
+    rc.check_against_plain(tiny_model_dirs["b"], "b", reqs, steps, outs[0], dtype, label="native")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
 def test_schedules_agree_with_each_other(tiny_model_dirs, dtype):
     """Cutting, batching and page placement change the logits by rounding only."""
     reqs = rc.requests_for("b", seed=5, lengths=[25, 64, 124, 9])
