@@ -61,10 +61,21 @@ LIBRARIES: Dict[str, dict] = {
     # (host code only; it calls the kernel libraries' entry points)
     "engine": {
         "kind": "hiphost",
-        "sources": ["engine/ops.cc", "engine/parts.cc", "engine/engine_api.cc"],
-        "headers": ["engine/ops.h", "engine/parts.h", "engine/kernels.h"],
+        "sources": ["engine/ops.cc", "engine/parts.cc", "engine/json.cc", "engine/weights.cc", "engine/arch.cc",
+                    "engine/engine.cc", "engine/engine_api.cc"],
+        "headers": ["engine/ops.h", "engine/parts.h", "engine/kernels.h", "engine/json.h", "engine/weights.h",
+                    "engine/arch.h", "engine/engine.h", "runtime/cache_manager.h", "runtime/scheduler.h"],
         "needs": ["elementwise", "gemm_f32", "gemm_bf16", "attention", "attention_decode", "attention_prefill",
-                  "sampling"],
+                  "sampling", "runtime"],
+    },
+    # the command line: a program, not a library (mini_llm_amd/_lib/mini-llm; bin/mini-llm starts it)
+    "cli": {
+        "kind": "hiphost",
+        "program": "mini-llm",
+        "sources": ["engine/main.cc"],
+        "headers": ["engine/engine.h", "engine/arch.h", "engine/weights.h", "engine/parts.h", "engine/ops.h",
+                    "engine/json.h", "runtime/cache_manager.h", "runtime/scheduler.h"],
+        "needs": ["engine", "runtime"],
     },
 }
 
@@ -100,7 +111,8 @@ def _source_hash(name: str) -> str:
 
 
 def lib_path(name: str) -> str:
-    return os.path.join(LIB_DIR, f"libmllm_{name}.so")
+    program = LIBRARIES[name].get("program")
+    return os.path.join(LIB_DIR, program if program else f"libmllm_{name}.so")
 
 
 def is_current(name: str) -> bool:
@@ -109,6 +121,16 @@ def is_current(name: str) -> bool:
         return False
     with open(stamp) as f:
         return f.read().strip() == _source_hash(name)
+
+
+def needed_by(name: str) -> List[str]:
+    """Every library that `name` links against, directly or through another."""
+    out: List[str] = []
+    for dep in LIBRARIES[name].get("needs", []):
+        for d in needed_by(dep) + [dep]:
+            if d not in out:
+                out.append(d)
+    return out
 
 
 def _find(tool: str, extra: List[str]) -> str:
@@ -132,18 +154,18 @@ def build_library(name: str, verbose: bool = True) -> str:
         cc = _find("hipcc", ["/opt/rocm/bin"])
         cmd = [cc] + HIPCC_FLAGS
     elif spec["kind"] == "hiphost":
-        for dep in spec.get("needs", []):          # link against the kernel libraries beside it
+        for dep in needed_by(name):                # link against the libraries beside it
             if not is_current(dep):
                 build_library(dep, verbose)
         cc = _find("g++", ["/usr/bin"])
-        cmd = [cc] + HIPHOST_FLAGS
-        link = [f"-L{LIB_DIR}"] + [f"-lmllm_{d}" for d in spec.get("needs", [])] + \
+        cmd = [cc] + [f for f in HIPHOST_FLAGS if not (spec.get("program") and f in ("-shared",))]
+        link = [f"-L{LIB_DIR}"] + [f"-lmllm_{d}" for d in needed_by(name)] + \
                ["-L/opt/rocm/lib", "-lamdhip64", "-Wl,-rpath,$ORIGIN", "-Wl,-rpath,/opt/rocm/lib"]
     else:
         cc = _find("g++", ["/usr/bin"])
         cmd = [cc] + CXX_FLAGS
     # Compile to a private name, then rename: a concurrent process never sees a half-written file.
-    fd, tmp = tempfile.mkstemp(prefix=f".{name}.", suffix=".so", dir=LIB_DIR)
+    fd, tmp = tempfile.mkstemp(prefix=f".{name}.", suffix=".tmp" if spec.get("program") else ".so", dir=LIB_DIR)
     os.close(fd)
     cmd = cmd + [f"-I{os.path.join(CSRC, 'kernels')}", f"-I{os.path.join(CSRC, 'runtime')}",
                  f"-I{os.path.join(CSRC, 'engine')}"] + srcs + ["-o", tmp] + link

@@ -1,0 +1,67 @@
+// Architectures: one registry from the name in config.json to what builds the model. An
+// architecture says which tensors it expects (for the loader and the random-weights mode) and
+// assembles a DecoderModel from parts by its typed configuration; no size or constant that
+// config.json gives stands in code.
+#pragma once
+
+#include <functional>
+#include <map>
+#include <memory>
+#include <string>
+#include <vector>
+
+#include "json.h"
+#include "parts.h"
+#include "weights.h"
+
+namespace minillm {
+
+class ConfigError : public std::runtime_error {
+public:
+    explicit ConfigError(const std::string& what) : std::runtime_error(what) {}
+};
+
+// What a cache of the execution order asks of the cache manager.
+struct CacheNeed {
+    int kind = 1;                        // 1 keys and values in pages, 2 fixed-size state, 0 none
+    int n_kv_heads = 0, head_dim = 0, window = 0;
+    size_t state_bytes = 0;
+    int n_heads = 0;                     // query heads of the mixer that uses it (sizes the attention scratch)
+};
+
+// A model with its weights on the device.
+struct LoadedModel {
+    std::string architecture;
+    Json config;
+    int dtype = BF16;
+    DecoderModel model;
+    DeviceTensors store;
+    std::vector<CacheNeed> caches;       // per cache index of the execution order
+    int max_positions = 0;               // 0: unbounded
+    int eos_token_id = -1;               // -1: none
+};
+
+struct Architecture {
+    std::string name;
+    // the tensors a model of this configuration expects
+    std::function<std::vector<ParamSpec>(const Json& config)> param_specs;
+    // builds the model from its tensors (already on the device, by name)
+    std::function<void(const Json& config, const std::map<std::string, Tensor2>& tensors, int dtype, LoadedModel& out)> assemble;
+    std::vector<std::string> optional_prefixes;
+    std::function<bool(const std::string&)> ignored_tensor;
+};
+
+void register_architecture(const Architecture& a, const std::string& model_type = "");
+// by config.json: architectures[0], else model_type; unknown -> ConfigError listing the registered names
+const Architecture& architecture_of(const Json& config);
+std::vector<std::string> registered_architectures();
+
+Json read_config(const std::string& model_dir);
+// dtype: BF16 or F32
+std::unique_ptr<LoadedModel> load_model(const std::string& model_dir, int dtype);
+std::unique_ptr<LoadedModel> random_model(const Json& config, uint64_t seed, int dtype,
+                                          const std::string& weights_dtype = "bfloat16");
+// a preset by name: config/presets/<name>.json beside the package
+Json read_preset(const std::string& presets_dir, const std::string& name);
+
+}  // namespace minillm

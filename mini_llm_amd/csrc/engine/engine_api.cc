@@ -10,6 +10,7 @@
 #include <string>
 #include <vector>
 
+#include "engine.h"
 #include "ops.h"
 #include "parts.h"
 
@@ -174,5 +175,67 @@ int mllm_model_forward(const void* m, const StepView* step, const CacheView* cac
         static_cast<const DecoderModel*>(m)->forward(*step, cv, a, logits ? *logits : Tensor2(), s);
     });
 }
+
+// -- the engine (engine.h) ---------------------------------------------------------------------------
+// options: kv_block_size, total_kv_blocks, max_batch_num, max_tokens_per_step, prefill_chunk, overlap (0/1)
+static EngineOptions options_of(const int* o) {
+    EngineOptions e;
+    e.kv_block_size = o[0]; e.total_kv_blocks = o[1]; e.max_batch_num = o[2]; e.max_tokens_per_step = o[3];
+    e.prefill_chunk = o[4]; e.overlap = o[5] != 0;
+    return e;
+}
+void* mllm_engine_from_pretrained(const char* model_dir, int dtype, const int* options6) {
+    Engine* e = nullptr;
+    guarded([&] { e = Engine::from_pretrained(model_dir, dtype, options_of(options6)).release(); });
+    return e;
+}
+// config_json: the text of a config.json
+void* mllm_engine_from_random(const char* config_json, unsigned long long seed, int dtype, const int* options6) {
+    Engine* e = nullptr;
+    guarded([&] { e = Engine::from_random(Json::parse(config_json), seed, dtype, options_of(options6)).release(); });
+    return e;
+}
+void mllm_engine_destroy(void* e) { delete static_cast<Engine*>(e); }
+// Returns the request's id, or -1 (see mllm_last_error).
+long long mllm_engine_add_request(void* e, const int* tokens, int n, float temperature, unsigned long long seed,
+                                  int max_new_tokens, int ignore_eos, long long request_id) {
+    long long id = -1;
+    guarded([&] {
+        SamplingParams sp;
+        sp.temperature = temperature; sp.seed = seed; sp.max_new_tokens = max_new_tokens; sp.ignore_eos = ignore_eos != 0;
+        id = static_cast<Engine*>(e)->add_request(std::vector<int>(tokens, tokens + n), sp, request_id);
+    });
+    return id;
+}
+int mllm_engine_has_unfinished(void* e) { return static_cast<Engine*>(e)->has_unfinished() ? 1 : 0; }
+// One iteration. Up to `cap` outputs are written (ids, tokens, finished flags; a token of -1 is a failed
+// request, whose reason mllm_last_error holds); returns their number, or -1 on an error.
+int mllm_engine_step(void* e, long long* ids, int* tokens, int* finished, int cap) {
+    int n = -1;
+    guarded([&] {
+        const std::vector<RequestOutput> outs = static_cast<Engine*>(e)->step();
+        if (static_cast<int>(outs.size()) > cap) fail("more outputs (%zu) than room (%d)", outs.size(), cap);
+        n = 0;
+        for (const RequestOutput& o : outs) {
+            ids[n] = o.request_id; tokens[n] = o.token; finished[n] = o.finished ? 1 : 0;
+            if (o.token < 0) g_error = o.error;
+            ++n;
+        }
+    });
+    return n;
+}
+int mllm_engine_abort(void* e, long long id) { return guarded([&] { static_cast<Engine*>(e)->abort(id); }); }
+// names: steps, scheduled_tokens, prefill_tokens, decode_tokens, deferred_decodes, deferred_prefills, preemptions,
+// failures, finished, peak_pages_used, free_pages, total_pages (in this order)
+void mllm_engine_stats(void* e, long long* out12) {
+    const auto st = static_cast<Engine*>(e)->stats();
+    const char* names[12] = {"steps", "scheduled_tokens", "prefill_tokens", "decode_tokens", "deferred_decodes", "deferred_prefills",
+                             "preemptions", "failures", "finished", "peak_pages_used", "free_pages", "total_pages"};
+    for (int i = 0; i < 12; ++i) out12[i] = st.at(names[i]);
+}
+int mllm_engine_vocab_size(void* e) { return static_cast<Engine*>(e)->model().model.vocab_size(); }
+// weights bytes read once per step, flops per token... are the Python model's business; here: the cache's bytes per token
+unsigned long long mllm_engine_cache_bytes_per_token(void* e) { return static_cast<Engine*>(e)->runner().cache().bytes_per_token(); }
+void mllm_engine_synchronize(void* e) { guarded([&] { static_cast<Engine*>(e)->runner().synchronize(); }); }
 
 }  // extern "C"

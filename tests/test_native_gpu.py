@@ -1,0 +1,167 @@
+"""The native engine and its command line (csrc/engine: loader, runner, engine loop, main.cc) on the
+GPU: replay against the plain implementation, generation against the plain implementation and
+against the Python engine, which composes the same native parts."""
+import json
+import os
+import subprocess
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+import plain_gpt2
+import replay_cases as rc
+import replay_util as ru
+from conftest import TINY
+
+pytestmark = pytest.mark.gpu
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+CLI = os.path.join(ROOT, "bin", "mini-llm")
+
+
+def _run(args, stdin=None, timeout=300):
+    r = subprocess.run([sys.executable, CLI] + args, input=stdin, capture_output=True, text=True, timeout=timeout)
+    assert r.returncode == 0, r.stderr
+    return r.stdout
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["a", "b"])
+def test_native_replay_matches_plain(tiny_model_dirs, tmp_path, name, dtype):
+    """`mini-llm replay`: the native loader, cache storage and runner under a mixed trace with a pool made for
+    exactly what the trace needs, page size 16 (the pages are used again)."""
+    reqs = rc.requests_for(name, seed=4, lengths=rc.LENGTHS[name][:4] + [2, 64])
+    steps, _ = ru.trace_mixed(reqs, seed=4)
+    out_dir = str(tmp_path / "out")
+    cmd = [sys.executable, CLI, "replay", "--model", tiny_model_dirs[name], "--dtype", dtype, "--out", out_dir,
+           "--max-tokens", str(ru.peak_tokens(steps))]
+    p = subprocess.Popen(cmd, stdin=subprocess.PIPE, stdout=subprocess.PIPE, text=True)
+    try:
+        for s in steps:
+            p.stdin.write(json.dumps(s) + "\n")
+            p.stdin.flush()
+            assert p.stdout.readline().strip() == f"done {s['step']}"
+        p.stdin.close()
+        assert p.wait(timeout=120) == 0
+    finally:
+        if p.poll() is None:
+            p.kill()
+    out = {}
+    for s in steps:
+        n = sum(len(e["want"]) for e in s["entries"])
+        if n:
+            out[s["step"]] = np.fromfile(os.path.join(out_dir, f"{s['step']}.f32"), dtype="<f4").reshape(n, -1)
+    rc.check_against_plain(tiny_model_dirs[name], name, reqs, steps, out, dtype, label="native replay")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_native_generation_matches_plain_and_the_python_engine(tiny_model_dirs, dtype):
+    """Greedy and sampled generation through the native program: continuous batching of more requests than
+    a step holds, prompts cut into portions, so few pages that requests are deferred or preempted."""
+    from mini_llm_amd import Engine, EngineOptions, SamplingParams
+    cfg, w = plain_gpt2.read_model(tiny_model_dirs["b"])
+    g = torch.Generator().manual_seed(8)
+    prompts = [torch.randint(0, 999, (n,), generator=g).tolist() for n in (1, 9, 40, 100, 17, 33, 64)]
+    lines = "\n".join(" ".join(map(str, p)) for p in prompts) + "\n"
+    common = ["--model", tiny_model_dirs["b"], "--dtype", dtype, "--max-new-tokens", "12", "--ignore-eos",
+              "--kv-block-size", "8", "--total-kv-blocks", "34", "--max-batch-num", "4", "--max-tokens-per-step", "40",
+              "--prefill-chunk", "16"]
+    opts = EngineOptions(kv_block_size=8, total_kv_blocks=34, max_batch_num=4, max_tokens_per_step=40, prefill_chunk=16)
+    # greedy
+    out = _run(["generate"] + common, stdin=lines).strip().splitlines()
+    assert len(out) == len(prompts) and all(l.endswith("[DONE]") for l in out)
+    native = [[int(t) for t in l[:-6].split()] for l in out]
+    for p, o in zip(prompts, native):
+        assert len(o) == 12
+        if dtype == "float32":
+            assert o == plain_gpt2.greedy_generate(cfg, w, p, 12)
+        else:
+            ids = list(p)
+            for t in o:
+                row = plain_gpt2.forward_logits(cfg, w, ids)[-1]
+                assert row[t] >= row.max() - 0.05, (t, int(row.argmax()))
+                ids.append(t)
+    python = Engine.from_pretrained(tiny_model_dirs["b"], dtype=dtype, options=opts).generate(
+        prompts, SamplingParams(max_new_tokens=12, ignore_eos=True))
+    if dtype == "float32":
+        assert native == python
+    # temperature sampling: the same draws as the Python engine (seed + request index, counter hash per output)
+    out = _run(["generate"] + common + ["--temperature", "0.8", "--seed", "10", "--stats"], stdin=lines).strip().splitlines()
+    native = [[int(t) for t in l[:-6].split()] for l in out]
+    python = Engine.from_pretrained(tiny_model_dirs["b"], dtype=dtype, options=opts).generate(
+        prompts, [SamplingParams(temperature=0.8, seed=10 + i, max_new_tokens=12, ignore_eos=True) for i in range(len(prompts))])
+    if dtype == "float32":
+        assert native == python
+    else:
+        same = sum(a == b for x, y in zip(native, python) for a, b in zip(x, y))
+        assert same >= 0.85 * 12 * len(prompts)
+    assert len({tuple(o) for o in native}) == len(prompts)
+
+
+def test_native_engine_ends_requests_at_the_end_of_sequence_token(tiny_model_dirs):
+    """Without --ignore-eos a request ends with the model's end-of-sequence token (read one step late while the
+    next step is already in flight); --no-overlap waits for every step and must give the same lines."""
+    g = torch.Generator().manual_seed(2)
+    prompts = [torch.randint(0, 510, (n,), generator=g).tolist() for n in (7, 19, 30)]
+    lines = "\n".join(" ".join(map(str, p)) for p in prompts) + "\n"
+    base = ["generate", "--model", tiny_model_dirs["a"], "--dtype", "float32", "--max-new-tokens", "14", "--temperature", "1.5",
+            "--seed", "3", "--kv-block-size", "4", "--total-kv-blocks", "60", "--max-batch-num", "4"]
+    free = [[int(t) for t in l[:-6].split()] for l in _run(base + ["--ignore-eos"], stdin=lines).strip().splitlines()]
+    cfg = json.load(open(os.path.join(tiny_model_dirs["a"], "config.json")))
+    eos = cfg["eos_token_id"]
+    # make a copy of the model whose end-of-sequence token is one that request 0 samples
+    j = next(j for j in range(2, 14) if free[0][j] not in free[0][:j])
+    import shutil
+    import tempfile
+    with tempfile.TemporaryDirectory() as d:
+        shutil.copy(os.path.join(tiny_model_dirs["a"], "model.safetensors"), d)
+        json.dump(dict(cfg, eos_token_id=free[0][j]), open(os.path.join(d, "config.json"), "w"))
+        expect = [o[:o.index(free[0][j]) + 1] if free[0][j] in o else o for o in free]
+        for extra in ([], ["--no-overlap"]):
+            args = [a if a != tiny_model_dirs["a"] else d for a in base] + extra
+            got = [[int(t) for t in l[:-6].split()] for l in _run(args, stdin=lines).strip().splitlines()]
+            assert got == expect, extra
+    assert eos == 511 and len(expect[0]) == j + 1
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_native_engine_through_its_python_face(tiny_model_dirs, dtype):
+    """`NativeEngine` (the C ABI mllm_engine_*): the same tokens as the Python engine, request by request
+    through add_request/step, random weights made in memory equal to a written folder's, counters and pages
+    accounted for, an unknown token refused."""
+    from mini_llm_amd import Engine, EngineOptions, NativeEngine, SamplingParams
+    g = torch.Generator().manual_seed(12)
+    prompts = [torch.randint(0, 511, (n,), generator=g).tolist() for n in (5, 17, 33, 3, 60)]
+    o = EngineOptions(kv_block_size=4, total_kv_blocks=24, max_batch_num=3, max_tokens_per_step=24, prefill_chunk=16)
+    sp = [SamplingParams(temperature=0.0 if i % 2 else 0.9, seed=i, max_new_tokens=10, ignore_eos=True) for i in range(5)]
+    native = NativeEngine.from_pretrained(tiny_model_dirs["a"], dtype=dtype, options=o)
+    python = Engine.from_pretrained(tiny_model_dirs["a"], dtype=dtype, options=o)
+    a, b = native.generate(prompts, sp), python.generate(prompts, sp)
+    if dtype == "float32":
+        assert a == b
+    else:
+        assert sum(x == y for p, q in zip(a, b) for x, y in zip(p, q)) >= 0.85 * 50
+    st = native.stats()
+    assert st["free_pages"] == st["total_pages"] == 24 and st["finished"] == 5 and st["failures"] == 0
+    assert st["deferred_prefills"] + st["deferred_decodes"] + st["preemptions"] > 0
+    # step by step, with an abort in flight
+    r0 = native.add_request(prompts[0], SamplingParams(max_new_tokens=6, ignore_eos=True))
+    r1 = native.add_request(prompts[1], SamplingParams(max_new_tokens=9, ignore_eos=True))
+    seen = {r0: [], r1: []}
+    steps = 0
+    while native.has_unfinished():
+        for out in native.step():
+            seen[out.request_id].append((out.token, out.finished))
+        steps += 1
+        if steps == 4:
+            native.abort(r1)
+    assert [f for _, f in seen[r0]] == [False] * 5 + [True] and 0 < len(seen[r1]) < 9
+    assert native.stats()["free_pages"] == 24
+    with pytest.raises(ValueError, match="token ids"):
+        native.add_request([5, 512])
+    # random weights in memory: the same model as the folder the generator writes
+    from conftest import TINY_A
+    mem = NativeEngine.from_random(dict(TINY_A), seed=0, dtype=dtype, options=o)
+    greedy = SamplingParams(max_new_tokens=8, ignore_eos=True)
+    assert mem.generate(prompts[:3], greedy) == native.generate(prompts[:3], greedy)
