@@ -32,19 +32,22 @@ def small_config(n_layer, size="gpt2-small"):
                 activation_function="gelu_new", eos_token_id=50256, bos_token_id=50256)
 
 
-def decode_run(model_dir, dtype, batch, prompt_len, steps, warmup, cfg):
+def decode_run(model_dir, dtype, batch, prompt_len, steps, warmup, cfg, engine_kind="python"):
     """Decode steps of `batch` requests through the whole engine. Every prompt is fed in ONE step before
     the clock starts, so that all requests decode in lockstep from position prompt_len on. Returns
     tokens/s, mean and median seconds per step, the mean context length, and the bytes one step has to
     read (every weight once, and the cache of the live requests), taken from the model and the cache."""
     import torch
-    from mini_llm_amd import Engine, EngineOptions, SamplingParams
+    from mini_llm_amd import Engine, EngineOptions, NativeEngine, SamplingParams
     pages = batch * (cfg["n_positions"] // 16) + 16
-    engine = Engine.from_pretrained(model_dir, dtype=dtype, device="cuda:0",
-                                    options=EngineOptions(kv_block_size=16, total_kv_blocks=pages,
-                                                          max_batch_num=max(batch, 1),
-                                                          max_tokens_per_step=batch * prompt_len,
-                                                          prefill_chunk=prompt_len))
+    options = EngineOptions(kv_block_size=16, total_kv_blocks=pages, max_batch_num=max(batch, 1),
+                            max_tokens_per_step=batch * prompt_len, prefill_chunk=prompt_len)
+    native = engine_kind == "native"
+    if native:
+        engine = NativeEngine.from_pretrained(model_dir, dtype=dtype, options=options)
+    else:
+        engine = Engine.from_pretrained(model_dir, dtype=dtype, device="cuda:0", options=options)
+    sync = engine.synchronize if native else torch.cuda.synchronize
     g = torch.Generator().manual_seed(2)
     prompts = [torch.randint(0, cfg["vocab_size"], (prompt_len,), generator=g).tolist() for _ in range(batch)]
     # The workload generates up to 512 tokens per request (as many as the positions allow); the timed
@@ -58,10 +61,11 @@ def decode_run(model_dir, dtype, batch, prompt_len, steps, warmup, cfg):
         engine.add_request(p, params)
     # untimed: the prompts (one step), then the warm-up steps
     engine.step()
-    assert engine.scheduler.queue_length("decode") == batch, "the prompts did not fit one step"
+    if not native:
+        assert engine.scheduler.queue_length("decode") == batch, "the prompts did not fit one step"
     for _ in range(skip + warmup):
         engine.step()
-    torch.cuda.synchronize()
+    sync()
     ctx0 = prompt_len + 1 + skip + warmup
     per_step = []
     n_tok = 0
@@ -71,12 +75,17 @@ def decode_run(model_dir, dtype, batch, prompt_len, steps, warmup, cfg):
         t_now = time.perf_counter()
         per_step.append(t_now - t_prev)
         t_prev = t_now
-    torch.cuda.synchronize()
+    sync()
     dt = time.perf_counter() - t0
     assert n_tok == batch * steps, (n_tok, batch, steps)
     mean_ctx = ctx0 + (steps - 1) / 2.0
-    cost = engine.model.step_cost()
-    bytes_step = cost["weight_bytes"] + batch * mean_ctx * engine.runner.cache.bytes_per_token()
+    if native:
+        from mini_llm_amd.models import load_model
+        cost = load_model(model_dir, dtype, "cpu").step_cost()      # (the sizes of the same model, read off its parts)
+        per_token = engine.cache_bytes_per_token()
+    else:
+        cost, per_token = engine.model.step_cost(), engine.runner.cache.bytes_per_token()
+    bytes_step = cost["weight_bytes"] + batch * mean_ctx * per_token
     per_step.sort()
     p50 = per_step[len(per_step) // 2]
     del engine
@@ -115,25 +124,30 @@ def prefill_run(model_dir, dtype, cfg, n_req=2, n_tok=1024, reps=5):
     return T / dt, dt, flops
 
 
-def serving_run(model_dir, dtype, cfg, n_req, prompt_lo, prompt_hi, new_tokens, max_batch, chunk, pages, seed):
+def serving_run(model_dir, dtype, cfg, n_req, prompt_lo, prompt_hi, new_tokens, max_batch, chunk, pages, seed,
+                engine_kind="python"):
     """Continuous batching from a full queue: n_req requests with prompt lengths uniform in
     [prompt_lo, prompt_hi] and new_tokens generated each, prompts fed in portions of `chunk`, at most
     max_batch requests a step, `pages` pages of 16 tokens in the pool. Returns a dictionary of
     totals, times and the scheduler's counters."""
     import torch
-    from mini_llm_amd import Engine, EngineOptions, SamplingParams
-    engine = Engine.from_pretrained(model_dir, dtype=dtype, device="cuda:0",
-                                    options=EngineOptions(kv_block_size=16, total_kv_blocks=pages,
-                                                          max_batch_num=max_batch,
-                                                          max_tokens_per_step=max(2048, max_batch + chunk),
-                                                          prefill_chunk=chunk))
-    engine.warmup()      # untimed, as a server does before it takes requests: the decode graphs are captured
+    from mini_llm_amd import Engine, EngineOptions, NativeEngine, SamplingParams
+    options = EngineOptions(kv_block_size=16, total_kv_blocks=pages, max_batch_num=max_batch,
+                            max_tokens_per_step=max(2048, max_batch + chunk), prefill_chunk=chunk)
+    native = engine_kind == "native"
+    if native:
+        engine = NativeEngine.from_pretrained(model_dir, dtype=dtype, options=options)
+        engine.generate([[0]] * min(max_batch, 8), SamplingParams(max_new_tokens=2, ignore_eos=True))     # loads the kernels
+    else:
+        engine = Engine.from_pretrained(model_dir, dtype=dtype, device="cuda:0", options=options)
+        engine.warmup()      # untimed, as a server does before it takes requests: the decode graphs are captured
+    sync = engine.synchronize if native else torch.cuda.synchronize
     g = torch.Generator().manual_seed(seed)
     lens = torch.randint(prompt_lo, prompt_hi + 1, (n_req,), generator=g).tolist()
     params = SamplingParams(max_new_tokens=new_tokens, ignore_eos=True)
     for n in lens:
         engine.add_request(torch.randint(0, cfg["vocab_size"], (n,), generator=g).tolist(), params)
-    torch.cuda.synchronize()
+    sync()
     t0 = time.perf_counter()
     n_out = n_steps = failed = 0
     first = None
@@ -141,15 +155,15 @@ def serving_run(model_dir, dtype, cfg, n_req, prompt_lo, prompt_hi, new_tokens, 
         outs = engine.step()
         n_steps += 1
         if outs and first is None:
-            torch.cuda.synchronize()
+            sync()
             first = time.perf_counter() - t0
         n_out += sum(1 for o in outs if o.token >= 0)
         failed += sum(1 for o in outs if o.token < 0)
-    torch.cuda.synchronize()
+    sync()
     dt = time.perf_counter() - t0
     st = engine.stats()
     assert n_out == (n_req - failed) * new_tokens, (n_out, n_req, failed, new_tokens)
-    assert st["free_pages"] == pages and engine.runner.manager.check() == ""
+    assert st["free_pages"] == pages and (native or engine.runner.manager.check() == "")
     return {"seconds": dt, "generated": n_out, "prompt_tokens": sum(lens), "steps": n_steps,
             "first_token_s": first, "failed": failed, "counters": st}
 
@@ -164,7 +178,8 @@ def serving_main(args, cfg, model_dir):
     else:
         n_req, lo, hi, new, max_batch, chunk = 256, 512, 512, 512, 64, 512
         pages = int(0.6 * max_batch * ((hi + new + 15) // 16))
-    r = serving_run(model_dir, args.dtype, cfg, n_req, lo, hi, new, max_batch, chunk, pages, seed=7)
+    r = serving_run(model_dir, args.dtype, cfg, n_req, lo, hi, new, max_batch, chunk, pages, seed=7,
+                    engine_kind=args.engine)
     c = r["counters"]
     rec = {"metric": f"generated tok/s, {args.workload} workload ({args.size} sizes)",
            "value": round(r["generated"] / r["seconds"], 1), "unit": "tok/s", "n_gpus": 1,
@@ -175,6 +190,7 @@ def serving_main(args, cfg, model_dir):
            "config": {"model": args.size + "-sizes", "n_layer": cfg["n_layer"], "n_layer_full": SIZES[args.size][0],
                       "requests": n_req, "prompt_min": lo, "prompt_max": hi, "new_tokens": new,
                       "max_batch_num": max_batch, "prefill_chunk": chunk, "kv_blocks": pages, "kv_block_size": 16,
+                      "engine": args.engine,
                       "prompt_tokens": r["prompt_tokens"], "generated_tokens": r["generated"],
                       "total_tok_per_s": round((r["generated"] + r["prompt_tokens"]) / r["seconds"], 1),
                       "seconds": round(r["seconds"], 3), "first_token_ms": round(1e3 * (r["first_token_s"] or 0), 2),
@@ -198,6 +214,9 @@ def main():
     ap.add_argument("--prefill-only", action="store_true", help="measure only the prefill step (profiling)")
     ap.add_argument("--prefill-requests", type=int, default=2, help="with --prefill-only: prompts in the step")
     ap.add_argument("--prefill-tokens", type=int, default=1024, help="with --prefill-only: tokens of each prompt")
+    ap.add_argument("--engine", default="python", choices=["python", "native"],
+                    help="python: the engine composed in Python over the native step function, decode steps replayed "
+                         "as HIP graphs; native: the engine that is native from loader to sampler (bin/mini-llm's)")
     ap.add_argument("--peaks-only", action="store_true",
                     help="measure this GPU's streaming bandwidth and matrix-core rate and print them")
     ap.add_argument("--workload", default="decode", choices=["decode", "continuous", "kv-pressure"],
@@ -235,7 +254,7 @@ def main():
                               "frac": round(flops / pdt / MFMA_PEAK[args.dtype], 5)}))
             return 0
         tps, step_s, p50_s, mean_ctx, bytes_step = decode_run(d, args.dtype, args.batch, args.prompt_len, steps,
-                                                             warmup, cfg)
+                                                             warmup, cfg, args.engine)
         # The reference's own decode numbers at this workload (GPT-2 small, 512-token prompts; fp32 on a
         # TITAN V: /root/reference benchmark gpt2_decode_batch_sweep_512.csv:2-5), where it has one.
         reference_tps = {1: 116.9, 2: 223.1, 4: 438.6, 8: 854.4}.get(args.batch) \
@@ -254,6 +273,7 @@ def main():
                        "n_positions": cfg["n_positions"], "global_batch": args.batch,
                        "prompt_len": args.prompt_len, "seq_len": cfg["n_positions"],
                        "mean_context": round(mean_ctx, 1), "kv_block_size": 16, "parallelism": "single-gpu",
+                       "engine": args.engine,
                        "baseline": (f"{reference_tps} tok/s: the reference, fp32, TITAN V" if reference_tps else "none")},
             "roofline": {"bound": "hbm", "achieved": round(achieved / 1e9, 2), "peak": HBM_PEAK / 1e9,
                          "unit": "GB/s", "frac": round(achieved / HBM_PEAK, 5),
@@ -266,7 +286,7 @@ def main():
             points = {}
             for b in (1, 64):
                 s = min(steps, 128)
-                v = decode_run(d, args.dtype, b, args.prompt_len, s, min(warmup, 16), cfg)[0]
+                v = decode_run(d, args.dtype, b, args.prompt_len, s, min(warmup, 16), cfg, args.engine)[0]
                 points[f"decode_b{b}"] = round(v, 1)
             rec["points"] = points
             # what this GPU gives on the engine's own micro-benchmarks, beside the published peaks

@@ -48,6 +48,8 @@ LIBRARIES: Dict[str, dict] = {
         "sources": ["runtime/cache_manager.cc", "runtime/scheduler.cc", "runtime/c_api.cc"],
         "headers": ["runtime/cache_manager.h", "runtime/scheduler.h"],
     },
+    # plain C++ twins of the device operations: the oracle of the kernel tests (host only)
+    "ref": {"kind": "cxx", "sources": ["ref/ref_ops.cc"], "headers": []},
     "elementwise": {"kind": "hip", "sources": ["kernels/elementwise.hip"], "headers": ["kernels/common.h"]},
     "gemm_f32": {"kind": "hip", "sources": ["kernels/gemm_f32.hip"], "headers": ["kernels/common.h"]},
     "gemm_bf16": {"kind": "hip", "sources": ["kernels/gemm_bf16.hip"], "headers": ["kernels/common.h"]},

@@ -7,6 +7,7 @@ import pytest
 import torch
 
 import plain_ops
+import ref_ops
 
 pytestmark = pytest.mark.gpu
 
@@ -401,6 +402,10 @@ def _attention_case(ops, dtype, H, Hkv, dh, page, seqs, window, gen, boost=None,
                         max_q_len=max(n for _, n in seqs), max_ctx_len=max(ctx), n_single=n_single)
     ref = torch.zeros(T, H * dh, dtype=torch.float64)
     plain_ops.paged_attention(q, 8, H, Hkv, dh, kp, vp, page, tables, token_seq, positions, scale, window, ref)
+    if sum(c * n for c, (_, n) in zip(ctx, seqs)) * H * dh <= 2e8:
+        # the second oracle, the plain C++ twin, says the same
+        twin = ref_ops.paged_attention(q, 8, H, Hkv, dh, kp, vp, page, tables, token_seq, positions, scale, window)
+        assert (twin.double() - ref).abs().max() <= 2e-6
     return out.cpu().double(), ref
 
 
@@ -610,6 +615,58 @@ def test_paged_attention_window_edge(ops, dtype, window):
     g = torch.Generator().manual_seed(window)
     out, ref = _attention_case(ops, dtype, 4, 2, 32, 8, [(0, 80), (130, 1), (63, 3)], window, g)
     assert (out - ref).abs().max() <= _tol(dtype, 2)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_kernels_against_their_cpp_twins(ops, dtype):
+    """Every kernel against the plain C++ statement of its operation (csrc/ref/ref_ops.cc)."""
+    g = torch.Generator().manual_seed(11)
+    V, P, D, T = 301, 40, 200, 37
+    wte, wpe = _rand((V, D), dtype, g), _rand((P, D), dtype, g)
+    ids = torch.randint(0, V, (T,), generator=g, dtype=torch.int32)
+    pos = torch.randint(0, P, (T,), generator=g, dtype=torch.int32)
+    x = torch.empty(T, D, dtype=torch.float32, device=DEV)
+    ops.embed(ids.to(DEV), pos.to(DEV), wte.to(DEV), wpe.to(DEV), x)
+    assert (x.cpu() - ref_ops.embed(ids, pos, wte, wpe)).abs().max() <= 1e-6
+    gamma, beta = 1 + 0.1 * _rand((D,), torch.float32, g), 0.1 * _rand((D,), torch.float32, g)
+    h = torch.empty(T, D, dtype=dtype, device=DEV)
+    ops.layernorm(x, gamma.to(DEV), beta.to(DEV), 1e-5, h)
+    assert (h.cpu().float() - ref_ops.layernorm(x.cpu(), gamma, beta, 1e-5)).abs().max() <= _tol(dtype, 4)
+    for M, N, K, epi in [(T, 3 * D, D, "store"), (5, 72, D, "gelu_tanh"), (T, D, D, "add_residual"), (70, V, D, "store_f32"),
+                         (3, 90, D, "gelu_erf")]:
+        a, w, bias = _rand((M, K), dtype, g), _rand((N, K), dtype, g, std=K ** -0.5), 0.5 * _rand((N,), torch.float32, g)
+        f32_out = epi in ("add_residual", "store_f32")
+        out0 = _rand((M, N), torch.float32 if f32_out else dtype, g)
+        out = out0.clone().to(DEV)
+        ops.linear(a.to(DEV), w.to(DEV), bias.to(DEV), out, epi)
+        tol = 3e-5 if dtype == torch.float32 else (2e-5 + 2e-5 * math.sqrt(K) if f32_out else 4e-2)
+        assert (out.cpu().float() - ref_ops.linear(a, w, bias, out0, epi)).abs().max() <= tol, (M, N, K, epi)
+        if epi != "add_residual":
+            xs = _rand((M, K), torch.float32, g) + 0.3
+            out = out0.clone().to(DEV)
+            ops.ln_linear(xs.to(DEV), gamma.to(DEV), beta.to(DEV), 1e-5, w.to(DEV), bias.to(DEV), out, epi)
+            hn = ref_ops.layernorm(xs, gamma, beta, 1e-5).to(dtype)
+            # (a normalised value next to a bf16 rounding boundary may round the other way in the kernel)
+            tol_ln = 3e-5 if dtype == torch.float32 else (2e-2 if epi == "store_f32" else 4e-2)
+            assert (out.cpu().float() - ref_ops.linear(hn, w, bias, out0, epi)).abs().max() <= tol_ln, (M, N, K, epi)
+    H, Hkv, dh, page = 6, 2, 32, 8
+    src = _rand((9, 3 * Hkv * dh), dtype, g)
+    slots = torch.tensor([5, -1, 0, 9, 70, 71, 72, 3, 11], dtype=torch.int32)
+    kp, vp = torch.zeros(80, Hkv * dh, dtype=dtype, device=DEV), torch.zeros(80, Hkv * dh, dtype=dtype, device=DEV)
+    ops.kv_append(src.to(DEV), Hkv * dh, 2 * Hkv * dh, Hkv * dh, kp, vp, slots.to(DEV))
+    k2, v2 = torch.zeros(80, Hkv * dh), torch.zeros(80, Hkv * dh)
+    ref_ops.kv_append(src, Hkv * dh, 2 * Hkv * dh, Hkv * dh, k2, v2, slots)
+    assert torch.equal(kp.cpu().float(), k2) and torch.equal(vp.cpu().float(), v2)
+    _attention_case(ops, dtype, H, Hkv, dh, page, [(40, 1), (0, 70), (9, 5), (130, 1)], 0, g)   # (compares both oracles)
+    logits = _rand((6, 1000), torch.float32, g, std=2.0)
+    out = torch.empty(6, dtype=torch.int32, device=DEV)
+    ops.argmax(logits.to(DEV), out)
+    assert torch.equal(out.cpu(), ref_ops.argmax(logits))
+    temp, u = torch.tensor([0.0, 0.7, 1.0, 1.3, 0.2, 5.0]), torch.tensor([0.3, 0.0, 0.999, 0.5, 0.25, 0.75])
+    ops.sample(logits.to(DEV), temp.to(DEV), u.to(DEV), out)
+    got, want = out.cpu(), ref_ops.sample(logits, temp, u)
+    for r in range(6):                  # next to a boundary of the cumulative mass either neighbour is right
+        assert abs(int(got[r]) - int(want[r])) <= 1, (r, got, want)
 
 
 def test_argmax_ties_take_lowest_index(ops):
