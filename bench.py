@@ -186,7 +186,9 @@ def serving_main(args, cfg, model_dir):
            "steps": r["steps"], "warmup": 0, "ms_per_step": round(1e3 * r["seconds"] / r["steps"], 4),
            "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
            "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
-           "data": "synthetic (random weights seed 2, uniform random token ids and prompt lengths, seed 7); decode graphs captured before the clock starts",
+           "data": "synthetic (random weights seed 2, uniform random token ids and prompt lengths, seed 7)"
+                   + ("; decode graphs captured before the clock starts" if args.engine == "python" else
+                      "; a few two-token requests before the clock starts"),
            "config": {"model": args.size + "-sizes", "n_layer": cfg["n_layer"], "n_layer_full": SIZES[args.size][0],
                       "requests": n_req, "prompt_min": lo, "prompt_max": hi, "new_tokens": new,
                       "max_batch_num": max_batch, "prefill_chunk": chunk, "kv_blocks": pages, "kv_block_size": 16,

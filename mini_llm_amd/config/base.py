@@ -14,7 +14,7 @@ The engine needs three things from a configuration, whatever the architecture:
 from __future__ import annotations
 
 from dataclasses import dataclass, field
-from typing import Any, Dict, List, Optional, Tuple
+from typing import Any, Dict, List, Optional, Tuple, Union
 
 
 class ConfigError(ValueError):
@@ -30,13 +30,24 @@ class PartSpec:
 
 @dataclass(frozen=True)
 class LayerSpec:
-    """One layer: a block arrangement over a mixer, a feed-forward and norms."""
+    """One layer: a block arrangement over a mixer, a feed-forward and norms.
+
+    ``mixer`` or ``feed_forward`` may be None: the arrangement then leaves that sub-layer (and its norm)
+    out. ``norm`` is one spec, built once for every norm position of the block, or a tuple with one spec
+    for each position (a layer whose norms differ in kind or constants)."""
     block: str                      # registered block arrangement, e.g. "pre_norm"
-    mixer: PartSpec
-    feed_forward: PartSpec
-    norm: PartSpec                  # built once for every norm position of the block
+    mixer: Optional[PartSpec]
+    feed_forward: Optional[PartSpec]
+    norm: Union[PartSpec, Tuple[PartSpec, ...]]
     weight_prefix: str              # tensor-name prefix of this layer's weights
     norm_names: Tuple[str, ...] = ("ln_1", "ln_2")   # tensor names of the block's norms
+
+    def norm_at(self, position: int) -> PartSpec:
+        if isinstance(self.norm, PartSpec):
+            return self.norm
+        if position >= len(self.norm):
+            raise ConfigError(f"layer '{self.weight_prefix}' gives {len(self.norm)} norms; its block asks for more")
+        return self.norm[position]
 
 
 @dataclass(frozen=True)

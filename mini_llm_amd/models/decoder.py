@@ -152,12 +152,12 @@ def build_layers(specs: Sequence[LayerSpec], dtype, device, position: Optional[P
     for ls in specs:
         if ls.block not in BLOCKS:
             raise KeyError(f"unknown block arrangement '{ls.block}'; registered: {sorted(BLOCKS)}")
-        mixer = build_part(MIXERS, ls.mixer, dtype, device, "mixer")
+        mixer = None if ls.mixer is None else build_part(MIXERS, ls.mixer, dtype, device, "mixer")
         if position is not None and position.applies_in_mixer and hasattr(mixer, "position"):
             mixer.position = position        # an encoding that turns queries and keys inside the mixer
-        ff = build_part(FEED_FORWARDS, ls.feed_forward, dtype, device, "feed-forward")
+        ff = None if ls.feed_forward is None else build_part(FEED_FORWARDS, ls.feed_forward, dtype, device, "feed-forward")
         block_cls = BLOCKS[ls.block]
-        norms = [build_part(NORMS, ls.norm, dtype, device, "norm") for _ in range(block_cls.n_norms)]
+        norms = [build_part(NORMS, ls.norm_at(i), dtype, device, "norm") for i in range(block_cls.n_norms)]
         layers.append(block_cls(mixer=mixer, feed_forward=ff, norms=norms, norm_names=ls.norm_names,
                                 dtype=dtype, device=device))
         prefixes.append(ls.weight_prefix)

@@ -85,7 +85,8 @@ def _params(lib, values: Dict[str, object]):
 def _native_kind(part) -> Optional[str]:
     """The native kind a part's own class names (a subclass that changes the part's behaviour in Python
     does not inherit it)."""
-    return type(part).__dict__.get("native_kind")
+    kind = type(part).__dict__.get("native_kind")
+    return kind.fget(part) if isinstance(kind, property) else kind
 
 
 def _part(lib, category: str, part) -> Optional[int]:

@@ -9,10 +9,14 @@ from .base import Block, FeedForward, Mixer, Norm, NormedInput, ParamSpec, regis
 @register_block("pre_norm")
 class PreNormBlock(Block):
     """x += mixer(norm1(x)); x += feed_forward(norm2(x)): the norm stands before each
-    sub-layer, on the residual stream (/root/reference/src/model/gpt2_model.cu:279-363)."""
+    sub-layer, on the residual stream (/root/reference/src/model/gpt2_model.cu:279-363).
+    A layer built without a mixer or without a feed-forward leaves that half, and its norm, out."""
 
     n_norms = 2
-    native_kind = "pre_norm"
+
+    @property
+    def native_kind(self):
+        return "pre_norm" if self.mixer is not None and self.feed_forward is not None else None
 
     def native_norms(self):
         return [self.norm1, self.norm2]
@@ -27,14 +31,20 @@ class PreNormBlock(Block):
         self.norm_names = tuple(norm_names)
 
     def param_specs(self, prefix: str) -> List[ParamSpec]:
-        return (self.norm1.param_specs(prefix + self.norm_names[0]) + self.mixer.param_specs(prefix)
-                + self.norm2.param_specs(prefix + self.norm_names[1]) + self.feed_forward.param_specs(prefix))
+        specs: List[ParamSpec] = []
+        if self.mixer is not None:
+            specs += self.norm1.param_specs(prefix + self.norm_names[0]) + self.mixer.param_specs(prefix)
+        if self.feed_forward is not None:
+            specs += self.norm2.param_specs(prefix + self.norm_names[1]) + self.feed_forward.param_specs(prefix)
+        return specs
 
     def cache_spec(self):
-        return self.mixer.cache_spec()
+        return None if self.mixer is None else self.mixer.cache_spec()
 
     def forward(self, x, ctx, cache_view, write: bool = True) -> None:
-        h = NormedInput(self.norm1, x) if self.mixer.accepts_normed_input else self.norm1.forward(x)
-        self.mixer.forward(h, ctx, cache_view, x, write)
-        h = NormedInput(self.norm2, x) if self.feed_forward.accepts_normed_input else self.norm2.forward(x)
-        self.feed_forward.forward(h, ctx, x)
+        if self.mixer is not None:
+            h = NormedInput(self.norm1, x) if self.mixer.accepts_normed_input else self.norm1.forward(x)
+            self.mixer.forward(h, ctx, cache_view, x, write)
+        if self.feed_forward is not None:
+            h = NormedInput(self.norm2, x) if self.feed_forward.accepts_normed_input else self.norm2.forward(x)
+            self.feed_forward.forward(h, ctx, x)

@@ -30,9 +30,19 @@ def _rand(shape, dtype, gen, std=1.0):
 
 
 def test_loaded_libraries_are_in_tree(ops):
+    """After an op has run, the native code mapped into this process is the in-tree build: the engine
+    library and the kernel libraries it links, all from the package's own folder and nowhere else."""
+    import os
     from mini_llm_amd import build
-    lib = build.load_library("elementwise")
-    assert build.lib_path("elementwise").startswith(build.LIB_DIR) and lib is not None
+    out = torch.empty(2, dtype=torch.int32, device=DEV)
+    ops.argmax(torch.tensor([[0.0, 2.0, 1.0], [3.0, 2.0, 1.0]], device=DEV), out)
+    assert out.tolist() == [1, 0]
+    with open("/proc/self/maps") as f:
+        mapped = {line.split()[-1] for line in f if "libmllm_" in line}
+    names = {os.path.basename(m) for m in mapped}
+    for lib in ("engine", "elementwise", "gemm_bf16", "gemm_f32", "attention_decode", "attention_prefill", "sampling"):
+        assert os.path.basename(build.lib_path(lib)) in names, (lib, names)
+    assert all(os.path.dirname(os.path.realpath(m)) == os.path.realpath(build.LIB_DIR) for m in mapped), mapped
 
 
 def test_ops_refuse_cpu_tensors(ops):

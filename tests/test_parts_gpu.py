@@ -137,7 +137,9 @@ def test_attention_part_in_portions_over_page_edges(dtype, H, Hkv, dh, window):
 # ---------------------------------------------------------------------------------------------
 # A toy architecture defined entirely in this test: one attention layer and one layer whose
 # mixer keeps a running mean in a fixed-size state slot, run in an order that names the
-# attention layer twice (the second call only reads the cache the first one wrote).
+# attention layer twice (the second call only reads the cache the first one wrote). The attention
+# layer's two norms differ in kind (the second is defined here too) and the other layer has no
+# feed-forward: a layer's make-up is the specification's business, not the framework's.
 # ---------------------------------------------------------------------------------------------
 
 def _define_toy():
@@ -145,7 +147,7 @@ def _define_toy():
     from mini_llm_amd.config.base import LayerCall, LayerSpec, ModelConfig, PartSpec
     from mini_llm_amd.config.registry import register_architecture
     from mini_llm_amd.models.decoder import DecoderModel, build_layers
-    from mini_llm_amd.parts.base import MIXERS, Mixer, ParamSpec, register_mixer
+    from mini_llm_amd.parts.base import MIXERS, Mixer, Norm, ParamSpec, register_mixer, register_norm
     from mini_llm_amd.parts.embedding import NoPositions, TiedHead, TokenEmbedding
     from mini_llm_amd.parts.norms import LayerNorm
 
@@ -188,6 +190,24 @@ def _define_toy():
                 state.copy_(torch.where(own.sum(0)[:, None] > 0, own.T @ s, state))
                 x.index_add_(0, t, self.gain * s)
 
+    @register_norm("toy_scale_norm", replace=True)
+    class ScaleNorm(Norm):
+        """x / sqrt(mean(x^2) + eps) * gain: another norm kind than the first position's."""
+
+        def __init__(self, size, eps, dtype, device):
+            super().__init__(dtype, device)
+            self.size, self.eps, self.gain = size, eps, None
+
+        def param_specs(self, prefix):
+            return [ParamSpec(prefix + ".gain", (self.size,), "vector", self._set, (1.0, 0.1))]
+
+        def _set(self, t):
+            self.gain = t
+
+        def forward(self, x, rows=None):
+            x = x if rows is None else x[rows.long()]
+            return (x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + self.eps) * self.gain).to(self.dtype)
+
     @dataclasses.dataclass(frozen=True)
     class ToyConfig(ModelConfig):
         vocab: int
@@ -221,8 +241,10 @@ def _define_toy():
                 scale=1.0 / math.sqrt(self.width // self.heads), window=None, bias=False, weight_layout="out_in",
                 names={"qkv": "qkv", "out": "o"}))
             mean = PartSpec("toy_running_mean", {"size": self.width, "decay": self.decay})
-            return [LayerSpec("pre_norm", att, ff, norm, "l0.", ("n1", "n2")),
-                    LayerSpec("pre_norm", mean, ff, norm, "l1.", ("n1", "n2"))]
+            scale_norm = PartSpec("toy_scale_norm", {"size": self.width, "eps": 10 * self.eps})
+            # the first layer's two norms differ in kind; the second layer has no feed-forward
+            return [LayerSpec("pre_norm", att, ff, (norm, scale_norm), "l0.", ("n1", "n2")),
+                    LayerSpec("pre_norm", mean, None, norm, "l1.", ("n1", "n2"))]
 
         def layer_order(self):
             return [LayerCall(0, 0), LayerCall(1, 1), LayerCall(0, 0, write=False)]
@@ -263,7 +285,9 @@ def _toy_plain(w, cfg, ids):
                 s = cfg["decay"] * s + (1 - cfg["decay"]) * h[t]
                 add.append(w[p + "mean.gain"] * s)
             x = x + torch.stack(add)
-        x = x + ffn(ln(x, p + "n2"), p)
+            continue                                     # this layer has no feed-forward
+        h = x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + 10 * cfg["eps"]) * w[p + "n2.gain"]
+        x = x + ffn(h, p)
     return ln(x, "final") @ w["emb.weight"].T
 
 
