@@ -90,8 +90,9 @@ int mllm_op_merge_splits(const AttentionSplits* a, const Tensor2* out, hipStream
     return guarded([&] { merge_splits(*a, *out, s); });
 }
 int mllm_op_ln_linear(const Tensor2* x, const float* gamma, const float* beta, float eps, const Tensor2* w,
-                      const float* bias, const Tensor2* out, int epilogue, const int* rows, void* tmp, hipStream_t s) {
-    return guarded([&] { ln_linear(*x, gamma, beta, eps, *w, bias, *out, epilogue, rows, tmp, s); });
+                      const float* bias, const Tensor2* out, int epilogue, const int* rows, void* tmp,
+                      const KvScatter* kv, hipStream_t s) {
+    return guarded([&] { ln_linear(*x, gamma, beta, eps, *w, bias, *out, epilogue, rows, tmp, kv, s); });
 }
 // *unmerged = 1 and *splits filled when the result was left as splits (only with may_split)
 int mllm_op_paged_attention(const AttentionArgs* a, AttentionSplits* splits, int* unmerged, hipStream_t s) {

@@ -264,12 +264,15 @@ void linear_from_splits(const AttentionSplits& a, const Tensor2& w, const float*
 
 void ln_linear(const Tensor2& x, const float* gamma, const float* beta, float eps, const Tensor2& w,
                const float* bias, const Tensor2& out, int epilogue, const int* rows, void* tmp,
-               hipStream_t stream) {
+               const KvScatter* kv, hipStream_t stream) {
     const int64_t M = out.rows, K = x.cols;
     if (x.dtype != F32) fail("ln_linear: the input must be the float32 stream");
     check_linear(M, K, w.dtype, w, out, epilogue, "ln_linear");
     if (rows == nullptr && x.rows != M) fail("ln_linear: out has %lld rows, the input %lld", (long long)M, (long long)x.rows);
-    if (w.dtype == BF16 && M <= tuning().ln_fuse_max_rows && x.contiguous() && aligned(gamma, 16) &&
+    // (More rows than that: the norm is a kernel of its own. Normalising in the tiled product while it stages
+    // its rows was measured at 64 to 256 rows and lost: every workgroup of a row tile has to pull the tile's
+    // fp32 rows through its own L1 for the statistics, 6.5 us at 64 rows of 768, more than the norm's kernel.)
+    if (kv == nullptr && w.dtype == BF16 && M <= tuning().ln_fuse_max_rows && x.contiguous() && aligned(gamma, 16) &&
         (beta == nullptr || aligned(beta, 16))) {
         const int rc = mllm_ln_gemm_bf16(static_cast<const float*>(x.data), static_cast<int>(x.stride), rows, gamma, beta, eps,
                                          w.data, static_cast<int>(w.stride), bias, out.data, static_cast<int>(out.stride),
@@ -280,7 +283,7 @@ void ln_linear(const Tensor2& x, const float* gamma, const float* beta, float ep
     if (tmp == nullptr) fail("ln_linear: these sizes need a buffer for the normalised rows");
     Tensor2 h(tmp, w.dtype, M, K);
     layernorm(x, gamma, beta, eps, h, rows, stream);
-    linear(h, w, bias, out, epilogue, nullptr, stream);
+    linear(h, w, bias, out, epilogue, kv, stream);
 }
 
 // ---------------------------------------------------------------------------------------------

@@ -122,10 +122,10 @@ void linear_from_splits(const AttentionSplits& a, const Tensor2& w, const float*
                         int epilogue, void* tmp, hipStream_t stream);
 void merge_splits(const AttentionSplits& a, const Tensor2& out, hipStream_t stream);
 // out = epilogue(LayerNorm(x[rows]) w^T + bias), the norm fused into the product where the kernels allow;
-// `tmp` ([out.rows, K] in w's dtype) holds the normalised rows otherwise.
+// `tmp` ([out.rows, K] in w's dtype) holds the normalised rows otherwise. `kv` as for linear.
 void ln_linear(const Tensor2& x, const float* gamma, const float* beta, float eps, const Tensor2& w,
                const float* bias, const Tensor2& out, int epilogue, const int* rows, void* tmp,
-               hipStream_t stream);
+               const KvScatter* kv, hipStream_t stream);
 // Causal attention of the step's queries over the pages. Returns true and fills *splits when the result is
 // left unmerged (only with may_split); otherwise `out` holds it.
 bool paged_attention(const AttentionArgs& a, AttentionSplits* splits, hipStream_t stream);

@@ -48,9 +48,9 @@ Linear::Linear(const Tensor2& w, const Tensor2* b) : weight(w) {
 
 // ---------------------------------------------------------------------------------------------
 void Norm::linear(const Tensor2& x, const Linear& lin, const Tensor2& out, int epilogue, const int* rows,
-                  Arena& arena, hipStream_t s) const {
+                  const KvScatter* kv, Arena& arena, hipStream_t s) const {
     const Tensor2 h = forward(x, rows, static_cast<int>(out.rows), arena, s);
-    lin(h, out, epilogue, nullptr, s);
+    lin(h, out, epilogue, kv, s);
 }
 
 const Tensor2& NormedInput::tensor(Arena& arena, hipStream_t s) {
@@ -63,11 +63,8 @@ const Tensor2& NormedInput::tensor(Arena& arena, hipStream_t s) {
 
 void NormedInput::linear(const Linear& lin, const Tensor2& out, int epilogue, const KvScatter* kv, Arena& arena,
                          hipStream_t s) {
-    // Options of the linear map itself (a key/value scatter) are its own business: with them the norm
-    // runs first, unfused.
-    if (kv != nullptr) lin(tensor(arena, s), out, epilogue, kv, s);
-    else if (have_) lin(h_, out, epilogue, nullptr, s);
-    else norm_.linear(x_, lin, out, epilogue, nullptr, arena, s);
+    if (have_) lin(h_, out, epilogue, kv, s);
+    else norm_.linear(x_, lin, out, epilogue, nullptr, kv, arena, s);
 }
 
 // y = (x - mean) * rsqrt(var + eps) * gamma + beta over the last dimension, biased variance,
@@ -91,12 +88,12 @@ public:
         layernorm(x, gamma_, beta_, eps_, h, rows, s);
         return h;
     }
-    void linear(const Tensor2& x, const Linear& lin, const Tensor2& out, int epilogue, const int* rows, Arena& arena,
-                hipStream_t s) const override {
+    void linear(const Tensor2& x, const Linear& lin, const Tensor2& out, int epilogue, const int* rows,
+                const KvScatter* kv, Arena& arena, hipStream_t s) const override {
         // the norm fused into the product where the kernels allow it; otherwise the rows pass through the arena
         const size_t mark = arena.mark();
         void* tmp = arena.take(static_cast<size_t>(out.rows) * size_ * dtype_size(lin.weight.dtype));
-        ln_linear(x, gamma_, beta_, eps_, lin.weight, lin.bias, out, epilogue, rows, tmp, s);
+        ln_linear(x, gamma_, beta_, eps_, lin.weight, lin.bias, out, epilogue, rows, tmp, kv, s);
         arena.release(mark);
     }
     size_t workspace_bytes(int rows) const override { return static_cast<size_t>(rows) * size_ * dtype_size(dtype) + 256; }
@@ -346,7 +343,7 @@ void DecoderModel::forward(const StepView& step, const std::vector<CacheView>& c
     if (logits.rows != step.n_logits || logits.cols != vocab_size() || logits.dtype != F32)
         fail("logits must be float32 [%d, %d]", step.n_logits, vocab_size());
     Linear head(wte, nullptr);
-    final_norm->linear(x, head, logits, STORE_F32, step.logit_rows, arena, s);
+    final_norm->linear(x, head, logits, STORE_F32, step.logit_rows, nullptr, arena, s);
 }
 
 }  // namespace minillm

@@ -105,8 +105,9 @@ public:
     // h[i,:] = norm(x[rows ? rows[i] : i, :]), n rows, from the arena
     virtual Tensor2 forward(const Tensor2& x, const int* rows, int n, Arena& arena, hipStream_t s) const = 0;
     // out = epilogue(lin(norm(x[rows]))); a norm with a fused kernel overrides this
+    // (kv: a key/value scatter of the linear map, passed through to it)
     virtual void linear(const Tensor2& x, const Linear& lin, const Tensor2& out, int epilogue, const int* rows,
-                        Arena& arena, hipStream_t s) const;
+                        const KvScatter* kv, Arena& arena, hipStream_t s) const;
     virtual size_t workspace_bytes(int rows) const = 0;
     int dtype = BF16;
 };

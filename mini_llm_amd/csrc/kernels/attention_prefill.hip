@@ -23,9 +23,10 @@ typedef float f32x4 __attribute__((ext_vector_type(4)));
 
 #define PF_BM 64
 #define PF_BN 128
-#define PF_TABLE_LDS 2048   // block-table entries staged in LDS (longer tables are read from memory)
-#define PF_VT_STRIDE (PF_BN + 2)   // elements per transposed value row: an odd number of words, so that the staging
-                                   // writes of rows 8 apart and the fragment reads of neighbouring rows spread over banks
+#define PF_TABLE_LDS 2048   // most block-table entries of a sequence (the table is staged in LDS)
+#define PF_VT_STRIDE (PF_BN + 12)   // elements per transposed value row: 70 words, which spreads both the staging writes
+                                    // (rows 8 apart) and the fragment reads (16 neighbouring rows, 4 word pairs each)
+                                    // evenly over the banks (measured against 65, 66 and 68 words: 3 to 8 % of the kernel)
 
 union Frag8 {
     bf16x8 v;
@@ -47,9 +48,10 @@ prefill_attention_kernel(const bf16_t* __restrict__ q, int q_stride, int q_col,
     constexpr int KS = DH / 32;            // k steps of S^T
     constexpr int DT = DH / 16;            // 16-dim tiles of O^T
     constexpr int KSTRIDE = DH + 8;
-    __shared__ __attribute__((aligned(16))) bf16_t Ks[PF_BN * KSTRIDE];
-    __shared__ __attribute__((aligned(16))) bf16_t Vt[DH * PF_VT_STRIDE];
-    __shared__ int sm_table[PF_TABLE_LDS];
+    // two buffers of keys and of values: a tile is staged while the one before it is multiplied
+    __shared__ __attribute__((aligned(16))) bf16_t Ks2[2][PF_BN * KSTRIDE];
+    __shared__ __attribute__((aligned(16))) bf16_t Vt2[2][DH * PF_VT_STRIDE];
+    extern __shared__ int sm_table[];          // the sequence's block table (max_blocks entries)
 
     // Which sequence and which of its 64-query tiles this workgroup has. Heads vary fastest and the
     // tiles are handed out last-first: a causal tile's work grows with its position, so the long
@@ -111,8 +113,7 @@ prefill_attention_kernel(const bf16_t* __restrict__ q, int q_stride, int q_col,
     constexpr int KPT = PF_BN * CH / 256;                    // keys per thread: 2, 4, 8 for head sizes 32, 64, 128
     static_assert(KPT * 256 == PF_BN * CH && (KPT & (KPT - 1)) == 0, "whole key groups per thread");
     typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
-    u32x4 ak[KPT], av[KPT];      // register set a
-    u32x4 bk[KPT], bv[KPT];      // register set b
+    u32x4 ak[KPT], av[KPT];      // the tile in flight from memory
     const int ch = tid % CH, grp = tid / CH;
     const int g_lo = k_lo & ~(KPT - 1), g_hi = p_last & ~(KPT - 1);      // first keys of the groups that hold k_lo and p_last
     auto fetch = [&](u32x4 (&rk)[KPT], u32x4 (&rv)[KPT], int kt) {
@@ -125,8 +126,10 @@ prefill_attention_kernel(const bf16_t* __restrict__ q, int q_stride, int q_col,
             rv[u] = *reinterpret_cast<const u32x4*>(v_pages + base + off);
         }
     };
-    auto stage = [&](const u32x4 (&rk)[KPT], const u32x4 (&rv)[KPT]) {
+    auto stage = [&](const u32x4 (&rk)[KPT], const u32x4 (&rv)[KPT], int buf) {
         // keys row-major; values transposed: dim i of the thread's KPT keys becomes KPT/2 neighbouring words
+        bf16_t* Ks = Ks2[buf];
+        bf16_t* Vt = Vt2[buf];
 #pragma unroll
         for (int u = 0; u < KPT; ++u)
             *reinterpret_cast<u32x4*>(Ks + (grp * KPT + u) * KSTRIDE + 8 * ch) = rk[u];
@@ -148,9 +151,11 @@ prefill_attention_kernel(const bf16_t* __restrict__ q, int q_stride, int q_col,
     // Positions of this wavefront's first and last query: a key tile that every one of them sees
     // in full needs no mask.
     const int pw_min = start + q0 + wave * 16, pw_max = pw_min + 15;
-    auto compute = [&](int kt, auto masked_tag) {
+    auto compute = [&](int kt, int buf, auto masked_tag) {
         constexpr bool MASKED = decltype(masked_tag)::value;
         const int j_base = kt * PF_BN;
+        const bf16_t* Ks = Ks2[buf];
+        const bf16_t* Vt = Vt2[buf];
         // S^T: s[nt][r] is the score of key j_base + 16*nt + 4*G + r with this lane's query
         float s[PF_BN / 16][4];
         float tile_max = -INFINITY;
@@ -216,29 +221,27 @@ prefill_attention_kernel(const bf16_t* __restrict__ q, int q_stride, int q_col,
         }
     };
 
-    auto run_tile = [&](int kt) {
+    auto run_tile = [&](int kt, int buf) {
         const int j_base = kt * PF_BN;
         const bool full = j_base + PF_BN - 1 <= pw_min && (window <= 0 || j_base > pw_max - window);
-        if (full) compute(kt, std::false_type{}); else compute(kt, std::true_type{});
+        if (full) compute(kt, buf, std::false_type{}); else compute(kt, buf, std::true_type{});
     };
 
-    // Two register sets, each fetched two tiles ahead of its use. The loop body has no branch
-    // around a load; past the last tile the fetches repeat clamped keys and nothing is computed.
+    // Tile t is multiplied from LDS buffer t % 2 while tile t+1, fetched during the tile before, is
+    // written to the other buffer and tile t+2 is requested from memory: one barrier per tile. The
+    // loop body has no branch around a load; past the last tile the fetches repeat clamped keys,
+    // which are staged and never multiplied.
     const int kt_first = k_lo / PF_BN, kt_last = p_last / PF_BN;
     fetch(ak, av, kt_first);
-    __builtin_amdgcn_sched_barrier(0);     // set a's loads stay the older ones, as on every later iteration
-    fetch(bk, bv, kt_first + 1);
-    for (int kt = kt_first; kt <= kt_last; kt += 2) {
-        lds_barrier();                     // the previous tile's readers are done
-        stage(ak, av);
-        lds_barrier();
+    stage(ak, av, 0);
+    fetch(ak, av, kt_first + 1);
+    lds_barrier();
+    for (int kt = kt_first; kt <= kt_last; ++kt) {
+        const int buf = (kt - kt_first) & 1;
+        stage(ak, av, buf ^ 1);            // (its last readers passed the barrier that ended the tile before)
         fetch(ak, av, kt + 2);
-        run_tile(kt);
+        run_tile(kt, buf);
         lds_barrier();
-        stage(bk, bv);
-        lds_barrier();
-        fetch(bk, bv, kt + 3);
-        if (kt + 1 <= kt_last) run_tile(kt + 1);
     }
     l += __shfl_xor(l, 16, MLLM_WAVE);
     l += __shfl_xor(l, 32, MLLM_WAVE);
@@ -271,14 +274,24 @@ int mllm_prefill_attention_bf16(const void* q, int q_stride, int q_col, const vo
     if (n_heads % n_kv_heads != 0 || n_tiles_upper > 65535) return -1;
     if ((page_size & (page_size - 1)) != 0 || page_size < head_dim / 16 || max_blocks > PF_TABLE_LDS) return -1;
     const dim3 grid(n_heads, n_tiles_upper);
+    const size_t table_bytes = static_cast<size_t>(max_blocks) * sizeof(int);
     const float sl2 = scale * 1.44269504088896340736f;
 #define PF_CASE(D)                                                                                          \
-    case D:                                                                                                 \
-        prefill_attention_kernel<D><<<grid, 256, 0, stream>>>(                                              \
+    case D: {                                                                                               \
+        static bool lds_allowed = false;      /* static and dynamic LDS together pass 64 KB: asked for once */ \
+        if (!lds_allowed) {                                                                                 \
+            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(prefill_attention_kernel<D>),  \
+                                               hipFuncAttributeMaxDynamicSharedMemorySize,                  \
+                                               PF_TABLE_LDS * static_cast<int>(sizeof(int)));               \
+            if (e != hipSuccess) return static_cast<int>(e);                                                \
+            lds_allowed = true;                                                                             \
+        }                                                                                                   \
+        prefill_attention_kernel<D><<<grid, 256, table_bytes, stream>>>(                                            \
             (const bf16_t*)q, q_stride, q_col, (const bf16_t*)k_pages, (const bf16_t*)v_pages, kv_dim,      \
             block_tables, max_blocks, cu_q, ctx_len, n_seqs, n_heads, n_kv_heads, page_size, sl2, window,   \
             (bf16_t*)out, out_stride);                                                                      \
-        break;
+        break;                                                                                              \
+    }
     switch (head_dim) {
         PF_CASE(32) PF_CASE(64) PF_CASE(128)
         default: return -1;

@@ -75,7 +75,7 @@ def engine_library():
         "mllm_op_linear": (_i, [T2p, T2p, _vp, T2p, _i, ctypes.POINTER(KvScatterC), _vp]),
         "mllm_op_linear_from_splits": (_i, [ctypes.POINTER(AttentionSplitsC), T2p, _vp, T2p, _i, _vp, _vp]),
         "mllm_op_merge_splits": (_i, [ctypes.POINTER(AttentionSplitsC), T2p, _vp]),
-        "mllm_op_ln_linear": (_i, [T2p, _vp, _vp, _f, T2p, _vp, T2p, _i, _vp, _vp, _vp]),
+        "mllm_op_ln_linear": (_i, [T2p, _vp, _vp, _f, T2p, _vp, T2p, _i, _vp, _vp, _vp, _vp]),
         "mllm_op_paged_attention": (_i, [ctypes.POINTER(AttentionArgsC), ctypes.POINTER(AttentionSplitsC),
                                          ctypes.POINTER(_i), _vp]),
         "mllm_op_argmax": (_i, [T2p, _vp, _vp]),
@@ -203,8 +203,8 @@ def reserve_scratch(device, rows: int, vocab: int, n_heads: int = 0, head_dim: i
 DECODE_SHAPE_OVERRIDE = None      # (nsplit, waves): forced launch shape of decode attention merged in its kernel
 DECODE_UNMERGED_SHAPE = None      # (nsplit, waves): forced shape of splits that the next product merges
 MERGE_MAX_ROWS = 16               # tokens whose attention splits a product merges while loading (one row block)
-LN_FUSE_MAX_ROWS = 32             # above this many rows the norm is faster as a kernel of its own (measured: 1-2 % of a
-                                  # decode step gained at 24 and 32 rows, 3 % lost at 64)
+LN_FUSE_MAX_ROWS = 32             # rows up to which the few-row product normalises its input itself (measured: 1-2 % of
+                                  # a decode step gained at 24 and 32 rows, 3 % lost at 64)
 _pushed_tuning = None
 
 
@@ -348,9 +348,9 @@ def linear(a, w: torch.Tensor, bias: Optional[torch.Tensor], out: torch.Tensor,
 
 def ln_linear(x: torch.Tensor, gamma: torch.Tensor, beta: Optional[torch.Tensor], eps: float,
               w: torch.Tensor, bias: Optional[torch.Tensor], out: torch.Tensor, epilogue: str = "store",
-              rows: Optional[torch.Tensor] = None) -> torch.Tensor:
+              rows: Optional[torch.Tensor] = None, kv_scatter: Optional[tuple] = None) -> torch.Tensor:
     """out = epilogue(LayerNorm(x) @ w.T + bias) with x the fp32 stream [*,K] and w [N,K]; with
-    ``rows`` (int32 [M]) row m of the input is x[rows[m]].
+    ``rows`` (int32 [M]) row m of the input is x[rows[m]]; ``kv_scatter`` as for ``linear``.
 
     For bfloat16 weights, at most 32 rows and fewer than 16384 columns the norm is fused into the
     product (one kernel); otherwise the norm and the product run one after the other. Same numerics
@@ -371,9 +371,15 @@ def ln_linear(x: torch.Tensor, gamma: torch.Tensor, beta: Optional[torch.Tensor]
     push_tuning()
     # (room for the normalised rows, used when the fused kernel does not take these sizes)
     tmp = torch.empty((M, K), dtype=w.dtype, device=x.device)
+    kv = None
+    if kv_scatter is not None:
+        slots, k_pages, v_pages, q_cols = kv_scatter
+        _gpu(slots, k_pages, v_pages)
+        _i32(slots, "slots", M)
+        kv = ctypes.byref(KvScatterC(slots.data_ptr(), t2(k_pages, "k_pages"), t2(v_pages, "v_pages"), int(q_cols)))
     _ok(engine_library().mllm_op_ln_linear(ctypes.byref(t2(x, "x")), _p(gamma), _p(beta), eps, ctypes.byref(t2(w, "w")),
                                            _p(bias), ctypes.byref(t2(out, "out")), EPILOGUES[epilogue], _p(rows),
-                                           _p(tmp), _stream()))
+                                           _p(tmp), kv, _stream()))
     return out
 
 

@@ -54,9 +54,10 @@ class Norm(Part):
         raise NotImplementedError
 
     def linear(self, x: torch.Tensor, lin, out: torch.Tensor, epilogue: str = "store",
-               rows: Optional[torch.Tensor] = None) -> torch.Tensor:
-        """out = epilogue(lin(norm(x[rows]))). A norm with a fused kernel overrides this."""
-        return lin(self.forward(x, rows), out, epilogue)
+               rows: Optional[torch.Tensor] = None, **linear_options) -> torch.Tensor:
+        """out = epilogue(lin(norm(x[rows]))); ``linear_options`` are options of the linear map itself
+        (such as a key/value scatter) and are passed through. A norm with a fused kernel overrides this."""
+        return lin(self.forward(x, rows), out, epilogue, **linear_options)
 
 
 class NormedInput:
@@ -76,13 +77,11 @@ class NormedInput:
         return self._h
 
     def linear(self, lin, out: torch.Tensor, epilogue: str = "store", **linear_options) -> torch.Tensor:
-        """``lin`` applied to the normalised input. Options of the linear map itself (such as a
-        key/value scatter) are its own business: with them the norm runs first, unfused."""
-        if linear_options:
-            return lin(self.tensor(), out, epilogue, **linear_options)
+        """``lin`` applied to the normalised input; ``linear_options`` are options of the linear map
+        itself (such as a key/value scatter)."""
         if self._h is not None:
-            return lin(self._h, out, epilogue)
-        return self.norm.linear(self.x, lin, out, epilogue)
+            return lin(self._h, out, epilogue, **linear_options)
+        return self.norm.linear(self.x, lin, out, epilogue, **linear_options)
 
 
 class Mixer(Part):

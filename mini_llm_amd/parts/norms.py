@@ -39,9 +39,10 @@ class LayerNorm(Norm):
         self.beta = t
 
     def linear(self, x: torch.Tensor, lin, out: torch.Tensor, epilogue: str = "store",
-               rows: Optional[torch.Tensor] = None) -> torch.Tensor:
+               rows: Optional[torch.Tensor] = None, **linear_options) -> torch.Tensor:
         """out = epilogue(lin(norm(x[rows]))): the norm fused into the product where the kernels allow it."""
-        return ops.ln_linear(x, self.gamma, self.beta, self.eps, lin.weight, lin.bias, out, epilogue, rows)
+        return ops.ln_linear(x, self.gamma, self.beta, self.eps, lin.weight, lin.bias, out, epilogue, rows,
+                             **linear_options)
 
     def forward(self, x: torch.Tensor, rows: Optional[torch.Tensor] = None) -> torch.Tensor:
         n = rows.numel() if rows is not None else x.shape[0]

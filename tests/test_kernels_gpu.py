@@ -197,6 +197,34 @@ def test_linear_bf16_scatters_keys_and_values(ops, M, H, Hkv, dh, K):
                    kv_scatter=(perm.to(DEV), kp, vp, q_cols))
 
 
+@pytest.mark.parametrize("M,H,Hkv,dh,K", [(65, 12, 12, 64, 768), (256, 25, 25, 64, 1600), (100, 6, 2, 32, 200), (8, 4, 4, 16, 64),
+                                          (64, 12, 12, 64, 768), (300, 3, 3, 32, 96)])
+def test_ln_linear_scatters_keys_and_values(ops, M, H, Hkv, dh, K):
+    """The norm, the QKV product and the page write in one call: the output of the norm followed by the
+    product, and the key and value columns in their slots."""
+    g = torch.Generator().manual_seed(M + K)
+    q_cols, kv_dim = H * dh, Hkv * dh
+    N = q_cols + 2 * kv_dim
+    x = _rand((M, K), torch.float32, g, std=2.0) + 0.3
+    gamma, beta = 1 + 0.1 * _rand((K,), torch.float32, g), 0.1 * _rand((K,), torch.float32, g)
+    w = _rand((N, K), torch.bfloat16, g, std=1.0 / math.sqrt(K))
+    bias = 0.5 * _rand((N,), torch.float32, g)
+    rows = M + 37
+    slots = torch.randperm(rows, generator=g)[:M].to(torch.int32)
+    slots[::7] = -1
+    k0, v0 = _rand((rows, kv_dim), torch.bfloat16, g), _rand((rows, kv_dim), torch.bfloat16, g)
+    kp, vp = k0.clone().to(DEV), v0.clone().to(DEV)
+    out = torch.empty((M, N), dtype=torch.bfloat16, device=DEV)
+    ops.ln_linear(x.to(DEV), gamma.to(DEV), beta.to(DEV), 1e-5, w.to(DEV), bias.to(DEV), out, "store",
+                  kv_scatter=(slots.to(DEV), kp, vp, q_cols))
+    h = plain_ops.layernorm(x, gamma, beta, 1e-5, torch.empty(M, K, dtype=torch.bfloat16))
+    ref = plain_ops.linear(h, w, bias, torch.empty((M, N), dtype=torch.float64))
+    assert (out.cpu().double() - ref).abs().max().item() <= 4e-2
+    kr, vr = k0.clone(), v0.clone()
+    plain_ops.kv_append(out.cpu(), q_cols, q_cols + kv_dim, kv_dim, kr, vr, slots)
+    assert torch.equal(kp.cpu(), kr) and torch.equal(vp.cpu(), vr)
+
+
 @pytest.mark.parametrize("M", [1, 8, 16, 17, 48, 64])
 @pytest.mark.parametrize("N,K", [(2304, 768), (768, 3072), (1000, 96), (50257, 768), (72, 1600), (4800, 1600),
                                  (1600, 6400), (1024, 4096),
@@ -279,8 +307,9 @@ def test_linear_bf16_few_rows_long_k_shares_tiles(ops, M, N, K):
                                    (64, 50257, 768), (64, 104, 1600), (65, 96, 64),
                                    # more than 256 tiles: two per workgroup
                                    (8, 4800, 1600), (3, 4104, 72), (16, 8190, 200),
-                                   # more than 16 rows: the norm runs as a kernel of its own
-                                   (64, 3072, 768), (48, 4096, 1024), (17, 40, 72), (31, 1000, 2048), (50, 136, 200)])
+                                   # more than 32 rows: the norm runs as a kernel of its own
+                                   (64, 3072, 768), (48, 4096, 1024), (50, 136, 200), (100, 320, 96), (200, 4800, 1600),
+                                   (256, 3072, 776), (17, 40, 72), (31, 1000, 2048), (300, 320, 96)])
 @pytest.mark.parametrize("epi", ["store", "gelu_tanh", "gelu_erf", "store_f32"])
 def test_ln_linear(ops, dtype, M, N, K, epi):
     """LayerNorm fused into the product (bf16, few rows) and its unfused form give the plain result."""
@@ -605,7 +634,7 @@ def test_paged_attention_long_contexts(ops, dtype, H, Hkv, dh, page):
     a window."""
     g = torch.Generator().manual_seed(dh + page)
     for seqs, window in (([(9000, 1), (5, 1)], 0), ([(8300, 200)], 0), ([(0, 2300)], 777), ([(20000, 1)], 0),
-                         ([(8190, 3), (100, 40)], 777)):
+                         ([(8190, 3), (100, 40)], 777), ([(8000, 192)], 0)):        # (the last: 2048 blocks of 4 exactly)
         out, ref = _attention_case(ops, dtype, H, Hkv, dh, page, seqs, window, g)
         assert torch.isfinite(out).all()
         assert (out - ref).abs().max() <= _tol(dtype, 2), (seqs, window)
