@@ -34,6 +34,10 @@ HIPCC_FLAGS = [
     # the first 16 dwords of a kernel's arguments arrive in registers with the wavefront instead of
     # being loaded by it: saves the load's latency at the head of every short kernel
     "-mllvm", "-amdgpu-kernarg-preload-count=16",
+    # MFMA results go to ordinary vector registers, not to the accumulation registers: the kernels here
+    # read every result with vector instructions (softmax, epilogues), and each such read or write of an
+    # accumulation register is a move of its own (12 % of prefill attention's vector instructions)
+    "-mllvm", "-amdgpu-mfma-vgpr-form=1",
     "-Wno-unused-command-line-argument", "-Wno-unknown-warning-option",
 ]
 CXX_FLAGS = ["-O2", "-std=c++17", "-fPIC", "-shared", "-Wall"]
