@@ -160,7 +160,15 @@ def build_library(name: str, verbose: bool = True) -> str:
         cc = _find("hipcc", ["/opt/rocm/bin"])
         cmd = [cc] + HIPCC_FLAGS
     elif spec["kind"] == "hiphost":
-        for dep in needed_by(name):                # link against the libraries beside it
+        # link against the libraries beside it; stale ones are compiled first, those without needs of
+        # their own side by side
+        stale = [d for d in needed_by(name) if not is_current(d)]
+        leaves = [d for d in stale if not LIBRARIES[d].get("needs")]
+        if len(leaves) > 1:
+            from concurrent.futures import ThreadPoolExecutor
+            with ThreadPoolExecutor(max_workers=4) as ex:
+                list(ex.map(lambda d: build_library(d, verbose), leaves))
+        for dep in stale:
             if not is_current(dep):
                 build_library(dep, verbose)
         cc = _find("g++", ["/usr/bin"])
