@@ -360,8 +360,25 @@ std::vector<int> ModelRunner::collect() {
 // ---------------------------------------------------------------------------------------------
 // engine
 // ---------------------------------------------------------------------------------------------
+// Pages that `fraction` of the free device memory holds, for caches with these needs.
+static int pages_for_memory_fraction(const std::vector<CacheNeed>& needs, int dtype, int page_size, double fraction) {
+    if (fraction > 1.0) throw EngineError("kv_memory_fraction must be at most 1");
+    size_t per_token = 0;
+    for (const CacheNeed& n : needs)
+        if (n.kind == 1) per_token += 2 * static_cast<size_t>(n.n_kv_heads) * n.head_dim * dtype_size(dtype);
+    if (per_token == 0) return 1;
+    size_t free_bytes = 0, total_bytes = 0;
+    HIP_OK(hipMemGetInfo(&free_bytes, &total_bytes));
+    const double pages = fraction * static_cast<double>(free_bytes) / (static_cast<double>(per_token) * page_size);
+    const double most = 2147483647.0 / page_size;          // rows of a pool are indexed with 32 bits
+    if (pages < 1.0) throw EngineError("kv_memory_fraction leaves no room for a single page");
+    return static_cast<int>(std::min(pages, most));
+}
+
 Engine::Engine(std::unique_ptr<LoadedModel> model, const EngineOptions& o) : model_(std::move(model)), options_(o) {
-    runner_.reset(new ModelRunner(*model_, o.kv_block_size, o.total_kv_blocks, o.max_batch_num));
+    if (o.kv_memory_fraction > 0.0)
+        options_.total_kv_blocks = pages_for_memory_fraction(model_->caches, model_->dtype, o.kv_block_size, o.kv_memory_fraction);
+    runner_.reset(new ModelRunner(*model_, o.kv_block_size, options_.total_kv_blocks, o.max_batch_num));
     SchedulerOptions so;
     so.max_num_seqs = o.max_batch_num;
     so.max_tokens_per_step = o.max_tokens_per_step;

@@ -35,6 +35,8 @@ public:
 struct EngineOptions {
     int kv_block_size = 16;            // tokens per page (reference: DEFAULT_KV_BLOCK_SIZE, constants.h:16)
     int total_kv_blocks = 4096;        // pages in the pool (reference: DEFAULT_TOTAL_KV_BLOCKS, constants.h:17)
+    double kv_memory_fraction = 0.0;   // > 0: the pool takes this share of the device memory that is free once the
+                                       // weights are loaded, whatever total_kv_blocks says
     int max_batch_num = 16;            // sequences in one step (reference: MAX_BATCH_NUM, constants.h:20)
     int max_tokens_per_step = 2048;    // token budget of one step
     int prefill_chunk = 512;           // longest prompt portion

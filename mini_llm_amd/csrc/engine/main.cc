@@ -139,6 +139,7 @@ int cmd_generate(int argc, char** argv) {
     EngineOptions o;
     o.kv_block_size = static_cast<int>(a.integer("kv-block-size", 16));
     o.total_kv_blocks = static_cast<int>(a.integer("total-kv-blocks", 4096));
+    o.kv_memory_fraction = a.has("kv-memory-fraction") ? std::atof(a.get("kv-memory-fraction").c_str()) : 0.0;
     o.max_batch_num = static_cast<int>(a.integer("max-batch-num", 16));
     o.max_tokens_per_step = static_cast<int>(a.integer("max-tokens-per-step", 2048));
     o.prefill_chunk = static_cast<int>(a.integer("prefill-chunk", 512));
@@ -285,7 +286,7 @@ int main(int argc, char** argv) {
                  "usage: mini-llm generate|make-model|replay [options]\n"
                  "  generate   --model DIR | --preset NAME [--weights-seed S]  [--dtype bfloat16|float32] [--prompt-ids \"1 2 3\"]...\n"
                  "             [--prompts-file F] [--max-new-tokens 8] [--temperature 0] [--seed 0] [--ignore-eos] [--stream] [--stats]\n"
-                 "             [--kv-block-size 16] [--total-kv-blocks 4096] [--max-batch-num 16] [--max-tokens-per-step 2048]\n"
+                 "             [--kv-block-size 16] [--total-kv-blocks 4096 | --kv-memory-fraction F] [--max-batch-num 16] [--max-tokens-per-step 2048]\n"
                  "             [--prefill-chunk 512]\n"
                  "  make-model (--preset NAME | --config FILE) --seed S --out DIR [--weights-dtype bfloat16|float32]\n"
                  "  replay     --model DIR --dtype bfloat16|float32 --out DIR --max-tokens N [--page-size 16]\n");

@@ -44,6 +44,19 @@ static double gelu_tanh(double v) { return 0.5 * v * (1.0 + std::tanh(0.79788456
 // 0.5 v (1 + erf(v / sqrt 2)): the exact form (the reference has only the tanh form)
 static double gelu_erf(double v) { return 0.5 * v * (1.0 + std::erf(v * 0.70710678118654752440)); }
 
+// The epilogues as operations of their own (the reference: /root/reference/src/kernels/gelu.cu:7-21,
+// /root/reference/src/kernels/residual.cu:6-31; its bias is added inside the product, linear.cu:8-27).
+void ref_gelu(const float* x, float* out, long n, int exact) {
+    for (long i = 0; i < n; ++i) out[i] = static_cast<float>(exact ? gelu_erf(x[i]) : gelu_tanh(x[i]));
+}
+void ref_add_bias(float* x, const float* bias, int M, int N) {
+    for (int m = 0; m < M; ++m)
+        for (int n = 0; n < N; ++n) x[static_cast<size_t>(m) * N + n] += bias[n];
+}
+void ref_residual_add(float* x, const float* y, long n) {
+    for (long i = 0; i < n; ++i) x[i] += y[i];
+}
+
 // out = epilogue(a w^T + bias): a [M,K], w [N,K] (both k-contiguous), bias [N] or null.
 // epilogue: 0 store, 1 gelu_tanh, 2 gelu_erf, 3 add into out, 4 store (the kernels' fp32 store)
 // -- /root/reference/src/kernels/linear.cu:8-87, the store path /root/reference/src/kernels/gemm.cu:534-564

@@ -29,6 +29,8 @@ from .step import ModelRunner, StepEntry
 class EngineOptions:
     kv_block_size: int = 16             # tokens per page (reference: DEFAULT_KV_BLOCK_SIZE, constants.h:16)
     total_kv_blocks: int = 4096         # pages in the pool (reference: DEFAULT_TOTAL_KV_BLOCKS, constants.h:17)
+    kv_memory_fraction: float = 0.0     # > 0: the pool takes this share of the device memory that is free once the
+                                        # weights are loaded, whatever total_kv_blocks says
     max_batch_num: int = 16             # sequences in one step (reference: MAX_BATCH_NUM, constants.h:20)
     max_tokens_per_step: int = 2048     # token budget of one step
     prefill_chunk: int = 512            # longest prompt portion
@@ -63,12 +65,31 @@ class _Request:
         return self.tokens[self.prompt_len:]
 
 
+def pages_for_memory_fraction(model, page_size: int, fraction: float) -> int:
+    """Pages that ``fraction`` of the device memory free now holds, for the caches this model asks for."""
+    from ..cache.manager import KVCacheSpec
+    if fraction > 1:
+        raise ValueError("kv_memory_fraction must be at most 1")
+    esize = torch.empty((), dtype=model.dtype).element_size()
+    per_token = sum(2 * s.n_kv_heads * s.head_dim * esize for s in model.cache_specs() if isinstance(s, KVCacheSpec))
+    if per_token == 0:
+        return 1
+    free_bytes, _ = torch.cuda.mem_get_info(model.device)
+    pages = int(fraction * free_bytes / (per_token * page_size))
+    if pages < 1:
+        raise ValueError("kv_memory_fraction leaves no room for a single page")
+    return min(pages, (2 ** 31 - 1) // page_size)          # rows of a pool are indexed with 32 bits
+
+
 class Engine:
     def __init__(self, model, options: Optional[EngineOptions] = None):
         self.model = model
         self.options = options or EngineOptions()
         o = self.options
-        self.runner = ModelRunner(model, o.kv_block_size, o.total_kv_blocks, o.max_batch_num)
+        n_pages = o.total_kv_blocks
+        if o.kv_memory_fraction > 0:
+            n_pages = pages_for_memory_fraction(model, o.kv_block_size, o.kv_memory_fraction)
+        self.runner = ModelRunner(model, o.kv_block_size, n_pages, o.max_batch_num)
         self.scheduler = Scheduler(self.runner.manager, o.max_batch_num, o.max_tokens_per_step,
                                    o.prefill_chunk, model.max_positions)
         self.eos_token_id = model.config.eos_token_id

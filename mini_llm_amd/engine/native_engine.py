@@ -76,8 +76,8 @@ class NativeEngine:
 
     @staticmethod
     def _pack(o: EngineOptions):
-        return (ctypes.c_int * 6)(o.kv_block_size, o.total_kv_blocks, o.max_batch_num, o.max_tokens_per_step,
-                                  o.prefill_chunk, 1 if o.overlap_decode else 0)
+        return (ctypes.c_int * 7)(o.kv_block_size, o.total_kv_blocks, o.max_batch_num, o.max_tokens_per_step,
+                                  o.prefill_chunk, 1 if o.overlap_decode else 0, int(round(o.kv_memory_fraction * 1e6)))
 
     @classmethod
     def from_pretrained(cls, model_dir: str, dtype="bfloat16", options: Optional[EngineOptions] = None, **kw):

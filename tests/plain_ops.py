@@ -83,10 +83,10 @@ def linear(a, w, bias, out, epilogue="store", kv_scatter=None):
     return out
 
 
-def ln_linear(x, gamma, beta, eps, w, bias, out, epilogue="store", rows=None):
+def ln_linear(x, gamma, beta, eps, w, bias, out, epilogue="store", rows=None, kv_scatter=None):
     n = x.shape[0] if rows is None else rows.numel()
     h = layernorm(x, gamma, beta, eps, torch.empty((n, x.shape[1]), dtype=w.dtype), rows)
-    return linear(h, w, bias, out, epilogue)
+    return linear(h, w, bias, out, epilogue, kv_scatter=kv_scatter)
 
 
 def kv_append(src, k_col, v_col, kv_dim, k_pages, v_pages, slots):

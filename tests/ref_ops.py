@@ -82,3 +82,22 @@ def sample(logits, temperature, u):
     out = torch.empty(l.shape[0], dtype=torch.int32)
     _lib().ref_sample(_p(l), l.shape[0], l.shape[1], _p(t), _p(uu), _p(out))
     return out
+
+
+def gelu(x, exact=False):
+    x = _f(x)
+    out = torch.empty_like(x)
+    _lib().ref_gelu(_p(x), _p(out), ctypes.c_long(x.numel()), 1 if exact else 0)
+    return out
+
+
+def add_bias(x, bias):
+    out = _f(x).clone()
+    _lib().ref_add_bias(_p(out), _p(_f(bias)), out.shape[0], out.shape[1])
+    return out
+
+
+def residual_add(x, y):
+    out, y = _f(x).clone(), _f(y)
+    _lib().ref_residual_add(_p(out), _p(y), ctypes.c_long(out.numel()))
+    return out

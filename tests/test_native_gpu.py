@@ -165,3 +165,21 @@ def test_native_engine_through_its_python_face(tiny_model_dirs, dtype):
     mem = NativeEngine.from_random(dict(TINY_A), seed=0, dtype=dtype, options=o)
     greedy = SamplingParams(max_new_tokens=8, ignore_eos=True)
     assert mem.generate(prompts[:3], greedy) == native.generate(prompts[:3], greedy)
+
+
+def test_pool_sized_from_free_device_memory(tiny_model_dirs):
+    """`kv_memory_fraction`: both engines size the page pool from the device memory that is free once the
+    weights are loaded (tiny A in bfloat16 holds 512 bytes per token: 2 caches x K and V x 64 columns)."""
+    from mini_llm_amd import Engine, EngineOptions, NativeEngine, SamplingParams
+    free_before, _ = torch.cuda.mem_get_info()
+    o = EngineOptions(kv_block_size=4, total_kv_blocks=7, kv_memory_fraction=0.002, max_batch_num=2)
+    native = NativeEngine.from_pretrained(tiny_model_dirs["a"], dtype="bfloat16", options=o)
+    pages = native.stats()["total_pages"]
+    expect = 0.002 * free_before / (4 * 512)
+    assert 0.5 * expect <= pages <= 1.05 * expect and pages > 1000, (pages, expect)
+    python = Engine.from_pretrained(tiny_model_dirs["a"], dtype="bfloat16", options=o)
+    assert 0.5 * expect <= python.stats()["total_pages"] <= 1.05 * expect
+    sp = SamplingParams(max_new_tokens=5, ignore_eos=True)
+    assert native.generate([[1, 2, 3]], sp) == python.generate([[1, 2, 3]], sp)
+    with pytest.raises((RuntimeError, ValueError), match="at most 1"):
+        NativeEngine.from_pretrained(tiny_model_dirs["a"], dtype="bfloat16", options=EngineOptions(kv_memory_fraction=1.5))

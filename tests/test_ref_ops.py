@@ -96,3 +96,18 @@ def test_token_choice():
     plain_ops.sample(logits, temp, u, want)
     assert torch.equal(ref_ops.sample(logits, temp, u), want)
     assert ref_ops.sample(logits, temp, u)[0] == logits[0].argmax()
+
+
+def test_unfused_epilogues():
+    # the reference's vector for its GELU: x = 0.01 i, 1027 values, tolerance 1e-5 (/root/reference/tests/kernels/gelu/gen.py:5-12)
+    x = 0.01 * torch.arange(1027, dtype=torch.float32) - 5.0
+    assert (ref_ops.gelu(x) - F.gelu(x.double(), approximate="tanh")).abs().max() <= 1e-6
+    assert (ref_ops.gelu(x, exact=True) - F.gelu(x.double())).abs().max() <= 1e-6
+    assert (ref_ops.gelu(x) - ref_ops.gelu(x, exact=True)).abs().max() > 1e-4          # the two forms are told apart
+    g = torch.Generator().manual_seed(4)
+    a, b, bias = torch.randn(5, 7, generator=g), torch.randn(5, 7, generator=g), torch.randn(7, generator=g)
+    assert torch.equal(ref_ops.add_bias(a, bias), a + bias) and torch.equal(ref_ops.residual_add(a, b), a + b)
+    # the fused epilogue of the product is these, one after the other
+    w = torch.randn(7, 7, generator=g)
+    fused = ref_ops.linear(a, w, bias, None, "gelu_tanh")
+    assert (fused - ref_ops.gelu(ref_ops.add_bias(ref_ops.linear(a, w, None), bias))).abs().max() <= 1e-6
