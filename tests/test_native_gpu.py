@@ -183,3 +183,66 @@ def test_pool_sized_from_free_device_memory(tiny_model_dirs):
     assert native.generate([[1, 2, 3]], sp) == python.generate([[1, 2, 3]], sp)
     with pytest.raises((RuntimeError, ValueError), match="at most 1"):
         NativeEngine.from_pretrained(tiny_model_dirs["a"], dtype="bfloat16", options=EngineOptions(kv_memory_fraction=1.5))
+
+
+def test_native_loader_lists_every_mismatch_and_reads_shards(tmp_path):
+    """The C++ loader: ONE error that lists missing, unexpected and wrong-shape tensors; a checkpoint in two
+    float16 shards gives the logits of the whole one; a configuration it cannot honour is refused by name."""
+    import json
+    from safetensors import safe_open
+    from safetensors.torch import save_file
+    from conftest import TINY_A, TINY_B
+    from mini_llm_amd import EngineOptions, NativeEngine, SamplingParams, write_random_model
+    o = EngineOptions(kv_block_size=4, total_kv_blocks=64, max_batch_num=2)
+
+    def tensors(d):
+        with safe_open(os.path.join(d, "model.safetensors"), framework="pt") as f:
+            return {k: f.get_tensor(k) for k in f.keys()}
+
+    d = write_random_model(dict(TINY_A), str(tmp_path / "m"), seed=0)
+    t = tensors(d)
+    del t["h.1.ln_2.bias"], t["wpe.weight"]
+    t["h.0.mlp.c_fc.weight"] = torch.zeros(256, 64, dtype=torch.bfloat16)     # transposed by mistake
+    t["h.0.attn.c_attn.bias"] = torch.zeros(64)
+    t["h.7.extra.weight"] = torch.zeros(2)
+    save_file(t, os.path.join(d, "model.safetensors"))
+    with pytest.raises(RuntimeError) as ei:
+        NativeEngine.from_pretrained(d, dtype="float32", options=o)
+    msg = str(ei.value)
+    for piece in ("missing tensors (2)", "h.1.ln_2.bias", "wpe.weight", "unexpected tensors (1)", "h.7.extra.weight",
+                  "wrong shapes (2)", "h.0.mlp.c_fc.weight", "h.0.attn.c_attn.bias", "[64, 256]", "[256, 64]"):
+        assert piece in msg, (piece, msg)
+    os.remove(os.path.join(d, "model.safetensors"))
+    with pytest.raises(RuntimeError, match="neither model.safetensors"):
+        NativeEngine.from_pretrained(d, dtype="float32", options=o)
+
+    # two float16 shards against the whole file
+    whole = write_random_model(dict(TINY_B), str(tmp_path / "whole"), seed=4, weights_dtype="float16")
+    t = tensors(whole)
+    sharded = tmp_path / "sharded"
+    sharded.mkdir()
+    names = sorted(t)
+    parts = {"model-00001-of-00002.safetensors": names[:len(names) // 2],
+             "model-00002-of-00002.safetensors": names[len(names) // 2:]}
+    for fname, ns in parts.items():
+        save_file({n: t[n] for n in ns}, str(sharded / fname))
+    json.dump({"metadata": {}, "weight_map": {n: f for f, ns in parts.items() for n in ns}},
+              open(sharded / "model.safetensors.index.json", "w"))
+    json.dump(json.load(open(os.path.join(whole, "config.json"))), open(sharded / "config.json", "w"))
+    sp = SamplingParams(max_new_tokens=12, ignore_eos=True)
+    prompts = [[3, 1, 4, 1, 5, 9, 2, 6], [27, 18, 28]]
+    o8 = EngineOptions(kv_block_size=8, total_kv_blocks=32, max_batch_num=2)
+    a = NativeEngine.from_pretrained(whole, dtype="float32", options=o8).generate(prompts, sp)
+    b = NativeEngine.from_pretrained(str(sharded), dtype="float32", options=o8).generate(prompts, sp)
+    assert a == b and all(len(x) == 12 for x in a)
+    save_file({names[0]: t[names[0]], **{n: t[n] for n in parts["model-00002-of-00002.safetensors"]}},
+              str(sharded / "model-00002-of-00002.safetensors"))
+    with pytest.raises(RuntimeError, match="two files"):
+        NativeEngine.from_pretrained(str(sharded), dtype="float32", options=o8)
+
+    # configurations
+    for change, match in [({"n_head": 5}, "divisible"), ({"activation_function": "relu"}, "activation_function"),
+                          ({"tie_word_embeddings": False}, "untied"), ({"scale_attn_by_inverse_layer_idx": True}, "not supported"),
+                          ({"architectures": ["SomethingElse"], "model_type": "other"}, "no known architecture")]:
+        with pytest.raises(RuntimeError, match=match):
+            NativeEngine.from_random(dict(TINY_A, **change), seed=0, dtype="float32", options=o)
