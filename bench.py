@@ -25,10 +25,10 @@ SIZES = {   # BASELINE.json configs[2..4]: n_layer, n_embd, n_head, n_inner
 }
 
 
-def small_config(n_layer, size="gpt2-small"):
+def small_config(n_layer, size="gpt2-small", n_positions=1024):
     full_layers, d, h, f = SIZES[size]
     return dict(architectures=["GPT2LMHeadModel"], model_type="gpt2", n_layer=n_layer or full_layers, n_embd=d,
-                n_head=h, n_inner=f, vocab_size=50257, n_positions=1024, layer_norm_epsilon=1e-5,
+                n_head=h, n_inner=f, vocab_size=50257, n_positions=n_positions, layer_norm_epsilon=1e-5,
                 activation_function="gelu_new", eos_token_id=50256, bos_token_id=50256)
 
 
@@ -212,6 +212,8 @@ def main():
     ap.add_argument("--layers", type=int, default=0, help="fewer layers than the size has (named in config)")
     ap.add_argument("--size", default="gpt2-small", choices=sorted(SIZES), help="layer sizes (default: configs[2])")
     ap.add_argument("--prompt-len", type=int, default=512)
+    ap.add_argument("--positions", type=int, default=1024,
+                    help="n_positions of the random model (the benchmark's context length; longer: further context lengths)")
     ap.add_argument("--no-points", action="store_true", help="skip the batch-1/64 and prefill measurements")
     ap.add_argument("--prefill-only", action="store_true", help="measure only the prefill step (profiling)")
     ap.add_argument("--prefill-requests", type=int, default=2, help="with --prefill-only: prompts in the step")
@@ -231,7 +233,7 @@ def main():
     import torch
     from mini_llm_amd import write_random_model
 
-    cfg = small_config(args.layers, args.size)
+    cfg = small_config(args.layers, args.size, args.positions)
     if args.peaks_only:
         from mini_llm_amd.kernels.peaks import NOMINAL, measure_peaks
         print(json.dumps({"metric": "measured peaks of this GPU", "measured": measure_peaks("cuda:0"),

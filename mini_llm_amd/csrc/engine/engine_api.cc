@@ -45,7 +45,7 @@ void* mllm_scratch_address(const char* name) {
     guarded([&] { p = scratch_address(name); });
     return p;
 }
-// name: "decode_shape" (nsplit, waves; 0, 0 = automatic), "unmerged_shape", "merge_max_rows" (a), "ln_fuse_max_rows" (a)
+// name: "decode_shape" (nsplit, waves; 0, 0 = automatic), "unmerged_shape", "merge_max_rows" (a), "ln_fuse_max_rows" (a), "long_context_splits" (a: 0 off, 1 on)
 int mllm_set_tuning(const char* name, int a, int b) {
     return guarded([&] {
         Tuning& t = tuning();
@@ -54,6 +54,7 @@ int mllm_set_tuning(const char* name, int a, int b) {
         else if (n == "unmerged_shape") { t.unmerged_nsplit = a; t.unmerged_waves = b; }
         else if (n == "merge_max_rows") t.merge_max_rows = a;
         else if (n == "ln_fuse_max_rows") t.ln_fuse_max_rows = a;
+        else if (n == "long_context_splits") t.long_context_splits = a;
         else fail("unknown tuning value '%s'", name);
     });
 }

@@ -94,7 +94,8 @@ void reserve_scratch(int rows, int vocab, int n_heads, int head_dim) {
     argmax_indices(rows * chunks);
     gemm_workspace();
     if (n_heads > 0 && head_dim > 0) {
-        decode_partials(static_cast<size_t>(rows) * n_heads * DECODE_MAX_SPLIT * (head_dim + 2));
+        // (every launch shape keeps pairs x splits within max(4 x pairs, 256))
+        decode_partials(std::max<size_t>(static_cast<size_t>(rows) * n_heads * DECODE_MAX_SPLIT, 256) * (head_dim + 2));
         decode_counters(static_cast<size_t>(rows) * n_heads);
     }
 }
@@ -290,10 +291,11 @@ void ln_linear(const Tensor2& x, const float* gamma, const float* beta, float ep
 // attention
 // ---------------------------------------------------------------------------------------------
 // How many workgroups share one (token, head) pair's keys, and wavefronts per workgroup.
-static void decode_launch_shape(int pairs, int max_ctx_len, bool unmerged, int* nsplit, int* waves) {
+static void decode_launch_shape(int pairs, int max_ctx_len, bool unmerged, int* nsplit, int* waves, bool* merge_kernel) {
     const Tuning& t = tuning();
+    *merge_kernel = false;
     if (t.decode_nsplit > 0) { *nsplit = t.decode_nsplit; *waves = t.decode_waves; return; }
-    if (unmerged) {
+    if (unmerged && !(t.long_context_splits && std::min(256 / std::max(pairs, 1), max_ctx_len / 512) >= 8)) {
         // The splits cost nothing to merge here (the next product does it while it loads), so few pairs
         // are spread over the compute units: a unit streams keys at 35 to 90 GB/s, and a pair's keys
         // and values at 768 tokens are 200 KB. Every split keeps at least 128 keys. (Measured at GPT-2
@@ -305,6 +307,20 @@ static void decode_launch_shape(int pairs, int max_ctx_len, bool unmerged, int* 
             const int keys = (max_ctx_len + n - 1) / n;
             *nsplit = n;
             *waves = std::max(2, std::min(12, (keys + 63) / 64));
+            return;
+        }
+    }
+    // Long contexts at few pairs (batch 1 to 3 at GPT-2 sizes): up to 4 workgroups a pair leave most of the
+    // chip idle while each streams megabytes (12 pairs at 32,000 keys: 51 us a layer, 1.9 TB/s). They are
+    // split over up to 256 workgroups, at least 512 keys each, and a small kernel merges the states: one
+    // more launch, which pays from 8 splits on.
+    if (t.long_context_splits) {
+        const int n = std::min({256 / std::max(pairs, 1), max_ctx_len / 512, 64});
+        if (n >= 8) {
+            const int keys = (max_ctx_len + n - 1) / n;
+            *nsplit = n;
+            *waves = std::max(2, std::min(12, (keys + 63) / 64));
+            *merge_kernel = true;
             return;
         }
     }
@@ -380,8 +396,9 @@ bool paged_attention(const AttentionArgs& a, AttentionSplits* splits, hipStream_
         bool unmerged = a.may_split && splits != nullptr && a.q.dtype == BF16 && T <= tuning().merge_max_rows &&
                         a.head_dim % 8 == 0 && tuning().decode_nsplit == 0;
         int nsplit = 1, waves = 12;
-        decode_launch_shape(pairs, a.max_ctx_len, unmerged, &nsplit, &waves);
-        unmerged = unmerged && nsplit > 1;
+        bool merge_kernel = false;
+        decode_launch_shape(pairs, a.max_ctx_len, unmerged, &nsplit, &waves, &merge_kernel);
+        unmerged = unmerged && nsplit > 1 && !merge_kernel;
         float* ws = decode_partials(nsplit > 1 ? static_cast<size_t>(pairs) * nsplit * (a.head_dim + 2) : 1);
         int* counters = decode_counters(pairs);
         // every sequence of the batch brings one token: token t is sequence t, and the kernel need not load that
@@ -389,8 +406,11 @@ bool paged_attention(const AttentionArgs& a, AttentionSplits* splits, hipStream_
         check(mllm_decode_attention(a.q.data, static_cast<int>(a.q.stride), a.q_col, a.k_pages.data, a.v_pages.data, kv_dim,
                                     a.block_tables, a.max_blocks, seq_of_token, a.positions, T, a.n_heads, a.n_kv_heads,
                                     a.head_dim, a.page_size, a.scale, a.window, nsplit, waves, a.out.data,
-                                    static_cast<int>(a.out.stride), ws, counters, a.k_col, a.v_col, slots, unmerged ? 1 : 0,
-                                    a.q.dtype, stream), "decode_attention");
+                                    static_cast<int>(a.out.stride), ws, counters, a.k_col, a.v_col, slots,
+                                    unmerged || merge_kernel ? 1 : 0, a.q.dtype, stream), "decode_attention");
+        if (merge_kernel)
+            check(mllm_merge_attention_splits(ws, T, a.n_heads, a.head_dim, nsplit, a.out.data, static_cast<int>(a.out.stride),
+                                              a.q.dtype, stream), "merge_splits");
         if (unmerged) {
             splits->ws = ws;
             splits->n_tokens = T;

@@ -98,6 +98,7 @@ struct Tuning {
     int decode_nsplit = 0, decode_waves = 0;          // > 0: forced launch shape of merged decode attention
     int unmerged_nsplit = 0, unmerged_waves = 0;      // > 0: forced shape of splits merged by the next product
     int merge_max_rows = 16;                          // tokens whose splits a product merges while loading
+    int long_context_splits = 1;                      // 1: few pairs with long contexts are split over up to 256 workgroups
     int ln_fuse_max_rows = 32;                        // rows up to which the norm is fused into the few-row product
 };
 Tuning& tuning();

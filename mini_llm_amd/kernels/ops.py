@@ -203,6 +203,7 @@ def reserve_scratch(device, rows: int, vocab: int, n_heads: int = 0, head_dim: i
 DECODE_SHAPE_OVERRIDE = None      # (nsplit, waves): forced launch shape of decode attention merged in its kernel
 DECODE_UNMERGED_SHAPE = None      # (nsplit, waves): forced shape of splits that the next product merges
 MERGE_MAX_ROWS = 16               # tokens whose attention splits a product merges while loading (one row block)
+LONG_CONTEXT_SPLITS = True        # few pairs with long contexts: keys split over up to 256 workgroups, merged by a small kernel
 LN_FUSE_MAX_ROWS = 32             # rows up to which the few-row product normalises its input itself (measured: 1-2 % of
                                   # a decode step gained at 24 and 32 rows, 3 % lost at 64)
 _pushed_tuning = None
@@ -211,7 +212,7 @@ _pushed_tuning = None
 def push_tuning() -> None:
     """Hands the module's tuning values to the native side if they have changed."""
     global _pushed_tuning
-    now = (DECODE_SHAPE_OVERRIDE, DECODE_UNMERGED_SHAPE, MERGE_MAX_ROWS, LN_FUSE_MAX_ROWS)
+    now = (DECODE_SHAPE_OVERRIDE, DECODE_UNMERGED_SHAPE, MERGE_MAX_ROWS, LN_FUSE_MAX_ROWS, LONG_CONTEXT_SPLITS)
     if now == _pushed_tuning:
         return
     lib = engine_library()
@@ -221,6 +222,7 @@ def push_tuning() -> None:
     _ok(lib.mllm_set_tuning(b"unmerged_shape", int(a), int(b)))
     _ok(lib.mllm_set_tuning(b"merge_max_rows", int(MERGE_MAX_ROWS), 0))
     _ok(lib.mllm_set_tuning(b"ln_fuse_max_rows", int(LN_FUSE_MAX_ROWS), 0))
+    _ok(lib.mllm_set_tuning(b"long_context_splits", 1 if LONG_CONTEXT_SPLITS else 0, 0))
     _pushed_tuning = now
 
 

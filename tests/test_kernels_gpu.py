@@ -641,6 +641,26 @@ def test_paged_attention_long_contexts(ops, dtype, H, Hkv, dh, page):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+def test_decode_attention_splits_long_contexts_over_the_chip(ops, dtype):
+    """Few pairs with thousands of keys: the keys of a pair are split over up to 256 workgroups and a small
+    kernel merges their states. Same result as one workgroup a pair, with a short sequence beside the long
+    ones (splits that hold no key) and with a window."""
+    g = torch.Generator().manual_seed(5)
+    for seqs, window in (([(6000, 1), (3, 1), (4500, 1)], 0), ([(9000, 1)], 0), ([(7000, 1), (5000, 1)], 1300)):
+        results = []
+        for on in (True, False):
+            ops.LONG_CONTEXT_SPLITS = on
+            try:
+                gg = torch.Generator().manual_seed(int(g.initial_seed()) + len(seqs))
+                out, ref = _attention_case(ops, dtype, 6, 2, 64, 16, seqs, window, gg)
+            finally:
+                ops.LONG_CONTEXT_SPLITS = True
+            assert (out - ref).abs().max() <= _tol(dtype, 2), (seqs, window, on)
+            results.append(out)
+        assert (results[0] - results[1]).abs().max() <= _tol(dtype, 2)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
 def test_paged_attention_far_key_stands_out(ops, dtype):
     """One key hundreds of positions back carries almost all the weight of the last query."""
     g = torch.Generator().manual_seed(7)
