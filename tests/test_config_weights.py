@@ -275,3 +275,32 @@ def test_sizes_the_kernels_cannot_take_are_refused_when_the_model_is_built(tmp_p
     with pytest.raises(ValueError, match="head"):
         write_random_model(cfg2, d2, seed=0)
         load_model(d2, "float32", "cpu")
+
+
+def test_the_native_program_writes_the_same_model_folder(tmp_path):
+    """`mini-llm make-model` (C++: its own JSON, generator and safetensors writer) and `write_random_model`
+    (Python) make the same folder from a preset and a seed: the tensor file byte for byte, the same
+    configuration. No GPU is needed for it."""
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    native = str(tmp_path / "native")
+    r = subprocess.run([sys.executable, os.path.join(root, "bin", "mini-llm"), "make-model", "--preset", "tiny-b",
+                        "--seed", "5", "--out", native], capture_output=True, text=True, timeout=900)
+    assert r.returncode == 0, r.stderr
+    preset = json.load(open(os.path.join(root, "mini_llm_amd", "config", "presets", "tiny-b.json")))
+    python = write_random_model(dict(preset), str(tmp_path / "python"), seed=5)
+    with open(os.path.join(native, "model.safetensors"), "rb") as a, open(os.path.join(python, "model.safetensors"), "rb") as b:
+        assert a.read() == b.read()
+    assert json.load(open(os.path.join(native, "config.json"))) == json.load(open(os.path.join(python, "config.json")))
+    for dtype in ("float32",):
+        r = subprocess.run([sys.executable, os.path.join(root, "bin", "mini-llm"), "make-model", "--preset", "tiny-a",
+                            "--seed", "0", "--weights-dtype", dtype, "--out", native + dtype], capture_output=True, text=True, timeout=900)
+        assert r.returncode == 0, r.stderr
+        preset = json.load(open(os.path.join(root, "mini_llm_amd", "config", "presets", "tiny-a.json")))
+        python = write_random_model(dict(preset), str(tmp_path / ("python" + dtype)), seed=0, weights_dtype=dtype)
+        with open(os.path.join(native + dtype, "model.safetensors"), "rb") as a, open(os.path.join(python, "model.safetensors"), "rb") as b:
+            assert a.read() == b.read()
+    bad = subprocess.run([sys.executable, os.path.join(root, "bin", "mini-llm"), "make-model", "--preset", "nothing",
+                          "--seed", "0", "--out", native + "x"], capture_output=True, text=True, timeout=900)
+    assert bad.returncode == 1 and "unknown preset" in bad.stderr
