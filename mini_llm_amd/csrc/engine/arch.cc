@@ -90,6 +90,23 @@ std::unique_ptr<LoadedModel> load_model(const std::string& model_dir, int dtype)
     return build(config, source, dtype, model_dir);
 }
 
+ModelFolderSummary check_model_dir(const std::string& model_dir) {
+    const Json config = read_config(model_dir);
+    const Architecture& a = architecture_of(config);
+    const auto specs = a.param_specs(config);
+    CheckpointSource source(model_dir);
+    check_checkpoint(specs, source, a.optional_prefixes, a.ignored_tensor, model_dir);
+    ModelFolderSummary s;
+    s.architecture = a.name;
+    s.n_tensors = static_cast<int>(specs.size());
+    for (const auto& sp : specs) {
+        int64_t n = 1;
+        for (int64_t d : sp.shape) n *= d;
+        s.n_parameters += n;
+    }
+    return s;
+}
+
 std::unique_ptr<LoadedModel> random_model(const Json& config, uint64_t seed, int dtype, const std::string& weights_dtype) {
     RandomSource source(seed, weights_dtype);
     return build(config, source, dtype, "random weights");

@@ -59,6 +59,14 @@ std::vector<std::string> registered_architectures();
 Json read_config(const std::string& model_dir);
 // dtype: BF16 or F32
 std::unique_ptr<LoadedModel> load_model(const std::string& model_dir, int dtype);
+// Reads a folder's config.json and tensor headers and checks them against the architecture (the
+// configuration's refusals, then names and shapes, all mismatches in one WeightsError). No device is touched.
+struct ModelFolderSummary {
+    std::string architecture;
+    int n_tensors = 0;
+    int64_t n_parameters = 0;
+};
+ModelFolderSummary check_model_dir(const std::string& model_dir);
 std::unique_ptr<LoadedModel> random_model(const Json& config, uint64_t seed, int dtype,
                                           const std::string& weights_dtype = "bfloat16");
 // a preset by name: config/presets/<name>.json beside the package

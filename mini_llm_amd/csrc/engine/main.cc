@@ -191,6 +191,18 @@ int cmd_generate(int argc, char** argv) {
     return 0;
 }
 
+// check --model DIR: configuration and tensors against the architecture, without a GPU
+int cmd_check(int argc, char** argv) {
+    const Args a = parse_args(argc, argv, 2, {"model"}, {});
+    if (!a.has("model")) {
+        std::fprintf(stderr, "usage: mini-llm check --model DIR\n");
+        return 1;
+    }
+    const ModelFolderSummary s = check_model_dir(a.get("model"));
+    std::printf("ok: %s, %d tensors, %lld parameters\n", s.architecture.c_str(), s.n_tensors, static_cast<long long>(s.n_parameters));
+    return 0;
+}
+
 int cmd_make_model(int argc, char** argv) {
     const Args a = parse_args(argc, argv, 2, {"preset", "config", "seed", "out", "weights-dtype"}, {});
     if (a.has("preset") == a.has("config") || !a.has("seed") || !a.has("out")) {
@@ -278,17 +290,19 @@ int main(int argc, char** argv) {
         if (cmd == "generate") return cmd_generate(argc, argv);
         if (cmd == "make-model") return cmd_make_model(argc, argv);
         if (cmd == "replay") return cmd_replay(argc, argv);
+        if (cmd == "check") return cmd_check(argc, argv);
     } catch (const std::exception& e) {
         std::fprintf(stderr, "mini-llm: %s\n", e.what());
         return 1;
     }
     std::fprintf(stderr,
-                 "usage: mini-llm generate|make-model|replay [options]\n"
+                 "usage: mini-llm generate|make-model|replay|check [options]\n"
                  "  generate   --model DIR | --preset NAME [--weights-seed S]  [--dtype bfloat16|float32] [--prompt-ids \"1 2 3\"]...\n"
                  "             [--prompts-file F] [--max-new-tokens 8] [--temperature 0] [--seed 0] [--ignore-eos] [--stream] [--stats]\n"
                  "             [--kv-block-size 16] [--total-kv-blocks 4096 | --kv-memory-fraction F] [--max-batch-num 16] [--max-tokens-per-step 2048]\n"
                  "             [--prefill-chunk 512]\n"
                  "  make-model (--preset NAME | --config FILE) --seed S --out DIR [--weights-dtype bfloat16|float32]\n"
-                 "  replay     --model DIR --dtype bfloat16|float32 --out DIR --max-tokens N [--page-size 16]\n");
+                 "  replay     --model DIR --dtype bfloat16|float32 --out DIR --max-tokens N [--page-size 16]\n"
+                 "  check      --model DIR     (configuration and tensors against the architecture; needs no GPU)\n");
     return cmd.empty() || cmd == "--help" || cmd == "-h" ? (cmd.empty() ? 1 : 0) : 1;
 }

@@ -307,15 +307,14 @@ static std::string shape_text(const std::vector<int64_t>& s) {
     return t + "]";
 }
 
-std::map<std::string, Tensor2> load_tensors(const std::vector<ParamSpec>& specs, const TensorSource& source,
-                                            int compute_dtype, DeviceTensors& store,
-                                            const std::vector<std::string>& optional_prefixes,
-                                            const std::function<bool(const std::string&)>& ignored,
-                                            const std::string& where) {
+std::map<std::string, std::string> check_checkpoint(const std::vector<ParamSpec>& specs, const TensorSource& source,
+                                                    const std::vector<std::string>& optional_prefixes,
+                                                    const std::function<bool(const std::string&)>& ignored,
+                                                    const std::string& where) {
     std::map<std::string, const ParamSpec*> by_name;
     for (const auto& s : specs) by_name[s.name] = &s;
     std::map<std::string, std::string> available;     // short name -> stored name
-    if (!source.generates()) {
+    {
         for (const std::string& name : source.names()) {
             std::string short_name = name;
             if (!by_name.count(name)) {
@@ -348,6 +347,16 @@ std::map<std::string, Tensor2> load_tensors(const std::vector<ParamSpec>& specs,
             throw WeightsError(msg);
         }
     }
+    return available;
+}
+
+std::map<std::string, Tensor2> load_tensors(const std::vector<ParamSpec>& specs, const TensorSource& source,
+                                            int compute_dtype, DeviceTensors& store,
+                                            const std::vector<std::string>& optional_prefixes,
+                                            const std::function<bool(const std::string&)>& ignored,
+                                            const std::string& where) {
+    std::map<std::string, std::string> available;     // short name -> stored name
+    if (!source.generates()) available = check_checkpoint(specs, source, optional_prefixes, ignored, where);
     std::map<std::string, Tensor2> out;
     std::vector<float> values, turned;
     for (const auto& s : specs) {

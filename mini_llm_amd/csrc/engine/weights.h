@@ -144,6 +144,14 @@ private:
     size_t bytes_ = 0;
 };
 
+// Compares what a checkpoint holds with what the model expects (names, with an optional prefix accepted and
+// `ignored` names skipped; shapes) and returns spec name -> stored name. ONE WeightsError lists missing,
+// unexpected and wrong-shape tensors. Touches no device.
+std::map<std::string, std::string> check_checkpoint(const std::vector<ParamSpec>& specs, const TensorSource& source,
+                                                    const std::vector<std::string>& optional_prefixes,
+                                                    const std::function<bool(const std::string&)>& ignored,
+                                                    const std::string& where);
+
 // Looks every spec up in the source (an optional name prefix is accepted, `ignored` names are skipped),
 // checks shapes, converts (matrices -> compute dtype, transposed once if stored [in, out]; vectors -> fp32)
 // and uploads. ONE WeightsError lists missing, unexpected and wrong-shape tensors.

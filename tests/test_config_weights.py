@@ -304,3 +304,59 @@ def test_the_native_program_writes_the_same_model_folder(tmp_path):
     bad = subprocess.run([sys.executable, os.path.join(root, "bin", "mini-llm"), "make-model", "--preset", "nothing",
                           "--seed", "0", "--out", native + "x"], capture_output=True, text=True, timeout=900)
     assert bad.returncode == 1 and "unknown preset" in bad.stderr
+
+
+def _native_check(folder):
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    r = subprocess.run([sys.executable, os.path.join(root, "bin", "mini-llm"), "check", "--model", str(folder)],
+                       capture_output=True, text=True, timeout=900)
+    return r.returncode, r.stdout + r.stderr
+
+
+def test_the_native_loader_checks_a_folder_without_a_gpu(tmp_path):
+    """`mini-llm check` runs the C++ side's configuration, safetensors reader and name/shape check: the
+    same verdicts as the Python loader, every mismatch in one message."""
+    d = write_random_model(dict(TINY_A), str(tmp_path / "m"), seed=0)
+    rc, out = _native_check(d)
+    good = _tensors(d)
+    n_params = sum(t.numel() for t in good.values())
+    assert rc == 0 and f"ok: GPT2LMHeadModel, {len(good)} tensors, {n_params} parameters" in out, out
+    # the prefix and the mask buffers of exported checkpoints are accepted
+    t = {"transformer." + k: v for k, v in good.items()}
+    t["transformer.h.0.attn.bias"] = torch.ones(1, 1, 8, 8)
+    t["lm_head.weight"] = t["transformer.wte.weight"].clone()
+    save_file(t, os.path.join(d, "model.safetensors"))
+    assert _native_check(d)[0] == 0
+    # every mismatch in one message
+    t = dict(good)
+    del t["h.1.ln_2.bias"], t["wpe.weight"]
+    t["h.0.mlp.c_fc.weight"] = torch.zeros(256, 64, dtype=torch.bfloat16)
+    t["h.7.extra.weight"] = torch.zeros(2)
+    save_file(t, os.path.join(d, "model.safetensors"))
+    rc, out = _native_check(d)
+    assert rc == 1
+    for piece in ("missing tensors (2)", "h.1.ln_2.bias", "wpe.weight", "unexpected tensors (1)", "h.7.extra.weight",
+                  "wrong shapes (1)", "expected [64, 256], found [256, 64]"):
+        assert piece in out, (piece, out)
+    # files that are no safetensors files
+    raw = open(os.path.join(d, "model.safetensors"), "rb").read()
+    for broken, match in ((raw[:5], "too short"), ((10 ** 9).to_bytes(8, "little") + raw[8:], "header length"),
+                          (raw[:8] + b"{" * 20 + raw[28:], "JSON"), (raw[:len(raw) // 2], "offsets")):
+        open(os.path.join(d, "model.safetensors"), "wb").write(broken)
+        rc, out = _native_check(d)
+        assert rc == 1 and match in out, (match, out)
+    os.remove(os.path.join(d, "model.safetensors"))
+    rc, out = _native_check(d)
+    assert rc == 1 and "neither model.safetensors" in out
+    # the configuration is judged first
+    cfg = json.load(open(os.path.join(d, "config.json")))
+    json.dump(dict(cfg, n_head=5), open(os.path.join(d, "config.json"), "w"))
+    rc, out = _native_check(d)
+    assert rc == 1 and "divisible" in out
+    json.dump(dict(cfg, architectures=["Other"], model_type="other"), open(os.path.join(d, "config.json"), "w"))
+    rc, out = _native_check(d)
+    assert rc == 1 and "no known architecture" in out and "GPT2LMHeadModel" in out
+    open(os.path.join(d, "config.json"), "w").write("{not json")
+    assert _native_check(d)[0] == 1
