@@ -151,12 +151,12 @@ int cmd_generate(int argc, char** argv) {
     else
         engine = Engine::from_pretrained(a.get("model"), dtype, o);
     const bool stream = a.has("stream");
-    std::vector<std::string> verdict(lines.size());         // a message instead of tokens
+    std::vector<std::string> answer(lines.size());         // a message instead of tokens
     std::vector<std::vector<int>> tokens(lines.size());
     std::map<int64_t, size_t> index_of;
     std::vector<int> ids;
     for (size_t i = 0; i < lines.size(); ++i) {
-        if (!parse_request(lines[i], ids)) { verdict[i] = "invalid request"; continue; }
+        if (!parse_request(lines[i], ids)) { answer[i] = "invalid request"; continue; }
         SamplingParams sp;
         sp.temperature = static_cast<float>(a.real("temperature", 0.0));
         sp.seed = static_cast<uint64_t>(a.integer("seed", 0)) + i;
@@ -165,20 +165,20 @@ int cmd_generate(int argc, char** argv) {
         try {
             index_of[engine->add_request(ids, sp)] = i;
         } catch (const EngineError& e) {
-            verdict[i] = std::string("invalid request (") + e.what() + ")";
+            answer[i] = std::string("invalid request (") + e.what() + ")";
         }
     }
     while (engine->has_unfinished()) {
         for (const RequestOutput& out : engine->step()) {
             const size_t i = index_of.at(out.request_id);
-            if (out.token < 0) { verdict[i] = "failed: " + out.error; continue; }
+            if (out.token < 0) { answer[i] = "failed: " + out.error; continue; }
             tokens[i].push_back(out.token);
             if (stream) { std::printf("%zu %d%s\n", i, out.token, out.finished ? " [DONE]" : ""); std::fflush(stdout); }
         }
     }
     if (!stream) {
         for (size_t i = 0; i < lines.size(); ++i) {
-            if (!verdict[i].empty()) { std::printf("%s\n", verdict[i].c_str()); continue; }
+            if (!answer[i].empty()) { std::printf("%s\n", answer[i].c_str()); continue; }
             for (int t : tokens[i]) std::printf("%d ", t);
             std::printf("[DONE]\n");
         }

@@ -317,7 +317,7 @@ def _native_check(folder):
 
 def test_the_native_loader_checks_a_folder_without_a_gpu(tmp_path):
     """`mini-llm check` runs the C++ side's configuration, safetensors reader and name/shape check: the
-    same verdicts as the Python loader, every mismatch in one message."""
+    same findings as the Python loader, every mismatch in one message."""
     d = write_random_model(dict(TINY_A), str(tmp_path / "m"), seed=0)
     rc, out = _native_check(d)
     good = _tensors(d)
