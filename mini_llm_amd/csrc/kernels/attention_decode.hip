@@ -214,10 +214,10 @@ decode_attention_kernel(// the first 16 dwords arrive in registers with the wave
     auto block_merge = [&]() {
 #pragma unroll
         for (int off = LPK; off < MLLM_WAVE; off <<= 1) {
-            const float m2 = __shfl_xor(m, off, MLLM_WAVE), l2 = __shfl_xor(l, off, MLLM_WAVE);
+            const float m2 = lane_xor(m, off), l2 = lane_xor(l, off);
             float o2[EPL];
 #pragma unroll
-            for (int e = 0; e < EPL; ++e) o2[e] = __shfl_xor(o[e], off, MLLM_WAVE);
+            for (int e = 0; e < EPL; ++e) o2[e] = lane_xor(o[e], off);
             merge_state<T, EPL>(m, l, o, m2, l2, o2);
         }
         __syncthreads();                      // earlier readers of the LDS arrays are done
@@ -241,10 +241,10 @@ decode_attention_kernel(// the first 16 dwords arrive in registers with the wave
             }
 #pragma unroll
             for (int off = LPK; off < MLLM_WAVE; off <<= 1) {
-                const float m2 = __shfl_xor(m, off, MLLM_WAVE), l2 = __shfl_xor(l, off, MLLM_WAVE);
+                const float m2 = lane_xor(m, off), l2 = lane_xor(l, off);
                 float o2[EPL];
 #pragma unroll
-                for (int e = 0; e < EPL; ++e) o2[e] = __shfl_xor(o[e], off, MLLM_WAVE);
+                for (int e = 0; e < EPL; ++e) o2[e] = lane_xor(o[e], off);
                 merge_state<T, EPL>(m, l, o, m2, l2, o2);
             }
         }

@@ -85,6 +85,54 @@ constexpr int DPP_ROW_MIRROR = 0x140;     // lane i <-> 15 - i within 16
 __device__ __forceinline__ float row_lane(float v, int lane) {
     return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), lane));
 }
+// Exchange between the rows of 16 lanes, on the vector ALU: gfx950's v_permlane16_swap exchanges the odd
+// rows of its first operand with the even rows of its second, v_permlane32_swap the upper half of the
+// first with the lower half of the second. Given the same value twice, the two results hold, in every
+// lane, the lane's own value and that of lane ^ 16 (lane ^ 32), in an order that depends on the lane: a
+// commutative operation on the pair is the exchange-and-combine step of a reduction, without the trip
+// through LDS that __shfl_xor makes (ds_bpermute).
+__device__ __forceinline__ void lane_pair_16(float v, float& a, float& b) {
+    const unsigned u = __builtin_bit_cast(unsigned, v);
+    const auto r = __builtin_amdgcn_permlane16_swap(u, u, false, false);
+    a = __builtin_bit_cast(float, static_cast<unsigned>(r[0]));
+    b = __builtin_bit_cast(float, static_cast<unsigned>(r[1]));
+}
+__device__ __forceinline__ void lane_pair_32(float v, float& a, float& b) {
+    const unsigned u = __builtin_bit_cast(unsigned, v);
+    const auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+    a = __builtin_bit_cast(float, static_cast<unsigned>(r[0]));
+    b = __builtin_bit_cast(float, static_cast<unsigned>(r[1]));
+}
+// The value of lane (l ^ off) for off = 8, 16 or 32 on the vector ALU (a rotation by 8 within the row of 16
+// lanes; the row swaps above and a select); other distances go through LDS. `off` is a constant once the
+// caller's loop is unrolled.
+constexpr int DPP_ROW_ROR_8 = 0x128;      // lane i <- lane (i + 8) % 16 of its row
+__device__ __forceinline__ float lane_xor(float v, int off) {
+    if (off == 8) return dpp_move<DPP_ROW_ROR_8>(v);
+    if (off == 16 || off == 32) {
+        float a, b;
+        if (off == 16) lane_pair_16(v, a, b); else lane_pair_32(v, a, b);
+        return (threadIdx.x & off) ? a : b;      // (wavefronts start at multiples of 64 threads)
+    }
+    return __shfl_xor(v, off, MLLM_WAVE);
+}
+
+// Maximum / sum over the four lanes l, l ^ 16, l ^ 32, l ^ 48 (one lane of each row), in all four.
+__device__ __forceinline__ float rows_max(float v) {
+    float a, b;
+    lane_pair_16(v, a, b);
+    v = fmaxf(a, b);
+    lane_pair_32(v, a, b);
+    return fmaxf(a, b);
+}
+__device__ __forceinline__ float rows_sum(float v) {
+    float a, b;
+    lane_pair_16(v, a, b);
+    v = a + b;
+    lane_pair_32(v, a, b);
+    return a + b;
+}
+
 // Sum over aligned groups of LANES consecutive lanes (a power of two), in every lane of the group.
 template <int LANES>
 __device__ __forceinline__ float group_sum(float v) {

@@ -45,6 +45,26 @@ def test_loaded_libraries_are_in_tree(ops):
     assert all(os.path.dirname(os.path.realpath(m)) == os.path.realpath(build.LIB_DIR) for m in mapped), mapped
 
 
+def test_lane_exchange_between_rows(ops):
+    """The reductions over one lane of each 16-lane row (built on gfx950's row swaps) against their meaning."""
+    import ctypes
+    from mini_llm_amd import build
+    lib = build.load_library("peaks")
+    g = torch.Generator().manual_seed(3)
+    v = torch.randn(64, generator=g)
+    out = torch.zeros(384, device=DEV)
+    rc = lib.mllm_rows_check(ctypes.c_void_p(v.to(DEV).data_ptr()), ctypes.c_void_p(out.data_ptr()),
+                             ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
+    assert rc == 0
+    groups = v.view(4, 16)
+    assert torch.equal(out[:64].cpu().view(4, 16), groups.max(0).values.expand(4, 16))
+    want = (groups[0] + groups[1]) + (groups[2] + groups[3])
+    assert torch.equal(out[64:128].cpu().view(4, 16), want.expand(4, 16))
+    lanes = torch.arange(64)
+    for i, off in enumerate((8, 16, 32, 4)):
+        assert torch.equal(out[128 + 64 * i:192 + 64 * i].cpu(), v[lanes ^ off]), off
+
+
 def test_ops_refuse_cpu_tensors(ops):
     x = torch.zeros(2, 8)
     with pytest.raises(ops.KernelError, match="not on the GPU"):
