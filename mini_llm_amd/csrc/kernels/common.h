@@ -73,7 +73,7 @@ __device__ __forceinline__ void load8(const bf16_t* p, float (&v)[8]) {
 // 16 lanes the values move through the DPP path of the vector ALU (lane swaps inside quads, then
 // the mirrored half row and the mirrored row: after each step all lanes of the growing group hold
 // the group's result, since the operation is commutative), the four row results are read as
-// scalars. A shuffle through LDS (__shfl_xor) has several times the latency per step.
+// scalars. A shuffle through LDS (__shfl_xor, ds_bpermute) has several times the latency per step.
 template <int CTRL>
 __device__ __forceinline__ float dpp_move(float v) {
     return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xF, 0xF, false));
@@ -141,8 +141,8 @@ __device__ __forceinline__ float group_sum(float v) {
     if (LANES >= 4) v += dpp_move<DPP_SWAP_2>(v);
     if (LANES >= 8) v += dpp_move<DPP_HALF_MIRROR>(v);
     if (LANES >= 16) v += dpp_move<DPP_ROW_MIRROR>(v);
-    if (LANES >= 32) v += __shfl_xor(v, 16, MLLM_WAVE);
-    if (LANES >= 64) v += __shfl_xor(v, 32, MLLM_WAVE);
+    if (LANES >= 32) v += lane_xor(v, 16);
+    if (LANES >= 64) v += lane_xor(v, 32);
     return v;
 }
 __device__ __forceinline__ float wave_sum(float v) {
