@@ -192,12 +192,16 @@ def serving_main(args, cfg, model_dir):
            "config": {"model": args.size + "-sizes", "n_layer": cfg["n_layer"], "n_layer_full": SIZES[args.size][0],
                       "requests": n_req, "prompt_min": lo, "prompt_max": hi, "new_tokens": new,
                       "max_batch_num": max_batch, "prefill_chunk": chunk, "kv_blocks": pages, "kv_block_size": 16,
-                      "engine": args.engine,
-                      "prompt_tokens": r["prompt_tokens"], "generated_tokens": r["generated"],
-                      "total_tok_per_s": round((r["generated"] + r["prompt_tokens"]) / r["seconds"], 1),
-                      "seconds": round(r["seconds"], 3), "first_token_ms": round(1e3 * (r["first_token_s"] or 0), 2),
-                      "preemptions": c["preemptions"], "deferred_decodes": c["deferred_decodes"],
-                      "deferred_prefills": c["deferred_prefills"], "failed": r["failed"]}}
+                      "engine": args.engine},
+           # what the run did (the configuration above holds sizes only)
+           "serving": {"prompt_tokens": r["prompt_tokens"], "generated_tokens": r["generated"],
+                       "total_tok_per_s": round((r["generated"] + r["prompt_tokens"]) / r["seconds"], 1),
+                       "seconds": round(r["seconds"], 3), "first_token_ms": round(1e3 * (r["first_token_s"] or 0), 2),
+                       # mean composition of a step: decoded tokens and prompt tokens in it
+                       "decode_rows_per_step": round(r["generated"] / r["steps"], 1),
+                       "prompt_tokens_per_step": round(r["prompt_tokens"] / r["steps"], 1),
+                       "preemptions": c["preemptions"], "deferred_decodes": c["deferred_decodes"],
+                       "deferred_prefills": c["deferred_prefills"], "failed": r["failed"]}}
     print(json.dumps(rec))
     return 0
 
