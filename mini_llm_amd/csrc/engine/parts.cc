@@ -1,8 +1,61 @@
 #include "parts.h"
 
 #include <algorithm>
+#include <cstdio>
+#include <cstdlib>
 
 namespace minillm {
+
+// ---------------------------------------------------------------------------------------------
+// stage times
+// ---------------------------------------------------------------------------------------------
+StageTimes::StageTimes() : enabled_(std::getenv("MINI_LLM_STAGE_TIMES") != nullptr) {}
+
+StageTimes& StageTimes::get() {
+    static StageTimes t;
+    return t;
+}
+
+hipEvent_t StageTimes::event(hipStream_t s) {
+    hipEvent_t e = nullptr;
+    if (!spare_.empty()) { e = spare_.back(); spare_.pop_back(); }
+    else if (hipEventCreate(&e) != hipSuccess) fail("stage times: an event could not be created");
+    if (hipEventRecord(e, s) != hipSuccess) fail("stage times: an event could not be recorded");
+    return e;
+}
+
+void StageTimes::begin_step(const char* kind, int batch, int tokens, hipStream_t s) {
+    if (!enabled_) return;
+    // (a step that is being captured into a graph is not timed: its events would become part of the graph)
+    hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(s, &capturing) != hipSuccess || capturing != hipStreamCaptureStatusNone) { start_ = nullptr; return; }
+    kind_ = kind; batch_ = batch; tokens_ = tokens; layer_ = -1;
+    start_ = event(s);
+}
+
+void StageTimes::mark(const char* stage, hipStream_t s) {
+    if (!enabled_ || start_ == nullptr) return;
+    marks_.push_back(Mark{layer_, stage, event(s)});
+}
+
+void StageTimes::end_step(hipStream_t s) {
+    if (!enabled_ || start_ == nullptr) return;
+    if (!marks_.empty() && hipEventSynchronize(marks_.back().at) != hipSuccess) fail("stage times: the step failed");
+    if (!header_) { std::fprintf(stderr, "kind,batch_size,total_tokens,layer,stage,ms\n"); header_ = true; }
+    hipEvent_t before = start_;
+    for (const Mark& m : marks_) {
+        float ms = 0.f;
+        (void)hipEventElapsedTime(&ms, before, m.at);
+        std::fprintf(stderr, "%s,%d,%d,%d,%s,%.4f\n", kind_, batch_, tokens_, m.layer, m.stage, ms);
+        spare_.push_back(before);
+        before = m.at;
+    }
+    spare_.push_back(before);
+    marks_.clear();
+    start_ = nullptr;
+    (void)s;
+}
+
 
 // ---------------------------------------------------------------------------------------------
 void* Arena::take(size_t bytes) {
@@ -143,6 +196,7 @@ public:
             kv.q_cols = q_dim_;
         }
         h.linear(qkv_, qkv, STORE, scatter ? &kv : nullptr, arena, s);
+        StageTimes::get().mark("qkv", s);
         AttentionArgs a;
         a.q = qkv;
         a.q_col = 0;
@@ -173,8 +227,11 @@ public:
         AttentionSplits splits;
         // (the result may come back unmerged, as the states of several workgroups per token and head:
         // the output projection takes either)
-        if (paged_attention(a, &splits, s)) linear_from_splits(splits, out_.weight, out_.bias, x, ADD_RESIDUAL, a.out.data, s);
+        const bool unmerged = paged_attention(a, &splits, s);
+        StageTimes::get().mark("attention", s);
+        if (unmerged) linear_from_splits(splits, out_.weight, out_.bias, x, ADD_RESIDUAL, a.out.data, s);
         else out_(a.out, x, ADD_RESIDUAL, nullptr, s);
+        StageTimes::get().mark("out_proj", s);
     }
     size_t workspace_bytes(int tokens) const override {
         return static_cast<size_t>(tokens) * (2 * q_dim_ + 2 * kv_dim_) * dtype_size(dtype_) + 1024;
@@ -203,7 +260,9 @@ public:
     void forward(NormedInput& h, const StepView& step, const Tensor2& x, Arena& arena, hipStream_t s) const override {
         Tensor2 inner = arena.tensor(dtype_, step.n_tokens, up_.out_features());
         h.linear(up_, inner, act_, nullptr, arena, s);
+        StageTimes::get().mark("fc1", s);
         down_(inner, x, ADD_RESIDUAL, nullptr, s);
+        StageTimes::get().mark("fc2", s);
     }
     size_t workspace_bytes(int tokens) const override {
         return static_cast<size_t>(tokens) * up_.out_features() * dtype_size(dtype_) + 512;
@@ -329,21 +388,28 @@ void DecoderModel::forward(const StepView& step, const std::vector<CacheView>& c
                            const Tensor2& logits, hipStream_t s) const {
     if (step.n_tokens < 1) fail("a step needs at least one token");
     // x[t,:] = wte[id[t],:] (+ the position table's row, fused into the same kernel)
+    StageTimes& times = StageTimes::get();
+    times.begin_step(step.max_q_len == 1 ? "decode" : (step.n_single > 0 ? "mixed" : "prefill"), step.n_seqs, step.n_tokens, s);
     Tensor2 x = arena.tensor(F32, step.n_tokens, hidden_size());
     embed(step.token_ids, step.positions, wte, wpe.data ? &wpe : nullptr, x, s);
+    times.mark("embed", s);
     for (const LayerCall& c : order) {
         if (c.layer < 0 || c.layer >= static_cast<int>(layers.size()) || c.cache < 0 || c.cache >= static_cast<int>(caches.size()))
             fail("the execution order names layer %d / cache %d, the model has %zu layers and %zu caches", c.layer, c.cache,
                  layers.size(), caches.size());
+        times.set_layer(c.layer);
         layers[c.layer]->forward(x, step, caches[c.cache], c.write, arena, s);
     }
-    if (step.n_logits == 0) return;
+    times.set_layer(-1);
+    if (step.n_logits == 0) { times.end_step(s); return; }
     // logits = norm(x[rows]) wte^T, fp32, no bias: the embedding matrix [V, D] is read in place as the
     // [N, K] operand (the reference builds a transposed copy: /root/reference/src/model/gpt2_model.cu:87-113)
     if (logits.rows != step.n_logits || logits.cols != vocab_size() || logits.dtype != F32)
         fail("logits must be float32 [%d, %d]", step.n_logits, vocab_size());
     Linear head(wte, nullptr);
     final_norm->linear(x, head, logits, STORE_F32, step.logit_rows, nullptr, arena, s);
+    times.mark("head", s);
+    times.end_step(s);
 }
 
 }  // namespace minillm

@@ -27,6 +27,35 @@
 
 namespace minillm {
 
+// Optional per-stage times of the native forward pass. With the environment variable MINI_LLM_STAGE_TIMES
+// set, every step records an event behind each stage (embedding; per layer the QKV product with its norm,
+// attention, output projection, first and second product of the feed-forward; final norm and head), waits
+// for the step once at its end, and prints one line per stage to standard error in the reference's format
+// `kind,batch_size,total_tokens,layer,stage,ms` (kind: prefill, decode or mixed)
+// (/root/reference/include/profiling/stage_timer.cuh:13-101, which synchronises the device around every
+// stage instead). Off: one branch per stage. A part of another kind marks its own stages with `mark`.
+class StageTimes {
+public:
+    static StageTimes& get();
+    bool enabled() const { return enabled_; }
+    void begin_step(const char* kind, int batch, int tokens, hipStream_t s);
+    void set_layer(int layer) { layer_ = layer; }
+    void mark(const char* stage, hipStream_t s);        // the stage that ends here
+    void end_step(hipStream_t s);                        // waits for the step and prints
+
+private:
+    StageTimes();
+    hipEvent_t event(hipStream_t s);
+    struct Mark { int layer; const char* stage; hipEvent_t at; };
+    bool enabled_ = false, header_ = false;
+    int layer_ = -1, batch_ = 0, tokens_ = 0;
+    const char* kind_ = "";
+    hipEvent_t start_ = nullptr;
+    std::vector<Mark> marks_;
+    std::vector<hipEvent_t> spare_;
+};
+
+
 // Memory for a step's temporaries: a bump allocator over one device buffer that the caller owns.
 class Arena {
 public:

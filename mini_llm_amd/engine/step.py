@@ -12,6 +12,8 @@ here they are built once per step and reach the device in one copy.
 """
 from __future__ import annotations
 
+import os
+
 import gc
 import weakref
 from dataclasses import dataclass, field
@@ -131,7 +133,10 @@ class ModelRunner:
         # Pure-decode batches may run from static buffers (`launch_decode`) unless a part of the model
         # plans on the host; on the GPU those steps are captured and replayed as HIP graphs.
         self.fast_decode = bool(getattr(model, "graph_safe", True))
-        self.use_graphs = self.device.type == "cuda" and self.fast_decode
+        # (with MINI_LLM_STAGE_TIMES set the native forward pass times its stages with events, which a
+        # replayed graph would not hold: every step is then launched as it is)
+        self.use_graphs = (self.device.type == "cuda" and self.fast_decode
+                           and os.environ.get("MINI_LLM_STAGE_TIMES") is None)
         # Kernel scratch is sized now for the largest decode batch, so that no captured graph is left
         # with the address of a buffer that a larger batch replaced; should one grow after all (a
         # step that wants more logits rows than that), the graphs are dropped and captured again.

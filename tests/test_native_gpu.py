@@ -281,3 +281,26 @@ def test_native_and_python_engines_agree_under_random_options(tiny_model_dirs):
         assert sa["preemptions"] == sb["preemptions"] and sa["deferred_decodes"] == sb["deferred_decodes"], (trial, sa, sb)
         preempted += sa["preemptions"] > 0
     assert preempted >= 3              # (the workloads do run out of pages)
+
+
+def test_stage_times_of_the_native_forward_pass(tiny_model_dirs):
+    """MINI_LLM_STAGE_TIMES: one line per stage and step on standard error, in the reference's format
+    (kind,batch_size,total_tokens,layer,stage,ms); the tokens on standard output are unchanged."""
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    cmd = [sys.executable, os.path.join(root, "bin", "mini-llm"), "generate", "--model", tiny_model_dirs["a"],
+           "--prompt-ids", "5 17 3 9 100", "--max-new-tokens", "4", "--ignore-eos", "--kv-block-size", "4",
+           "--total-kv-blocks", "32", "--no-overlap"]
+    plain = subprocess.run(cmd, capture_output=True, text=True, timeout=300)
+    timed = subprocess.run(cmd, capture_output=True, text=True, timeout=300, env=dict(os.environ, MINI_LLM_STAGE_TIMES="1"))
+    assert plain.returncode == 0 and timed.returncode == 0, (plain.stderr, timed.stderr)
+    assert plain.stdout == timed.stdout and plain.stdout.strip().endswith("[DONE]")
+    assert "kind,batch_size" not in plain.stderr
+    lines = [l for l in timed.stderr.splitlines() if l.count(",") == 5]
+    assert lines[0] == "kind,batch_size,total_tokens,layer,stage,ms"
+    rows = [l.split(",") for l in lines[1:]]
+    # four steps (the prompt, then three single tokens), each: embed, 2 layers x 5 stages, head
+    assert len(rows) == 4 * 12, timed.stderr
+    assert [r[4] for r in rows[:12]] == ["embed"] + ["qkv", "attention", "out_proj", "fc1", "fc2"] * 2 + ["head"]
+    assert [r[3] for r in rows[:12]] == ["-1"] + ["0"] * 5 + ["1"] * 5 + ["-1"]
+    assert rows[0][:3] == ["prefill", "1", "5"] and rows[12][:3] == ["decode", "1", "1"]
+    assert all(0.0 < float(r[5]) < 100.0 for r in rows)
