@@ -151,21 +151,37 @@ def serving_run(model_dir, dtype, cfg, n_req, prompt_lo, prompt_hi, new_tokens, 
     t0 = time.perf_counter()
     n_out = n_steps = failed = 0
     first = None
+    first_at, last_at, count = {}, {}, {}          # per request: when its first and its last token arrived, how many
     while engine.has_unfinished():
         outs = engine.step()
         n_steps += 1
+        now = time.perf_counter() - t0
         if outs and first is None:
             sync()
-            first = time.perf_counter() - t0
-        n_out += sum(1 for o in outs if o.token >= 0)
-        failed += sum(1 for o in outs if o.token < 0)
+            first = now = time.perf_counter() - t0
+        for o in outs:
+            if o.token >= 0:
+                n_out += 1
+                first_at.setdefault(o.request_id, now)
+                last_at[o.request_id] = now
+                count[o.request_id] = count.get(o.request_id, 0) + 1
+            else:
+                failed += 1
     sync()
     dt = time.perf_counter() - t0
+    # as the host sees them (tokens arrive one step late): time to the first token, time per later token, whole request
+    ttft = sorted(first_at.values())
+    e2e = sorted(last_at.values())
+    tpot = [(last_at[r] - first_at[r]) / (count[r] - 1) for r in count if count[r] > 1]
+    pct = lambda v, q: v[min(len(v) - 1, int(q * len(v)))] if v else 0.0
+    latency = {"ttft_ms_p50": round(1e3 * pct(ttft, 0.5), 2), "ttft_ms_p99": round(1e3 * pct(ttft, 0.99), 2),
+               "tpot_ms_mean": round(1e3 * sum(tpot) / max(len(tpot), 1), 3),
+               "e2e_ms_p50": round(1e3 * pct(e2e, 0.5), 1), "e2e_ms_p99": round(1e3 * pct(e2e, 0.99), 1)}
     st = engine.stats()
     assert n_out == (n_req - failed) * new_tokens, (n_out, n_req, failed, new_tokens)
     assert st["free_pages"] == pages and (native or engine.runner.manager.check() == "")
     return {"seconds": dt, "generated": n_out, "prompt_tokens": sum(lens), "steps": n_steps,
-            "first_token_s": first, "failed": failed, "counters": st}
+            "first_token_s": first, "failed": failed, "counters": st, "latency": latency}
 
 
 def serving_main(args, cfg, model_dir):
@@ -201,7 +217,7 @@ def serving_main(args, cfg, model_dir):
                        "decode_rows_per_step": round(r["generated"] / r["steps"], 1),
                        "prompt_tokens_per_step": round(r["prompt_tokens"] / r["steps"], 1),
                        "preemptions": c["preemptions"], "deferred_decodes": c["deferred_decodes"],
-                       "deferred_prefills": c["deferred_prefills"], "failed": r["failed"]}}
+                       "deferred_prefills": c["deferred_prefills"], "failed": r["failed"], **r["latency"]}}
     print(json.dumps(rec))
     return 0
 
