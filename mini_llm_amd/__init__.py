@@ -4,12 +4,12 @@
     engine = Engine.from_pretrained(model_dir, dtype="bfloat16")
     new_tokens = engine.generate([[15496, 11, 616]], SamplingParams(max_new_tokens=8))
 
-``Engine`` composes the model from parts in Python (any registered part, also ones written in
-Python) and runs it through the native step function; ``NativeEngine`` is the engine that is native
-from the loader to the sampler (the architectures registered natively), the one behind ``bin/mini-llm``.
+The engine is native (csrc/): configuration and registry, loader, parts, cache manager and storage,
+step function, scheduler, sampler, kernels; ``bin/mini-llm`` is its command line. This package is the
+thin Python entry over its C ABI.
 """
-from .engine.engine import Engine, EngineOptions, RequestOutput  # noqa: F401
-from .engine.native_engine import NativeEngine  # noqa: F401
-from .models import load_model  # noqa: F401
-from .sampling.sampler import SamplingParams  # noqa: F401
-from .weights.random_init import write_random_model  # noqa: F401
+from .config import describe_config, load_plugin, read_preset, registered_architectures  # noqa: F401
+from .engine.engine import Engine, EngineOptions, RequestOutput, SamplingParams  # noqa: F401
+from .engine.runner import Runner, StepEntry  # noqa: F401
+from .native import EngineError  # noqa: F401
+from .weights import check_model_dir, write_random_model  # noqa: F401

@@ -1,11 +1,14 @@
 """Builds the native libraries in-tree and loads them with ctypes.
 
-Two kinds of library live under ``mini_llm_amd/_lib``:
+These live under ``mini_llm_amd/_lib``:
 
 * ``runtime``: the host-only C++ runtime (cache manager, scheduler), built with g++;
-* one library per kernel source under ``csrc/kernels`` built with hipcc for gfx950.
-  A kernel library is built the first time one of its ops is called, so a model only
-  compiles what it needs.
+* one library per kernel source under ``csrc/kernels`` built with hipcc for gfx950;
+* ``engine``: the engine itself (host code that calls the kernel libraries), and the
+  program ``mini-llm``, its command line.
+
+A plugin (a shared library that registers further parts and architectures with the engine,
+``kind: "plugin"``) is described by its owner with ``register_library`` and built the same way.
 
 A library is rebuilt when the hash of its sources differs from the one recorded
 beside it, so a stale binary is never loaded.
@@ -68,7 +71,7 @@ LIBRARIES: Dict[str, dict] = {
     "engine": {
         "kind": "hiphost",
         "sources": ["engine/ops.cc", "engine/parts.cc", "engine/json.cc", "engine/weights.cc", "engine/arch.cc",
-                    "engine/engine.cc", "engine/engine_api.cc"],
+                    "engine/gpt2.cc", "engine/engine.cc", "engine/engine_api.cc"],
         "headers": ["engine/ops.h", "engine/parts.h", "engine/kernels.h", "engine/json.h", "engine/weights.h",
                     "engine/arch.h", "engine/engine.h", "runtime/cache_manager.h", "runtime/scheduler.h"],
         "needs": ["elementwise", "gemm_f32", "gemm_bf16", "attention", "attention_decode", "attention_prefill",
@@ -84,6 +87,15 @@ LIBRARIES: Dict[str, dict] = {
         "needs": ["engine", "runtime"],
     },
 }
+
+
+
+def register_library(name: str, spec: dict) -> None:
+    """Adds a library to build: ``spec`` as in LIBRARIES, with absolute paths for ``sources`` and ``headers``
+    and ``out_dir`` for the folder the built file goes to. ``kind: "plugin"`` is one hipcc source (host code
+    that registers parts and architectures, and their kernels) linked against the engine library."""
+    LIBRARIES[name] = spec
+
 
 _loaded: Dict[str, ctypes.CDLL] = {}
 _lock = threading.Lock()
@@ -107,18 +119,21 @@ def _paths(name: str):
 def _source_hash(name: str) -> str:
     spec, srcs, hdrs = _paths(name)
     h = hashlib.sha256()
-    flags = {"hip": HIPCC_FLAGS, "cxx": CXX_FLAGS, "hiphost": HIPHOST_FLAGS}[spec["kind"]]
+    flags = {"hip": HIPCC_FLAGS, "cxx": CXX_FLAGS, "hiphost": HIPHOST_FLAGS, "plugin": HIPCC_FLAGS}[spec["kind"]]
     h.update(" ".join(flags).encode())
+    if spec["kind"] == "plugin":
+        # a plugin sees the engine's classes: it is stale when their headers change
+        hdrs = hdrs + [os.path.join(CSRC, x) for x in LIBRARIES["engine"]["headers"]]
     for p in srcs + hdrs:
         with open(p, "rb") as f:
-            h.update(p[len(CSRC):].encode())
+            h.update(os.path.relpath(p, CSRC).encode())
             h.update(f.read())
     return h.hexdigest()
 
 
 def lib_path(name: str) -> str:
     program = LIBRARIES[name].get("program")
-    return os.path.join(LIB_DIR, program if program else f"libmllm_{name}.so")
+    return os.path.join(LIBRARIES[name].get("out_dir", LIB_DIR), program if program else f"libmllm_{name}.so")
 
 
 def is_current(name: str) -> bool:
@@ -153,12 +168,20 @@ def _find(tool: str, extra: List[str]) -> str:
 def build_library(name: str, verbose: bool = True) -> str:
     """Compiles one library unconditionally and returns its path."""
     spec, srcs, _ = _paths(name)
+    out_dir = spec.get("out_dir", LIB_DIR)
     os.makedirs(LIB_DIR, exist_ok=True)
+    os.makedirs(out_dir, exist_ok=True)
     so = lib_path(name)
     link: List[str] = []
     if spec["kind"] == "hip":
         cc = _find("hipcc", ["/opt/rocm/bin"])
         cmd = [cc] + HIPCC_FLAGS
+    elif spec["kind"] == "plugin":
+        if not is_current("engine"):
+            build_library("engine", verbose)
+        cc = _find("hipcc", ["/opt/rocm/bin"])
+        cmd = [cc] + HIPCC_FLAGS
+        link = [f"-L{LIB_DIR}", "-lmllm_engine", f"-Wl,-rpath,{LIB_DIR}"]
     elif spec["kind"] == "hiphost":
         # link against the libraries beside it; stale ones are compiled first, those without needs of
         # their own side by side
@@ -174,12 +197,12 @@ def build_library(name: str, verbose: bool = True) -> str:
         cc = _find("g++", ["/usr/bin"])
         cmd = [cc] + [f for f in HIPHOST_FLAGS if not (spec.get("program") and f in ("-shared",))]
         link = [f"-L{LIB_DIR}"] + [f"-lmllm_{d}" for d in needed_by(name)] + \
-               ["-L/opt/rocm/lib", "-lamdhip64", "-Wl,-rpath,$ORIGIN", "-Wl,-rpath,/opt/rocm/lib"]
+               ["-L/opt/rocm/lib", "-lamdhip64", "-ldl", "-Wl,-rpath,$ORIGIN", "-Wl,-rpath,/opt/rocm/lib"]
     else:
         cc = _find("g++", ["/usr/bin"])
         cmd = [cc] + CXX_FLAGS
     # Compile to a private name, then rename: a concurrent process never sees a half-written file.
-    fd, tmp = tempfile.mkstemp(prefix=f".{name}.", suffix=".tmp" if spec.get("program") else ".so", dir=LIB_DIR)
+    fd, tmp = tempfile.mkstemp(prefix=f".{name}.", suffix=".tmp" if spec.get("program") else ".so", dir=out_dir)
     os.close(fd)
     cmd = cmd + [f"-I{os.path.join(CSRC, 'kernels')}", f"-I{os.path.join(CSRC, 'runtime')}",
                  f"-I{os.path.join(CSRC, 'engine')}"] + srcs + ["-o", tmp] + link

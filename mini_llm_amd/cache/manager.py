@@ -1,9 +1,10 @@
-"""Python face of the native cache manager, and the device storage behind its pages.
+"""Python face of the native cache manager (tests drive it from here).
 
 ``CacheManager`` (C++: csrc/runtime/cache_manager.cc) decides which pages and state
-slots a request holds; it never touches device memory. ``CacheStorage`` owns the
-device tensors: for every group of layers one pool of pages shared by the layers of
-the group, and for state caches one array of slots.
+slots a request holds; it never touches device memory. The device memory behind the
+pages belongs to the engine's ``CacheStorage`` (csrc/engine/engine.cc): for every group
+of layers one pool of pages shared by the layers of the group, and for state caches one
+array of slots.
 
 The reference's pool and block manager:
 /root/reference/include/runtime/pool.cuh:11-68,
@@ -16,7 +17,6 @@ from dataclasses import dataclass
 from typing import Dict, List, Optional, Sequence, Tuple
 
 import numpy as np
-import torch
 
 from ..build import load_library
 
@@ -207,126 +207,3 @@ class CacheManager:
         buf = ctypes.create_string_buffer(4096)
         self._lib.mllm_cache_check(self._h, buf, 4096)
         return buf.value.decode()
-
-
-# --------------------------------------------------------------------------------
-# What a mixer asks of the cache
-# --------------------------------------------------------------------------------
-
-@dataclass(frozen=True)
-class KVCacheSpec:
-    """Keys and values of every token (or of a window of them), in pages."""
-    n_kv_heads: int
-    head_dim: int
-    window: int = 0
-
-    def group_key(self):
-        return ("kv", self.n_kv_heads, self.head_dim, self.window)
-
-
-@dataclass(frozen=True)
-class StateCacheSpec:
-    """A state of fixed size per request, in a slot."""
-    shape: Tuple[int, ...]
-    dtype: torch.dtype = torch.float32
-
-    def group_key(self):
-        return ("state", tuple(self.shape), self.dtype)
-
-
-@dataclass
-class KVCacheView:
-    """What a mixer sees of its cache during a step."""
-    k_pages: torch.Tensor      # [n_pages * page_size, n_kv_heads * head_dim]
-    v_pages: torch.Tensor
-    group: int                 # index into the step's per-group tables
-    page_size: int
-    window: int
-
-
-@dataclass
-class StateCacheView:
-    slots: torch.Tensor        # [n_state_slots, *shape]
-
-
-class CacheStorage:
-    """Device memory for the caches of a model, grouped by need.
-
-    ``specs[c]`` is what cache ``c`` of the model's execution order asks for. Caches
-    with equal KV specs form a group and share page ids, so one block table serves
-    all of them: pool layout ``[caches in group][K|V][n_pages * page_size][kv_dim]``.
-    """
-
-    def __init__(self, specs: Sequence[object], page_size: int, n_pages: int, n_state_slots: int,
-                 dtype: torch.dtype, device, n_pages_by_group: Optional[Dict[int, int]] = None):
-        self.page_size = int(page_size)
-        self.dtype = dtype
-        self.device = torch.device(device)
-        self.n_state_slots = int(n_state_slots)
-        keys: List[object] = []
-        self.cache_group: List[int] = []      # cache index -> kv group index, or -1 for state
-        members: List[List[int]] = []
-        for c, spec in enumerate(specs):
-            if isinstance(spec, KVCacheSpec):
-                k = spec.group_key()
-                if k not in keys:
-                    keys.append(k)
-                    members.append([])
-                g = keys.index(k)
-                members[g].append(c)
-                self.cache_group.append(g)
-            elif isinstance(spec, StateCacheSpec) or spec is None:
-                self.cache_group.append(-1)
-            else:
-                raise TypeError(f"cache {c}: unknown cache spec {spec!r}")
-        self.group_specs: List[GroupSpec] = []
-        self._pools: List[torch.Tensor] = []
-        self._views: List[Optional[object]] = [None] * len(specs)
-        for g, k in enumerate(keys):
-            _, hkv, hd, window = k
-            npg = (n_pages_by_group or {}).get(g, n_pages)
-            self.group_specs.append(GroupSpec(self.page_size, npg, window))
-            pool = torch.zeros((len(members[g]), 2, npg * self.page_size, hkv * hd),
-                               dtype=dtype, device=self.device)
-            self._pools.append(pool)
-            for j, c in enumerate(members[g]):
-                self._views[c] = KVCacheView(pool[j, 0], pool[j, 1], g, self.page_size, window)
-        self._state_views: List[StateCacheView] = []
-        for c, spec in enumerate(specs):
-            if isinstance(spec, StateCacheSpec):
-                slots = torch.zeros((self.n_state_slots,) + tuple(spec.shape), dtype=spec.dtype,
-                                    device=self.device)
-                self._views[c] = StateCacheView(slots)
-                self._state_views.append(self._views[c])
-        self.manager = CacheManager(self.group_specs, self.n_state_slots)
-
-    @property
-    def n_groups(self) -> int:
-        return len(self.group_specs)
-
-    def view(self, cache: int):
-        return self._views[cache]
-
-    def reset_fresh_states(self, ctx) -> None:
-        """Clears, on the device, the state slot of every request of the step that has no token
-        cached yet (``ctx.starts == 0``; a request that begins, or begins again after it was
-        preempted). Nothing to do for a model without state caches."""
-        if not self._state_views:
-            return
-        from ..kernels import ops
-        for view in self._state_views:
-            ops.reset_state(view.slots, ctx.state_slots, ctx.starts)
-
-    def bytes_per_token(self) -> int:
-        return sum(p.shape[0] * 2 * p.shape[3] * p.element_size() for p in self._pools)
-
-    def state_bytes_per_request(self) -> int:
-        return sum(v.slots[0].numel() * v.slots.element_size() for v in self._state_views)
-
-    def poison(self, value: float = float("nan")) -> None:
-        """Fills every page and every state slot with a value (tests: a stale or unwritten page, or
-        a state that was not cleared when its request began, must never be read)."""
-        for p in self._pools:
-            p.fill_(value)
-        for v in self._state_views:
-            v.slots.fill_(value)

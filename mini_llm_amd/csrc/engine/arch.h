@@ -21,14 +21,6 @@ public:
     explicit ConfigError(const std::string& what) : std::runtime_error(what) {}
 };
 
-// What a cache of the execution order asks of the cache manager.
-struct CacheNeed {
-    int kind = 1;                        // 1 keys and values in pages, 2 fixed-size state, 0 none
-    int n_kv_heads = 0, head_dim = 0, window = 0;
-    size_t state_bytes = 0;
-    int n_heads = 0;                     // query heads of the mixer that uses it (sizes the attention scratch)
-};
-
 // A model with its weights on the device.
 struct LoadedModel {
     std::string architecture;
@@ -36,7 +28,7 @@ struct LoadedModel {
     int dtype = BF16;
     DecoderModel model;
     DeviceTensors store;
-    std::vector<CacheNeed> caches;       // per cache index of the execution order
+    std::vector<CacheNeed> caches;       // per cache index of the execution order (from the model's mixers)
     int max_positions = 0;               // 0: unbounded
     int eos_token_id = -1;               // -1: none
 };
@@ -51,7 +43,14 @@ struct Architecture {
     std::function<bool(const std::string&)> ignored_tensor;
 };
 
+// Adding an architecture is one call of this (from anywhere: this library's own gpt2.cc, or a plugin's
+// static initialiser). `assemble` builds `out.model` from registered parts and sets `out.max_positions`
+// and `out.eos_token_id`; the caches' needs are read off the model afterwards.
 void register_architecture(const Architecture& a, const std::string& model_type = "");
+void register_gpt2();              // gpt2.cc
+// Loads a shared library whose initialisers register parts and architectures (dlopen; stays loaded).
+// Also called for every path in the environment variable MINI_LLM_PLUGINS (colon-separated), once.
+void load_plugin(const std::string& path);
 // by config.json: architectures[0], else model_type; unknown -> ConfigError listing the registered names
 const Architecture& architecture_of(const Json& config);
 std::vector<std::string> registered_architectures();
@@ -67,6 +66,9 @@ struct ModelFolderSummary {
     int64_t n_parameters = 0;
 };
 ModelFolderSummary check_model_dir(const std::string& model_dir);
+// The configuration's refusals, then the tensors a model of it expects, as JSON text:
+// {"architecture": ..., "tensors": [{"name", "shape", "role": "matrix"|"vector", "transpose", "mean", "std"}]}
+std::string describe_config(const Json& config);
 std::unique_ptr<LoadedModel> random_model(const Json& config, uint64_t seed, int dtype,
                                           const std::string& weights_dtype = "bfloat16");
 // a preset by name: config/presets/<name>.json beside the package

@@ -96,18 +96,63 @@ void CacheStorage::poison() {
 // ---------------------------------------------------------------------------------------------
 // runner
 // ---------------------------------------------------------------------------------------------
+// Pages that `fraction` of the free device memory holds, for caches with these needs.
+static int pages_for_memory_fraction(const std::vector<CacheNeed>& needs, int dtype, int page_size, double fraction) {
+    if (fraction > 1.0) throw EngineError("kv_memory_fraction must be at most 1");
+    size_t per_token = 0;
+    for (const CacheNeed& n : needs)
+        if (n.kind == 1) per_token += 2 * static_cast<size_t>(n.n_kv_heads) * n.head_dim * dtype_size(dtype);
+    if (per_token == 0) return 1;
+    size_t free_bytes = 0, total_bytes = 0;
+    HIP_OK(hipMemGetInfo(&free_bytes, &total_bytes));
+    // what later, small allocations may still want (buffers that grow, the runtime's own): kept out of the pool
+    const size_t margin = std::min<size_t>(free_bytes / 50, size_t(1) << 30);
+    const double pages = fraction * static_cast<double>(free_bytes - margin) / (static_cast<double>(per_token) * page_size);
+    const double most = 2147483647.0 / page_size;          // rows of a pool are indexed with 32 bits
+    if (pages < 1.0) throw EngineError("kv_memory_fraction leaves no room for a single page");
+    return static_cast<int>(std::min(pages, most));
+}
+
+ModelRunner::ModelRunner(LoadedModel& model, const RunnerOptions& o)
+    : model_(model), page_size_(o.page_size), n_pages_(o.n_pages), max_num_seqs_(std::max(o.max_num_seqs, 1)) {
+    init(o);
+}
+
 ModelRunner::ModelRunner(LoadedModel& model, int page_size, int n_pages, int max_num_seqs)
-    : model_(model), page_size_(page_size), n_pages_(n_pages), max_num_seqs_(max_num_seqs) {
-    cache_.reset(new CacheStorage(model.caches, page_size, n_pages, std::max(max_num_seqs, 1), model.dtype));
+    : model_(model), page_size_(page_size), n_pages_(n_pages), max_num_seqs_(std::max(max_num_seqs, 1)) {
+    RunnerOptions o;
+    o.page_size = page_size; o.n_pages = n_pages; o.max_num_seqs = max_num_seqs;
+    init(o);
+}
+
+void ModelRunner::init(const RunnerOptions& o) {
     HIP_OK(hipStreamCreate(&stream_));
     for (auto& st : staging_) HIP_OK(hipEventCreateWithFlags(&st.copied, hipEventDisableTiming));
     for (auto& e : host_tok_event_) HIP_OK(hipEventCreateWithFlags(&e, hipEventDisableTiming));
-    int n_heads = 0, head_dim = 0;
-    for (const CacheNeed& c : model.caches) { n_heads = std::max(n_heads, c.n_heads); head_dim = std::max(head_dim, c.head_dim); }
-    reserve_scratch((std::max(max_num_seqs, 1) + 7) / 8 * 8, model.model.vocab_size(), n_heads, head_dim);
-    host_tok_cap_ = std::max(max_num_seqs, 64) * 2;
+    // every part takes the scratch its kernels need, and the sampler its own, for the largest batch
+    const int rows = (max_num_seqs_ + 7) / 8 * 8;
+    model_.model.reserve(rows, stream_);
+    reserve_sampling_scratch(rows, model_.model.vocab_size(), stream_);
+    host_tok_cap_ = std::max(max_num_seqs_, 64) * 2;
     for (int i = 0; i < 2; ++i)
         HIP_OK(hipHostMalloc(reinterpret_cast<void**>(&host_tok_[i]), host_tok_cap_ * sizeof(int), hipHostMallocDefault));
+    if (o.max_tokens_per_step > 0) {
+        // the largest step's workspace, logits and index arrays now: nothing of that size is allocated in
+        // the middle of serving, and a pool sized from the free memory leaves room for them
+        const int T = std::max(o.max_tokens_per_step, max_num_seqs_);
+        arena_for(T, max_num_seqs_);
+        void* p = logits_;
+        grow(&p, &logits_bytes_, static_cast<size_t>(max_num_seqs_) * model_.model.vocab_size() * sizeof(float));
+        logits_ = static_cast<float*>(p);
+        p = dev_ints_;
+        size_t have = 0;
+        const size_t max_blocks = model_.max_positions > 0 ? (model_.max_positions + page_size_ - 1) / page_size_ : 256;
+        grow(&p, &have, (static_cast<size_t>(T) * (5 + 2 * model_.caches.size()) + static_cast<size_t>(max_num_seqs_) * (8 + max_blocks * model_.caches.size())) * sizeof(int));
+        dev_ints_ = static_cast<int*>(p);
+        dev_ints_cap_ = have / sizeof(int);
+    }
+    if (o.memory_fraction > 0.0) n_pages_ = pages_for_memory_fraction(model_.caches, model_.dtype, page_size_, o.memory_fraction);
+    cache_.reset(new CacheStorage(model_.caches, page_size_, n_pages_, max_num_seqs_, model_.dtype));
 }
 
 ModelRunner::~ModelRunner() {
@@ -122,7 +167,10 @@ ModelRunner::~ModelRunner() {
     }
     for (void* p : {static_cast<void*>(dev_ints_), arena_, static_cast<void*>(logits_), static_cast<void*>(tok_out_)})
         if (p) (void)hipFree(p);
-    if (stream_) (void)hipStreamDestroy(stream_);
+    if (stream_) {
+        release_scratch(stream_);
+        (void)hipStreamDestroy(stream_);
+    }
 }
 
 void ModelRunner::synchronize() { HIP_OK(hipStreamSynchronize(stream_)); }
@@ -360,25 +408,18 @@ std::vector<int> ModelRunner::collect() {
 // ---------------------------------------------------------------------------------------------
 // engine
 // ---------------------------------------------------------------------------------------------
-// Pages that `fraction` of the free device memory holds, for caches with these needs.
-static int pages_for_memory_fraction(const std::vector<CacheNeed>& needs, int dtype, int page_size, double fraction) {
-    if (fraction > 1.0) throw EngineError("kv_memory_fraction must be at most 1");
-    size_t per_token = 0;
-    for (const CacheNeed& n : needs)
-        if (n.kind == 1) per_token += 2 * static_cast<size_t>(n.n_kv_heads) * n.head_dim * dtype_size(dtype);
-    if (per_token == 0) return 1;
-    size_t free_bytes = 0, total_bytes = 0;
-    HIP_OK(hipMemGetInfo(&free_bytes, &total_bytes));
-    const double pages = fraction * static_cast<double>(free_bytes) / (static_cast<double>(per_token) * page_size);
-    const double most = 2147483647.0 / page_size;          // rows of a pool are indexed with 32 bits
-    if (pages < 1.0) throw EngineError("kv_memory_fraction leaves no room for a single page");
-    return static_cast<int>(std::min(pages, most));
-}
-
 Engine::Engine(std::unique_ptr<LoadedModel> model, const EngineOptions& o) : model_(std::move(model)), options_(o) {
-    if (o.kv_memory_fraction > 0.0)
-        options_.total_kv_blocks = pages_for_memory_fraction(model_->caches, model_->dtype, o.kv_block_size, o.kv_memory_fraction);
-    runner_.reset(new ModelRunner(*model_, o.kv_block_size, options_.total_kv_blocks, o.max_batch_num));
+    if (o.kv_block_size < 1 || o.max_batch_num < 1 || o.max_tokens_per_step < 1 || o.prefill_chunk < 1)
+        throw EngineError("kv_block_size, max_batch_num, max_tokens_per_step and prefill_chunk must be positive");
+    if (o.kv_memory_fraction < 0.0 || o.kv_memory_fraction > 1.0) throw EngineError("kv_memory_fraction must lie in [0, 1]");
+    RunnerOptions ro;
+    ro.page_size = o.kv_block_size;
+    ro.n_pages = o.total_kv_blocks;
+    ro.memory_fraction = o.kv_memory_fraction;
+    ro.max_num_seqs = o.max_batch_num;
+    ro.max_tokens_per_step = o.max_tokens_per_step;
+    runner_.reset(new ModelRunner(*model_, ro));
+    options_.total_kv_blocks = runner_->n_pages();
     SchedulerOptions so;
     so.max_num_seqs = o.max_batch_num;
     so.max_tokens_per_step = o.max_tokens_per_step;
@@ -435,7 +476,7 @@ std::vector<int> Engine::abort(int64_t request_id) {
     return std::vector<int>(r->tokens.begin() + r->prompt_len, r->tokens.end());
 }
 
-bool Engine::has_unfinished() const { return scheduler_->has_work() || in_flight_; }
+bool Engine::has_unfinished() const { return scheduler_->has_work() || in_flight_ || !undelivered_.empty(); }
 
 bool Engine::is_eos(const Request& r, int tok) const {
     return !r.params.ignore_eos && model_->eos_token_id >= 0 && tok == model_->eos_token_id;
@@ -547,6 +588,17 @@ std::vector<RequestOutput> Engine::step() {
     }
     if (!options_.overlap) append(collect());
     return outputs;
+}
+
+std::vector<RequestOutput> Engine::step_some(size_t cap) {
+    if (undelivered_.empty())
+        for (RequestOutput& o : step()) undelivered_.push_back(std::move(o));
+    std::vector<RequestOutput> out;
+    while (!undelivered_.empty() && out.size() < cap) {
+        out.push_back(std::move(undelivered_.front()));
+        undelivered_.pop_front();
+    }
+    return out;
 }
 
 std::vector<std::vector<int>> Engine::generate(const std::vector<std::vector<int>>& prompts,

@@ -36,7 +36,8 @@ struct EngineOptions {
     int kv_block_size = 16;            // tokens per page (reference: DEFAULT_KV_BLOCK_SIZE, constants.h:16)
     int total_kv_blocks = 4096;        // pages in the pool (reference: DEFAULT_TOTAL_KV_BLOCKS, constants.h:17)
     double kv_memory_fraction = 0.0;   // > 0: the pool takes this share of the device memory that is free once the
-                                       // weights are loaded, whatever total_kv_blocks says
+                                       // weights are loaded and the runner's buffers for the largest step are
+                                       // taken, whatever total_kv_blocks says
     int max_batch_num = 16;            // sequences in one step (reference: MAX_BATCH_NUM, constants.h:20)
     int max_tokens_per_step = 2048;    // token budget of one step
     int prefill_chunk = 512;           // longest prompt portion
@@ -93,9 +94,19 @@ struct StepEntry {
     int feed_row = -1;                 // >= 0: the single token is row feed_row of what the previous launch sampled
 };
 
-// Owns the cache storage and runs steps of a model.
+struct RunnerOptions {
+    int page_size = 16;
+    int n_pages = 0;                   // pages of every group's pool ...
+    double memory_fraction = 0.0;      // ... or, if > 0, this share of the device memory that is free once the
+                                       // runner's own buffers (workspace, logits, index arrays, scratch) exist
+    int max_num_seqs = 16;             // most sequences in a step: scratch, state slots and token buffers are sized for it
+    int max_tokens_per_step = 0;       // > 0: the step's workspace is taken now for this many tokens, not at the first large step
+};
+
+// Owns the cache storage and runs steps of a model, on a stream of its own.
 class ModelRunner {
 public:
+    ModelRunner(LoadedModel& model, const RunnerOptions& options);
     ModelRunner(LoadedModel& model, int page_size, int n_pages, int max_num_seqs);
     ~ModelRunner();
     CacheStorage& cache() { return *cache_; }
@@ -117,8 +128,11 @@ public:
     std::vector<int> collect();
     bool pending() const { return !pending_.empty(); }
     void synchronize();
+    hipStream_t stream() const { return stream_; }
+    int n_pages() const { return n_pages_; }
 
 private:
+    void init(const RunnerOptions& o);
     struct Staging {
         int* host = nullptr;
         size_t capacity = 0;
@@ -171,6 +185,9 @@ public:
     std::vector<int> abort(int64_t request_id);
     bool has_unfinished() const;
     std::vector<RequestOutput> step();
+    // The same, at most `cap` outputs at a time: what does not fit waits for the next call (which then runs
+    // no iteration of its own), and has_unfinished() stays true meanwhile. For callers with fixed buffers.
+    std::vector<RequestOutput> step_some(size_t cap);
     // Generates for every prompt (continuous batching) and returns the new tokens of each.
     std::vector<std::vector<int>> generate(const std::vector<std::vector<int>>& prompts,
                                            const std::vector<SamplingParams>& params);
@@ -202,6 +219,7 @@ private:
     int64_t next_id_ = 0;
     bool in_flight_ = false;
     std::vector<std::pair<RequestPtr, bool>> in_flight_rows_;      // (request, finished by that token)
+    std::deque<RequestOutput> undelivered_;                        // outputs that a step_some call had no room for
 };
 
 }  // namespace minillm

@@ -1,15 +1,17 @@
-// C ABI of the native engine: the checked device operations, the parts and the model's step
-// function. Loaded from Python with ctypes (kernels/ops.py, models/native.py); a C++ program links
-// the classes directly.
+// C ABI of the engine: the checked device operations, single parts, configurations and model folders,
+// the runner (step function) and the engine loop. Loaded from Python with ctypes (mini_llm_amd/native.py,
+// kernels/ops.py); a C++ program links the classes directly.
 //
 // Every function returns 0 on success and a non-zero code on failure; `mllm_last_error()` then
 // returns the message (per thread). Handles are opaque pointers; a handle passed to a function that
 // "takes" it is owned by the receiver from then on.
+#include <algorithm>
 #include <cstring>
 #include <memory>
 #include <string>
 #include <vector>
 
+#include "arch.h"
 #include "engine.h"
 #include "ops.h"
 #include "parts.h"
@@ -35,16 +37,28 @@ extern "C" {
 
 const char* mllm_last_error(void) { return g_error.c_str(); }
 
-// -- scratch and tuning ------------------------------------------------------------------------------
-int mllm_reserve_scratch(int rows, int vocab, int n_heads, int head_dim) {
-    return guarded([&] { reserve_scratch(rows, vocab, n_heads, head_dim); });
+// Copies `text` into out[cap] (truncated, always terminated) and returns its full length.
+static int put_text(const std::string& text, char* out, int cap) {
+    if (out != nullptr && cap > 0) {
+        const size_t n = std::min(text.size(), static_cast<size_t>(cap - 1));
+        std::memcpy(out, text.data(), n);
+        out[n] = 0;
+    }
+    return static_cast<int>(text.size());
 }
-unsigned long long mllm_scratch_generation(void) { return scratch_generation(); }
-void* mllm_scratch_address(const char* name) {
+
+// -- scratch and tuning ------------------------------------------------------------------------------
+void* mllm_scratch_address(const char* name, hipStream_t stream) {
     void* p = nullptr;
-    guarded([&] { p = scratch_address(name); });
+    guarded([&] { p = scratch_address(name, stream); });
     return p;
 }
+unsigned long long mllm_scratch_bytes(void) {
+    size_t n = 0;
+    guarded([&] { n = scratch_bytes(); });
+    return n;
+}
+int mllm_release_scratch(hipStream_t stream) { return guarded([&] { release_scratch(stream); }); }
 // name: "decode_shape" (nsplit, waves; 0, 0 = automatic), "unmerged_shape", "merge_max_rows" (a), "ln_fuse_max_rows" (a), "long_context_splits" (a: 0 off, 1 on)
 int mllm_set_tuning(const char* name, int a, int b) {
     return guarded([&] {
@@ -55,8 +69,20 @@ int mllm_set_tuning(const char* name, int a, int b) {
         else if (n == "merge_max_rows") t.merge_max_rows = a;
         else if (n == "ln_fuse_max_rows") t.ln_fuse_max_rows = a;
         else if (n == "long_context_splits") t.long_context_splits = a;
+        else if (n == "reset_seen") t.seen = Tuning::Seen();
         else fail("unknown tuning value '%s'", name);
     });
+}
+// What the ops chose since the last "reset_seen": "max_decode_splits" (most workgroups a (token, head) pair's keys
+// were split over), "merge_kernel_launches", "prefill_tile_launches", "generic_attention_launches". -1: unknown name.
+long long mllm_get_seen(const char* name) {
+    const Tuning::Seen& s = tuning().seen;
+    const std::string n(name);
+    if (n == "max_decode_splits") return s.max_decode_splits;
+    if (n == "merge_kernel_launches") return s.merge_kernel_launches;
+    if (n == "prefill_tile_launches") return s.prefill_tile_launches;
+    if (n == "generic_attention_launches") return s.generic_attention_launches;
+    return -1;
 }
 
 // -- the ops (see ops.h) -----------------------------------------------------------------------------
@@ -111,72 +137,213 @@ void mllm_params_set_number(void* p, const char* key, double v) { static_cast<Pa
 void mllm_params_set_string(void* p, const char* key, const char* v) { static_cast<Params*>(p)->str[key] = v; }
 void mllm_params_set_tensor(void* p, const char* key, const Tensor2* t) { static_cast<Params*>(p)->tensor[key] = *t; }
 
-// -- parts -------------------------------------------------------------------------------------------
+// -- single parts, for tests of a part alone -----------------------------------------------------------
+// (A mixer needs a step's index arrays and a cache: it is tested through a model, not here.)
 int mllm_has_part(const char* category, const char* kind) { return has_part(category, kind) ? 1 : 0; }
-
 void* mllm_norm_create(const char* kind, const void* params) {
     Norm* n = nullptr;
     guarded([&] { n = build_norm(kind, *static_cast<const Params*>(params)).release(); });
     return n;
 }
-void* mllm_mixer_create(const char* kind, const void* params) {
-    Mixer* m = nullptr;
-    guarded([&] { m = build_mixer(kind, *static_cast<const Params*>(params)).release(); });
-    return m;
+void mllm_norm_destroy(void* n) { delete static_cast<Norm*>(n); }
+// out[i,:] = norm(x[rows ? rows[i] : i, :]); `arena` is device memory for temporaries
+int mllm_norm_forward(const void* norm, const Tensor2* x, const int* rows, const Tensor2* out, void* arena, size_t arena_bytes,
+                      hipStream_t s) {
+    return guarded([&] {
+        Arena a(arena, arena_bytes);
+        const Tensor2 h = static_cast<const Norm*>(norm)->forward(*x, rows, static_cast<int>(out->rows), a, s);
+        if (h.dtype != out->dtype || h.cols != out->cols) fail("the norm's output is %s [%lld], the buffer %s [%lld]", dtype_name(h.dtype), (long long)h.cols, dtype_name(out->dtype), (long long)out->cols);
+        if (hipMemcpy2DAsync(out->data, out->stride * out->esz(), h.data, h.stride * h.esz(), h.cols * h.esz(), h.rows, hipMemcpyDeviceToDevice, s) != hipSuccess)
+            fail("copy of the norm's output failed");
+    });
 }
 void* mllm_feed_forward_create(const char* kind, const void* params) {
     FeedForward* f = nullptr;
     guarded([&] { f = build_feed_forward(kind, *static_cast<const Params*>(params)).release(); });
     return f;
 }
-// Takes the mixer, the feed-forward and the norms.
-void* mllm_block_create(const char* kind, void* mixer, void* feed_forward, void** norms, int n_norms) {
-    Block* b = nullptr;
-    std::unique_ptr<Mixer> m(static_cast<Mixer*>(mixer));
-    std::unique_ptr<FeedForward> f(static_cast<FeedForward*>(feed_forward));
-    std::vector<std::unique_ptr<Norm>> ns;
-    for (int i = 0; i < n_norms; ++i) ns.emplace_back(static_cast<Norm*>(norms[i]));
-    guarded([&] { b = build_block(kind, std::move(m), std::move(f), std::move(ns)).release(); });
-    return b;
-}
-void mllm_norm_destroy(void* n) { delete static_cast<Norm*>(n); }
-void mllm_block_destroy(void* b) { delete static_cast<Block*>(b); }
-
-// -- the model ---------------------------------------------------------------------------------------
-void* mllm_model_create(const Tensor2* wte, const Tensor2* wpe, int dtype) {
-    auto* m = new DecoderModel();
-    m->wte = *wte;
-    if (wpe != nullptr) m->wpe = *wpe;
-    m->dtype = dtype;
-    return m;
-}
-void mllm_model_destroy(void* m) { delete static_cast<DecoderModel*>(m); }
-// Takes the block. Returns the layer's index.
-int mllm_model_add_layer(void* m, void* block) {
-    auto* model = static_cast<DecoderModel*>(m);
-    model->layers.emplace_back(static_cast<Block*>(block));
-    return static_cast<int>(model->layers.size()) - 1;
-}
-void mllm_model_set_order(void* m, const int* layer, const int* cache, const int* write, int n) {
-    auto* model = static_cast<DecoderModel*>(m);
-    model->order.clear();
-    for (int i = 0; i < n; ++i) model->order.push_back({layer[i], cache[i], write[i] != 0});
-}
-// Takes the norm.
-void mllm_model_set_final_norm(void* m, void* norm) { static_cast<DecoderModel*>(m)->final_norm.reset(static_cast<Norm*>(norm)); }
-size_t mllm_model_workspace_bytes(const void* m, int tokens, int n_logits) {
-    return static_cast<const DecoderModel*>(m)->workspace_bytes(tokens, n_logits);
-}
-// One step: the tokens of `step` through every call of the execution order, fp32 logits of the wanted
-// rows into `logits`. `arena` is device memory of at least mllm_model_workspace_bytes bytes.
-int mllm_model_forward(const void* m, const StepView* step, const CacheView* caches, int n_caches, void* arena,
-                       size_t arena_bytes, const Tensor2* logits, hipStream_t s) {
+void mllm_feed_forward_destroy(void* f) { delete static_cast<FeedForward*>(f); }
+// x += feed_forward(h), h already normalised [T, hidden] in the compute dtype
+int mllm_feed_forward_forward(const void* ff, const Tensor2* h, const Tensor2* x, void* arena, size_t arena_bytes, hipStream_t s) {
     return guarded([&] {
         Arena a(arena, arena_bytes);
-        std::vector<CacheView> cv(caches, caches + n_caches);
-        static_cast<const DecoderModel*>(m)->forward(*step, cv, a, logits ? *logits : Tensor2(), s);
+        StepView step;
+        step.n_tokens = static_cast<int>(h->rows);
+        NormedInput in(*h);
+        static_cast<const FeedForward*>(ff)->forward(in, step, *x, a, s);
     });
 }
+void* mllm_embedding_create(const char* kind, const void* params) {
+    Embedding* e = nullptr;
+    guarded([&] { e = build_embedding(kind, *static_cast<const Params*>(params)).release(); });
+    return e;
+}
+void mllm_embedding_destroy(void* e) { delete static_cast<Embedding*>(e); }
+// x[t,:] = embedding(ids[t]) (+ row positions[t] of a position encoding of kind position_kind, built from position_params)
+int mllm_embedding_forward(const void* emb, const char* position_kind, const void* position_params, const int* ids,
+                           const int* positions, const Tensor2* x, hipStream_t s) {
+    return guarded([&] {
+        std::shared_ptr<const PositionEncoding> pos;
+        if (position_kind != nullptr && position_kind[0] != 0) pos = build_position(position_kind, *static_cast<const Params*>(position_params));
+        StepView step;
+        step.n_tokens = static_cast<int>(x->rows);
+        step.token_ids = ids;
+        step.positions = positions;
+        static_cast<const Embedding*>(emb)->forward(step, pos.get(), *x, s);
+    });
+}
+void* mllm_head_create(const char* kind, const void* params) {
+    Head* h = nullptr;
+    guarded([&] { h = build_head(kind, *static_cast<const Params*>(params)).release(); });
+    return h;
+}
+void mllm_head_destroy(void* h) { delete static_cast<Head*>(h); }
+// logits[i,:] = head(norm(x[rows ? rows[i] : i, :]))
+int mllm_head_forward(const void* head, const void* norm, const Tensor2* x, const int* rows, const Tensor2* logits, void* arena,
+                      size_t arena_bytes, hipStream_t s) {
+    return guarded([&] {
+        Arena a(arena, arena_bytes);
+        static_cast<const Head*>(head)->forward(*x, *static_cast<const Norm*>(norm), rows, *logits, a, s);
+    });
+}
+
+// -- configurations, architectures, model folders (no device is touched) -------------------------------
+int mllm_load_plugin(const char* path) { return guarded([&] { load_plugin(path); }); }
+// JSON array of names; returns the text's full length
+int mllm_registered_architectures(char* out, int cap) {
+    std::string text;
+    guarded([&] {
+        std::vector<Json> names;
+        for (const std::string& n : registered_architectures()) names.push_back(Json::of(n));
+        text = Json::array_of(names).dump();
+    });
+    return put_text(text, out, cap);
+}
+// The architecture and the tensors a model of this config.json expects, as JSON (arch.h: describe_config);
+// returns the text's full length, or -1 when the configuration is refused (mllm_last_error says why).
+int mllm_describe_config(const char* config_json, char* out, int cap) {
+    std::string text;
+    if (guarded([&] { text = describe_config(Json::parse(config_json)); }) != 0) return -1;
+    return put_text(text, out, cap);
+}
+// Checks a folder's config.json and tensor headers against its architecture; out: "architecture tensors parameters"
+int mllm_check_model_dir(const char* model_dir, char* out, int cap) {
+    return guarded([&] {
+        const ModelFolderSummary s = check_model_dir(model_dir);
+        put_text(s.architecture + " " + std::to_string(s.n_tensors) + " " + std::to_string(s.n_parameters), out, cap);
+    });
+}
+// Writes config.json and model.safetensors with random weights (weights_dtype: "bfloat16" or "float32")
+int mllm_write_random_model(const char* config_json, unsigned long long seed, const char* out_dir, const char* weights_dtype) {
+    return guarded([&] {
+        Json config = Json::parse(config_json);
+        const Architecture& arch = architecture_of(config);
+        if (!config.has("architectures")) config.set("architectures", Json::array_of({Json::of(arch.name)}));
+        write_random_model(out_dir, config, arch.param_specs(config), seed, weights_dtype);
+    });
+}
+// n values of the random generator for tensor `name` under `seed`, from element `first` on
+int mllm_normal_values(unsigned long long seed, const char* name, long long first, long long n, double mean, double std, float* out) {
+    return guarded([&] { normal_values(seed, name, first, n, mean, std, out); });
+}
+
+// -- a runner: a model, its caches and the step function (engine.h: ModelRunner) ------------------------
+namespace {
+struct RunnerBox {
+    std::unique_ptr<LoadedModel> model;
+    std::unique_ptr<ModelRunner> runner;
+};
+}  // namespace
+// Either model_dir, or config_json with a seed (random weights, rounded as a written folder holds them).
+void* mllm_runner_create(const char* model_dir, const char* config_json, unsigned long long seed, int dtype, int page_size,
+                         int n_pages, int max_num_seqs) {
+    RunnerBox* box = nullptr;
+    guarded([&] {
+        std::unique_ptr<RunnerBox> b(new RunnerBox());
+        if (model_dir != nullptr && model_dir[0] != 0) b->model = load_model(model_dir, dtype);
+        else b->model = random_model(Json::parse(config_json), seed, dtype);
+        b->runner.reset(new ModelRunner(*b->model, page_size, n_pages, max_num_seqs));
+        box = b.release();
+    });
+    return box;
+}
+void mllm_runner_destroy(void* box) { delete static_cast<RunnerBox*>(box); }
+void* mllm_runner_of_box(void* box) { return static_cast<RunnerBox*>(box)->runner.get(); }
+// One step of B entries: entry i is request ids[i] with its next n_tokens[i] tokens (flattened in `tokens`) and
+// n_want[i] wanted places among them (flattened in `want`). The fp32 logits [wanted, vocab] go to `logits`
+// (room for cap_rows rows). The runner registers new requests, takes pages and commits lengths itself.
+// Returns the number of rows, or -1.
+int mllm_runner_step(void* runner, const long long* ids, const int* n_tokens, const int* tokens, const int* n_want,
+                     const int* want, int B, float* logits, long long cap_rows) {
+    int rows = -1;
+    guarded([&] {
+        std::vector<StepEntry> entries(B);
+        size_t t = 0, w = 0;
+        long long total = 0;
+        for (int i = 0; i < B; ++i) {
+            entries[i].request_id = ids[i];
+            entries[i].tokens.assign(tokens + t, tokens + t + n_tokens[i]);
+            entries[i].want.assign(want + w, want + w + n_want[i]);
+            t += n_tokens[i];
+            w += n_want[i];
+            total += n_want[i];
+        }
+        if (total > cap_rows) fail("%lld rows of logits are wanted, the buffer holds %lld", total, cap_rows);
+        int n = 0;
+        const std::vector<float> host = static_cast<ModelRunner*>(runner)->step(entries, true, &n);
+        if (!host.empty()) std::memcpy(logits, host.data(), host.size() * sizeof(float));
+        rows = n;
+    });
+    return rows;
+}
+int mllm_runner_end_request(void* runner, long long id) {
+    return guarded([&] {
+        ModelRunner* r = static_cast<ModelRunner*>(runner);
+        if (!r->manager().has_request(id)) fail("request %lld is not live", id);
+        r->end_request(id);
+    });
+}
+int mllm_runner_poison(void* runner) { return guarded([&] { static_cast<ModelRunner*>(runner)->cache().poison(); }); }
+// The cache manager's consistency report (empty: no page or slot is lost, held twice or both held and free)
+int mllm_runner_check(void* runner, char* out, int cap) {
+    std::string text;
+    guarded([&] { text = static_cast<ModelRunner*>(runner)->manager().check(); });
+    return put_text(text, out, cap);
+}
+// Sizes and costs as JSON: architecture, vocab_size, hidden_size, max_positions, eos_token_id, dtype, n_layers,
+// n_calls, n_caches, n_groups, page_size, n_pages, free_pages, n_requests, cache_bytes_per_token, and the step's
+// cost (parts.h: StepCost): weight_bytes, flops_per_token, attention_flops_per_key, flops_per_logits_row
+int mllm_runner_info(void* runner, char* out, int cap) {
+    std::string text;
+    guarded([&] {
+        ModelRunner* r = static_cast<ModelRunner*>(runner);
+        const LoadedModel& m = r->model();
+        const StepCost c = m.model.cost();
+        Json j = Json::object();
+        j.set("architecture", Json::of(m.architecture));
+        j.set("vocab_size", Json::of(m.model.vocab_size()));
+        j.set("hidden_size", Json::of(m.model.hidden_size()));
+        j.set("max_positions", Json::of(m.max_positions));
+        j.set("eos_token_id", Json::of(m.eos_token_id));
+        j.set("dtype", Json::of(dtype_name(m.dtype)));
+        j.set("n_layers", Json::of(static_cast<int>(m.model.layers.size())));
+        j.set("n_calls", Json::of(static_cast<int>(m.model.order.size())));
+        j.set("n_caches", Json::of(static_cast<int>(m.caches.size())));
+        j.set("n_groups", Json::of(r->cache().n_groups()));
+        j.set("page_size", Json::of(r->cache().page_size()));
+        j.set("n_pages", Json::of(r->n_pages()));
+        j.set("free_pages", Json::of(r->manager().n_groups() ? r->manager().free_pages(0) : 0));
+        j.set("n_requests", Json::of(r->manager().n_requests()));
+        j.set("cache_bytes_per_token", Json::of(static_cast<int64_t>(r->cache().bytes_per_token())));
+        j.set("weight_bytes", Json::of(c.weight_bytes));
+        j.set("flops_per_token", Json::of(c.flops_per_token));
+        j.set("attention_flops_per_key", Json::of(c.attention_flops_per_key));
+        j.set("flops_per_logits_row", Json::of(c.flops_per_logits_row));
+        text = j.dump();
+    });
+    return put_text(text, out, cap);
+}
+void mllm_runner_synchronize(void* runner) { guarded([&] { static_cast<ModelRunner*>(runner)->synchronize(); }); }
 
 // -- the engine (engine.h) ---------------------------------------------------------------------------
 // options: kv_block_size, total_kv_blocks, max_batch_num, max_tokens_per_step, prefill_chunk, overlap (0/1),
@@ -192,13 +359,17 @@ void* mllm_engine_from_pretrained(const char* model_dir, int dtype, const int* o
     guarded([&] { e = Engine::from_pretrained(model_dir, dtype, options_of(options7)).release(); });
     return e;
 }
-// config_json: the text of a config.json
+// config_json: the text of a config.json. The weights are the values a written folder holds (matrices rounded
+// to bfloat16 whatever `dtype` computes in), so this and make-model + from_pretrained give the same model.
 void* mllm_engine_from_random(const char* config_json, unsigned long long seed, int dtype, const int* options7) {
     Engine* e = nullptr;
     guarded([&] { e = Engine::from_random(Json::parse(config_json), seed, dtype, options_of(options7)).release(); });
     return e;
 }
 void mllm_engine_destroy(void* e) { delete static_cast<Engine*>(e); }
+// The engine's runner, for the mllm_runner_* functions (borrowed: it lives as long as the engine). Requests
+// stepped through it directly must not share ids with requests added to the engine.
+void* mllm_engine_runner(void* e) { return &static_cast<Engine*>(e)->runner(); }
 // Returns the request's id, or -1 (see mllm_last_error).
 long long mllm_engine_add_request(void* e, const int* tokens, int n, float temperature, unsigned long long seed,
                                   int max_new_tokens, int ignore_eos, long long request_id) {
@@ -211,21 +382,26 @@ long long mllm_engine_add_request(void* e, const int* tokens, int n, float tempe
     return id;
 }
 int mllm_engine_has_unfinished(void* e) { return static_cast<Engine*>(e)->has_unfinished() ? 1 : 0; }
-// One iteration. Up to `cap` outputs are written (ids, tokens, finished flags; a token of -1 is a failed
-// request, whose reason mllm_last_error holds); returns their number, or -1 on an error.
+// One iteration. Up to `cap` outputs are written (ids, tokens, finished flags; a token of -1 is a failed request);
+// outputs beyond `cap` wait for the next call, and mllm_engine_has_unfinished stays 1 meanwhile. Returns their
+// number, or -1 on an error. The reason of the i-th output's failure: mllm_engine_output_error(e, i).
+namespace { thread_local std::vector<std::string> g_output_errors; }
 int mllm_engine_step(void* e, long long* ids, int* tokens, int* finished, int cap) {
     int n = -1;
     guarded([&] {
-        const std::vector<RequestOutput> outs = static_cast<Engine*>(e)->step();
-        if (static_cast<int>(outs.size()) > cap) fail("more outputs (%zu) than room (%d)", outs.size(), cap);
+        const std::vector<RequestOutput> outs = static_cast<Engine*>(e)->step_some(static_cast<size_t>(std::max(cap, 1)));
+        g_output_errors.assign(outs.size(), "");
         n = 0;
         for (const RequestOutput& o : outs) {
             ids[n] = o.request_id; tokens[n] = o.token; finished[n] = o.finished ? 1 : 0;
-            if (o.token < 0) g_error = o.error;
+            g_output_errors[n] = o.error;
             ++n;
         }
     });
     return n;
+}
+const char* mllm_engine_output_error(int i) {
+    return (i >= 0 && i < static_cast<int>(g_output_errors.size())) ? g_output_errors[i].c_str() : "";
 }
 int mllm_engine_abort(void* e, long long id) { return guarded([&] { static_cast<Engine*>(e)->abort(id); }); }
 // names: steps, scheduled_tokens, prefill_tokens, decode_tokens, deferred_decodes, deferred_prefills, preemptions,
@@ -236,9 +412,6 @@ void mllm_engine_stats(void* e, long long* out12) {
                              "preemptions", "failures", "finished", "peak_pages_used", "free_pages", "total_pages"};
     for (int i = 0; i < 12; ++i) out12[i] = st.at(names[i]);
 }
-int mllm_engine_vocab_size(void* e) { return static_cast<Engine*>(e)->model().model.vocab_size(); }
-// weights bytes read once per step, flops per token... are the Python model's business; here: the cache's bytes per token
-unsigned long long mllm_engine_cache_bytes_per_token(void* e) { return static_cast<Engine*>(e)->runner().cache().bytes_per_token(); }
 void mllm_engine_synchronize(void* e) { guarded([&] { static_cast<Engine*>(e)->runner().synchronize(); }); }
 
 }  // extern "C"

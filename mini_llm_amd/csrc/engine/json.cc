@@ -87,7 +87,16 @@ private:
         }
         return out;
     }
+    // Nesting deeper than any configuration or safetensors header goes is refused: the parser recurses once
+    // per level, and a text of a million '[' must end in an error, not in a stack overflow.
+    static constexpr int MAX_DEPTH = 64;
+    struct Level {
+        explicit Level(JsonParser& p) : p_(p) { if (++p_.depth_ > MAX_DEPTH) p_.bad("nested deeper than 64 levels"); }
+        ~Level() { --p_.depth_; }
+        JsonParser& p_;
+    };
     Json value() {
+        const Level level(*this);
         ws();
         if (i_ >= t_.size()) bad("unexpected end");
         const char c = t_[i_];
@@ -149,6 +158,7 @@ private:
     }
     const std::string& t_;
     size_t i_ = 0;
+    int depth_ = 0;
 };
 
 Json Json::parse(const std::string& text) { return JsonParser(text).run(); }

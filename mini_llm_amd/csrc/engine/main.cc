@@ -95,6 +95,13 @@ bool parse_request(const std::string& line, std::vector<int>& ids) {
     return !ids.empty();
 }
 
+// --plugin PATH (may be given several times): shared libraries that register parts and architectures
+void load_plugins(const Args& a) {
+    auto it = a.values.find("plugin");
+    if (it == a.values.end()) return;
+    for (const std::string& path : it->second) load_plugin(path);
+}
+
 int dtype_of(const std::string& name) {
     if (name == "bfloat16" || name == "bf16") return BF16;
     if (name == "float32" || name == "fp32") return F32;
@@ -116,9 +123,10 @@ std::string presets_dir(const char* argv0) {
 int cmd_generate(int argc, char** argv) {
     const Args a = parse_args(argc, argv, 2,
                               {"model", "preset", "weights-seed", "dtype", "device", "prompt-ids", "prompts-file", "max-new-tokens",
-                               "temperature", "seed", "kv-block-size", "total-kv-blocks", "max-batch-num", "max-tokens-per-step",
-                               "prefill-chunk"},
+                               "temperature", "seed", "kv-block-size", "total-kv-blocks", "kv-memory-fraction", "max-batch-num",
+                               "max-tokens-per-step", "prefill-chunk", "plugin"},
                               {"ignore-eos", "stream", "stats", "no-overlap"});
+    load_plugins(a);
     if (a.has("model") == a.has("preset")) { std::fprintf(stderr, "give either --model DIR or --preset NAME\n"); return 1; }
     const std::string device = a.get("device", "cuda:0");
     if (device.rfind("cuda", 0) != 0 && device != "gpu") {
@@ -139,7 +147,8 @@ int cmd_generate(int argc, char** argv) {
     EngineOptions o;
     o.kv_block_size = static_cast<int>(a.integer("kv-block-size", 16));
     o.total_kv_blocks = static_cast<int>(a.integer("total-kv-blocks", 4096));
-    o.kv_memory_fraction = a.has("kv-memory-fraction") ? std::atof(a.get("kv-memory-fraction").c_str()) : 0.0;
+    o.kv_memory_fraction = a.real("kv-memory-fraction", 0.0);
+    if (o.kv_memory_fraction < 0.0 || o.kv_memory_fraction > 1.0) throw EngineError("--kv-memory-fraction wants a number in (0, 1]");
     o.max_batch_num = static_cast<int>(a.integer("max-batch-num", 16));
     o.max_tokens_per_step = static_cast<int>(a.integer("max-tokens-per-step", 2048));
     o.prefill_chunk = static_cast<int>(a.integer("prefill-chunk", 512));
@@ -193,7 +202,8 @@ int cmd_generate(int argc, char** argv) {
 
 // check --model DIR: configuration and tensors against the architecture, without a GPU
 int cmd_check(int argc, char** argv) {
-    const Args a = parse_args(argc, argv, 2, {"model"}, {});
+    const Args a = parse_args(argc, argv, 2, {"model", "plugin"}, {});
+    load_plugins(a);
     if (!a.has("model")) {
         std::fprintf(stderr, "usage: mini-llm check --model DIR\n");
         return 1;
@@ -204,7 +214,8 @@ int cmd_check(int argc, char** argv) {
 }
 
 int cmd_make_model(int argc, char** argv) {
-    const Args a = parse_args(argc, argv, 2, {"preset", "config", "seed", "out", "weights-dtype"}, {});
+    const Args a = parse_args(argc, argv, 2, {"preset", "config", "seed", "out", "weights-dtype", "plugin"}, {});
+    load_plugins(a);
     if (a.has("preset") == a.has("config") || !a.has("seed") || !a.has("out")) {
         std::fprintf(stderr, "usage: mini-llm make-model (--preset NAME | --config FILE) --seed S --out DIR\n");
         return 1;
@@ -228,7 +239,8 @@ int cmd_make_model(int argc, char** argv) {
 }
 
 int cmd_replay(int argc, char** argv) {
-    const Args a = parse_args(argc, argv, 2, {"model", "dtype", "out", "max-tokens", "page-size", "max-requests", "device"}, {});
+    const Args a = parse_args(argc, argv, 2, {"model", "dtype", "out", "max-tokens", "page-size", "max-requests", "device", "plugin"}, {});
+    load_plugins(a);
     for (const char* k : {"model", "dtype", "out", "max-tokens"})
         if (!a.has(k)) { std::fprintf(stderr, "replay: --%s is required\n", k); return 1; }
     const int page = static_cast<int>(a.integer("page-size", 16));
@@ -301,6 +313,8 @@ int main(int argc, char** argv) {
                  "             [--prompts-file F] [--max-new-tokens 8] [--temperature 0] [--seed 0] [--ignore-eos] [--stream] [--stats]\n"
                  "             [--kv-block-size 16] [--total-kv-blocks 4096 | --kv-memory-fraction F] [--max-batch-num 16] [--max-tokens-per-step 2048]\n"
                  "             [--prefill-chunk 512]\n"
+                 "  every command: [--plugin LIB.so]...  shared libraries that register further parts and architectures\n"
+                 "             (also: the paths in the environment variable MINI_LLM_PLUGINS, separated by colons)\n"
                  "  make-model (--preset NAME | --config FILE) --seed S --out DIR [--weights-dtype bfloat16|float32]\n"
                  "  replay     --model DIR --dtype bfloat16|float32 --out DIR --max-tokens N [--page-size 16]\n"
                  "  check      --model DIR     (configuration and tensors against the architecture; needs no GPU)\n");

@@ -43,9 +43,18 @@ struct Buffer {
     void* ptr = nullptr;
     size_t bytes = 0;
 };
+struct Key {
+    int device;
+    hipStream_t stream;
+    std::string name;
+    bool operator<(const Key& o) const {
+        if (device != o.device) return device < o.device;
+        if (stream != o.stream) return std::less<const void*>()(stream, o.stream);
+        return name < o.name;
+    }
+};
 std::mutex g_scratch_mutex;
-std::map<std::pair<int, std::string>, Buffer> g_scratch;     // (device, name) -> buffer
-uint64_t g_generation = 0;
+std::map<Key, Buffer> g_scratch;
 constexpr size_t GEMM_WORKSPACE_BYTES = 16 * 1024 + 256 * 1024;   // counters, then 1 KB per workgroup of a shared-tile launch
 constexpr int DECODE_MAX_SPLIT = 8;
 
@@ -57,10 +66,9 @@ int current_device() {
 }
 
 // Grows only; a fresh buffer is cleared when `zero` (kernels that use counters leave them at zero).
-// Never called while a stream captures with a size beyond what is there: callers reserve first.
-void* scratch(const char* name, size_t bytes, bool zero) {
+void* scratch(const char* name, size_t bytes, bool zero, hipStream_t stream) {
     std::lock_guard<std::mutex> lock(g_scratch_mutex);
-    Buffer& b = g_scratch[{current_device(), name}];
+    Buffer& b = g_scratch[Key{current_device(), stream, name}];
     if (b.ptr != nullptr && b.bytes >= bytes) return b.ptr;
     void* fresh = nullptr;
     hipError_t e = hipMalloc(&fresh, bytes);
@@ -70,45 +78,65 @@ void* scratch(const char* name, size_t bytes, bool zero) {
         if (e != hipSuccess) fail("scratch '%s': hipMemset failed: %s", name, hipGetErrorString(e));
     }
     if (b.ptr != nullptr) {
-        // Work queued with the old buffer may still run: wait for it, then free. Graphs that hold the
-        // old address are the holders' business (scratch_generation()).
+        // work queued with the old buffer may still run: wait for it, then free
         (void)hipDeviceSynchronize();
         (void)hipFree(b.ptr);
-        ++g_generation;
     }
     b.ptr = fresh;
     b.bytes = bytes;
     return fresh;
 }
 
-float* argmax_values(size_t n) { return static_cast<float*>(scratch("argmax_values", std::max<size_t>(n, 4096) * 4, false)); }
-int* argmax_indices(size_t n) { return static_cast<int*>(scratch("argmax_indices", std::max<size_t>(n, 4096) * 4, false)); }
-float* decode_partials(size_t n) { return static_cast<float*>(scratch("decode_partials", std::max<size_t>(n, 1 << 16) * 4, false)); }
-int* decode_counters(size_t n) { return static_cast<int*>(scratch("decode_counters", std::max<size_t>(n, 4096) * 4, true)); }
-void* gemm_workspace() { return scratch("gemm_workspace", GEMM_WORKSPACE_BYTES, true); }
+float* argmax_values(size_t n, hipStream_t s) { return static_cast<float*>(scratch("argmax_values", std::max<size_t>(n, 4096) * 4, false, s)); }
+int* argmax_indices(size_t n, hipStream_t s) { return static_cast<int*>(scratch("argmax_indices", std::max<size_t>(n, 4096) * 4, false, s)); }
+float* decode_partials(size_t n, hipStream_t s) { return static_cast<float*>(scratch("decode_partials", std::max<size_t>(n, 1 << 16) * 4, false, s)); }
+int* decode_counters(size_t n, hipStream_t s) { return static_cast<int*>(scratch("decode_counters", std::max<size_t>(n, 4096) * 4, true, s)); }
+void* gemm_workspace(hipStream_t s) { return scratch("gemm_workspace", GEMM_WORKSPACE_BYTES, true, s); }
 }  // namespace
 
-void reserve_scratch(int rows, int vocab, int n_heads, int head_dim) {
+void reserve_attention_scratch(int rows, int n_heads, int head_dim, hipStream_t stream) {
+    if (rows < 1 || n_heads < 1 || head_dim < 1) return;
+    // (every launch shape keeps pairs x splits within max(8 x pairs, 256))
+    decode_partials(std::max<size_t>(static_cast<size_t>(rows) * n_heads * DECODE_MAX_SPLIT, 256) * (head_dim + 2), stream);
+    decode_counters(static_cast<size_t>(rows) * n_heads, stream);
+}
+
+void reserve_sampling_scratch(int rows, int vocab, hipStream_t stream) {
     const size_t chunks = static_cast<size_t>(mllm_argmax_chunks(vocab));
-    argmax_values(rows * chunks);
-    argmax_indices(rows * chunks);
-    gemm_workspace();
-    if (n_heads > 0 && head_dim > 0) {
-        // (every launch shape keeps pairs x splits within max(4 x pairs, 256))
-        decode_partials(std::max<size_t>(static_cast<size_t>(rows) * n_heads * DECODE_MAX_SPLIT, 256) * (head_dim + 2));
-        decode_counters(static_cast<size_t>(rows) * n_heads);
+    argmax_values(std::max(rows, 1) * chunks, stream);
+    argmax_indices(std::max(rows, 1) * chunks, stream);
+}
+
+void reserve_linear_scratch(hipStream_t stream) { gemm_workspace(stream); }
+
+void release_scratch(hipStream_t stream) {
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    const int dev = current_device();
+    bool any = false;
+    for (auto it = g_scratch.begin(); it != g_scratch.end();) {
+        if (it->first.device == dev && it->first.stream == stream) {
+            if (!any) { (void)hipStreamSynchronize(stream); any = true; }
+            (void)hipFree(it->second.ptr);
+            it = g_scratch.erase(it);
+        } else {
+            ++it;
+        }
     }
 }
 
-uint64_t scratch_generation() {
+void* scratch_address(const char* name, hipStream_t stream) {
     std::lock_guard<std::mutex> lock(g_scratch_mutex);
-    return g_generation;
+    auto it = g_scratch.find(Key{current_device(), stream, name});
+    return it == g_scratch.end() ? nullptr : it->second.ptr;
 }
 
-void* scratch_address(const char* name) {
+size_t scratch_bytes() {
     std::lock_guard<std::mutex> lock(g_scratch_mutex);
-    auto it = g_scratch.find({current_device(), name});
-    return it == g_scratch.end() ? nullptr : it->second.ptr;
+    const int dev = current_device();
+    size_t n = 0;
+    for (const auto& kv : g_scratch)
+        if (kv.first.device == dev) n += kv.second.bytes;
+    return n;
 }
 
 Tuning& tuning() {
@@ -228,7 +256,7 @@ void linear(const Tensor2& a, const Tensor2& w, const float* bias, const Tensor2
                                kv->slots, kv->k_pages.data, kv->v_pages.data, kv->q_cols, static_cast<int>(kv->k_pages.cols),
                                stream);
     } else {
-        void* ws = M <= 256 ? gemm_workspace() : nullptr;
+        void* ws = M <= 256 ? gemm_workspace(stream) : nullptr;
         rc = mllm_gemm_bf16(a.data, static_cast<int>(a.stride), w.data, static_cast<int>(w.stride), bias, out.data,
                             static_cast<int>(out.stride), static_cast<int>(M), static_cast<int>(N), static_cast<int>(K),
                             epilogue, ws, ws ? GEMM_WORKSPACE_BYTES : 0, stream);
@@ -399,8 +427,8 @@ bool paged_attention(const AttentionArgs& a, AttentionSplits* splits, hipStream_
         bool merge_kernel = false;
         decode_launch_shape(pairs, a.max_ctx_len, unmerged, &nsplit, &waves, &merge_kernel);
         unmerged = unmerged && nsplit > 1 && !merge_kernel;
-        float* ws = decode_partials(nsplit > 1 ? static_cast<size_t>(pairs) * nsplit * (a.head_dim + 2) : 1);
-        int* counters = decode_counters(pairs);
+        float* ws = decode_partials(nsplit > 1 ? static_cast<size_t>(pairs) * nsplit * (a.head_dim + 2) : 1, stream);
+        int* counters = decode_counters(pairs, stream);
         // every sequence of the batch brings one token: token t is sequence t, and the kernel need not load that
         const int* seq_of_token = (a.n_single == T && T == a.n_seqs) ? nullptr : a.token_seq;
         check(mllm_decode_attention(a.q.data, static_cast<int>(a.q.stride), a.q_col, a.k_pages.data, a.v_pages.data, kv_dim,
@@ -408,6 +436,8 @@ bool paged_attention(const AttentionArgs& a, AttentionSplits* splits, hipStream_
                                     a.head_dim, a.page_size, a.scale, a.window, nsplit, waves, a.out.data,
                                     static_cast<int>(a.out.stride), ws, counters, a.k_col, a.v_col, slots,
                                     unmerged || merge_kernel ? 1 : 0, a.q.dtype, stream), "decode_attention");
+        tuning().seen.max_decode_splits = std::max(tuning().seen.max_decode_splits, nsplit);
+        if (merge_kernel) tuning().seen.merge_kernel_launches += 1;
         if (merge_kernel)
             check(mllm_merge_attention_splits(ws, T, a.n_heads, a.head_dim, nsplit, a.out.data, static_cast<int>(a.out.stride),
                                               a.q.dtype, stream), "merge_splits");
@@ -424,12 +454,14 @@ bool paged_attention(const AttentionArgs& a, AttentionSplits* splits, hipStream_
     }
     if (tiles_ok) {
         // prompt portions: tiles of 64 queries on the matrix cores
+        tuning().seen.prefill_tile_launches += 1;
         check(mllm_prefill_attention_bf16(a.q.data, static_cast<int>(a.q.stride), a.q_col, a.k_pages.data, a.v_pages.data, kv_dim,
                                           a.block_tables, a.max_blocks, a.cu_q, a.ctx_len, a.n_seqs, T / 64 + a.n_seqs, a.n_heads,
                                           a.n_kv_heads, a.head_dim, a.page_size, a.scale, a.window, a.out.data,
                                           static_cast<int>(a.out.stride), stream), "prefill_attention");
         return false;
     }
+    tuning().seen.generic_attention_launches += 1;
     check(mllm_paged_attention_generic(a.q.data, static_cast<int>(a.q.stride), a.q_col, a.k_pages.data, a.v_pages.data, kv_dim,
                                        a.block_tables, a.max_blocks, a.token_seq, a.positions, T, a.n_heads, a.n_kv_heads,
                                        a.head_dim, a.page_size, a.scale, a.window, a.out.data, static_cast<int>(a.out.stride),
@@ -444,8 +476,8 @@ void argmax(const Tensor2& logits, int* out, hipStream_t stream) {
     if (logits.dtype != F32) fail("argmax: logits must be float32");
     const int n = static_cast<int>(logits.rows), V = static_cast<int>(logits.cols);
     const size_t chunks = static_cast<size_t>(mllm_argmax_chunks(V));
-    float* pv = argmax_values(n * chunks);
-    int* pi = argmax_indices(n * chunks);
+    float* pv = argmax_values(n * chunks, stream);
+    int* pi = argmax_indices(n * chunks, stream);
     check(mllm_argmax(static_cast<const float*>(logits.data), static_cast<int>(logits.stride), n, V, out, pv, pi, stream), "argmax");
 }
 

@@ -2,11 +2,11 @@
 //
 // Every op checks on the host that shapes, strides and dtypes are what the kernel it picks and
 // that kernel's grid assume, chooses among the kernels of an operation by size, and launches on
-// the stream it is given (so the calls can be captured in a HIP graph). A refusal is an OpError
+// the stream it is given. A refusal is an OpError
 // with a message that names the sizes. There is no CPU path.
 //
-// The native parts (parts.h) and, through the C ABI, the Python face (kernels/ops.py: tests and
-// parts written in Python) call the same functions, so the choice of kernels is made in one place.
+// The parts (parts.h) and, through the C ABI, the kernel tests (kernels/ops.py) call the same
+// functions, so the choice of kernels is made in one place.
 #pragma once
 
 #include <hip/hip_runtime.h>
@@ -56,7 +56,7 @@ struct KvScatter {
 // The output of decode attention that has not been merged yet: every (token, head) pair's keys were
 // split over `nsplit` workgroups whose states lie in the attention scratch (layout:
 // kernels/attention_decode.hip). `linear_from_splits` merges while it loads. Valid until the next
-// attention launch on the device.
+// attention launch on the same stream.
 struct AttentionSplits {
     float* ws = nullptr;
     int n_tokens = 0, n_heads = 0, head_dim = 0, nsplit = 0, dtype = BF16;
@@ -86,12 +86,18 @@ struct AttentionArgs {
     int may_split = 0;             // != 0: the caller takes an AttentionSplits in place of `out`
 };
 
-// -- scratch: device memory that kernels need beyond inputs and outputs, one set per device ----
-// A captured graph keeps the address it was captured with; `scratch_generation()` changes whenever
-// a buffer was replaced by a larger one, and whoever holds graphs compares it before replaying.
-void reserve_scratch(int rows, int vocab, int n_heads, int head_dim);
-uint64_t scratch_generation();
-void* scratch_address(const char* name);      // nullptr if not allocated yet (tests)
+// -- scratch: device memory that kernels need beyond inputs and outputs, one set per stream -----------
+// Work on one stream runs in order, so the kernels launched on it can share these buffers; two runners
+// (two streams) never share one, so their steps may overlap on the device. A part says what its kernels
+// need through the reserve_* calls when its runner is built, so that no step allocates; an op that is
+// called with more than was reserved (tests call ops directly) grows the buffer, which synchronises the
+// device. release_scratch frees a stream's buffers (the owner of the stream calls it before it destroys it).
+void reserve_attention_scratch(int rows, int n_heads, int head_dim, hipStream_t stream);
+void reserve_sampling_scratch(int rows, int vocab, hipStream_t stream);
+void reserve_linear_scratch(hipStream_t stream);
+void release_scratch(hipStream_t stream);
+void* scratch_address(const char* name, hipStream_t stream);      // nullptr if not allocated yet (tests)
+size_t scratch_bytes();                                            // all streams of the current device (tests)
 
 // -- tuning hooks (tests and tuning scripts) ---------------------------------------------------------
 struct Tuning {
@@ -100,6 +106,11 @@ struct Tuning {
     int merge_max_rows = 16;                          // tokens whose splits a product merges while loading
     int long_context_splits = 1;                      // 1: few pairs with long contexts are split over up to 256 workgroups
     int ln_fuse_max_rows = 32;                        // rows up to which the norm is fused into the few-row product
+    // what the ops chose since the last reset (tests read it back instead of trusting the thresholds)
+    struct Seen {
+        int max_decode_splits = 0;                    // most workgroups a (token, head) pair's keys were split over
+        long long merge_kernel_launches = 0, prefill_tile_launches = 0, generic_attention_launches = 0;
+    } seen;
 };
 Tuning& tuning();
 

@@ -8,10 +8,17 @@
 //
 // Interfaces (`x` is the fp32 residual stream [T, hidden]; `h` a normalised activation in the
 // compute dtype; `step` the batch's index arrays; `arena` memory for the step's temporaries):
+//   Embedding::forward(step, position, x)     x[t,:] = the token's row (+ the position table's)
+//   PositionEncoding::table() / in_mixer(qkv, heads, step)   a table for the embedding, or a turn of
+//                                             queries and keys inside the mixer before keys are written
 //   Norm::forward(x, rows, n) -> h            Norm::linear(x, lin, out, epilogue, rows)
 //   Mixer::forward(h, step, cache, x, write)  adds the mixer's output into x
 //   FeedForward::forward(h, step, x)          adds its output into x
 //   Block::forward(x, step, cache, write)     runs one layer on the stream
+//   Head::forward(x, final_norm, rows, logits)  fp32 logits of the wanted rows
+// Every part also says what it asks of the cache (Mixer::cache_need), what scratch its kernels need
+// (reserve), how much of the step's arena it takes (workspace_bytes) and what a step costs through it
+// (add_cost: bytes of weights, flops).
 //
 // The reference's model has these pieces fixed in one class
 // (/root/reference/src/model/gpt2_model.cu:275-363 block_prefill, :404-428 the head).
@@ -100,11 +107,29 @@ struct CacheView {
     int n_slots = 0;
 };
 
+// What a cache of the execution order asks of the cache manager: said by the mixer that writes it.
+struct CacheNeed {
+    int kind = 0;                        // 1 keys and values in pages, 2 fixed-size state, 0 none
+    int n_kv_heads = 0, head_dim = 0, window = 0;
+    size_t state_bytes = 0;
+};
+
+// What one step costs, summed over the parts (the benchmark's roofline figures are made from these).
+struct StepCost {
+    double weight_bytes = 0;             // weights a step reads once, whatever its batch
+    double flops_per_token = 0;          // matrix products of the layers, per token
+    double attention_flops_per_key = 0;  // per (token, attended key), summed over the attention calls
+    double flops_per_logits_row = 0;     // the head's product for one wanted row
+};
+
+class PositionEncoding;
+
 // A bag of parameters a part is built from.
 struct Params {
     std::map<std::string, double> num;
     std::map<std::string, std::string> str;
     std::map<std::string, Tensor2> tensor;
+    std::shared_ptr<const PositionEncoding> position;      // the model's position encoding, for mixers that take one
 
     double number(const std::string& key) const;
     double number(const std::string& key, double fallback) const;
@@ -126,6 +151,37 @@ public:
     const float* bias = nullptr;
     int in_features() const { return static_cast<int>(weight.cols); }
     int out_features() const { return static_cast<int>(weight.rows); }
+    void add_cost(StepCost& c) const {
+        c.weight_bytes += static_cast<double>(weight.rows) * weight.cols * weight.esz() + (bias ? 4.0 * weight.rows : 0.0);
+        c.flops_per_token += 2.0 * weight.rows * weight.cols;
+    }
+};
+
+// How positions enter the model. Either a table whose row is added to the token's embedding (learned
+// absolute positions: the embedding kernel adds it), or a turn of queries and keys inside the mixer,
+// in place on the qkv rows, before the keys go to the pages (rotary schemes), or nothing.
+class PositionEncoding {
+public:
+    virtual ~PositionEncoding() = default;
+    virtual const Tensor2* table() const { return nullptr; }
+    virtual bool applies_in_mixer() const { return false; }
+    // qkv rows: n_heads query heads, then n_kv_heads key heads, then the values (left alone)
+    virtual void in_mixer(const Tensor2& qkv, int n_heads, int n_kv_heads, int head_dim, const StepView& step,
+                          hipStream_t s) const {
+        (void)qkv; (void)n_heads; (void)n_kv_heads; (void)head_dim; (void)step; (void)s;
+    }
+    virtual int max_positions() const { return 0; }       // 0: unbounded
+    virtual void add_cost(StepCost&) const {}
+};
+
+// Token ids to rows of the fp32 stream.
+class Embedding {
+public:
+    virtual ~Embedding() = default;
+    virtual int vocab_size() const = 0;
+    virtual int hidden_size() const = 0;
+    virtual void forward(const StepView& step, const PositionEncoding* position, const Tensor2& x, hipStream_t s) const = 0;
+    virtual void add_cost(StepCost&) const {}
 };
 
 class Norm {
@@ -138,6 +194,7 @@ public:
     virtual void linear(const Tensor2& x, const Linear& lin, const Tensor2& out, int epilogue, const int* rows,
                         const KvScatter* kv, Arena& arena, hipStream_t s) const;
     virtual size_t workspace_bytes(int rows) const = 0;
+    virtual void add_cost(StepCost&) const {}
     int dtype = BF16;
 };
 
@@ -145,13 +202,14 @@ public:
 // absorb the norm.
 class NormedInput {
 public:
-    NormedInput(const Norm& norm, const Tensor2& x) : norm_(norm), x_(x) {}
+    NormedInput(const Norm& norm, const Tensor2& x) : norm_(&norm), x_(x) {}
+    explicit NormedInput(const Tensor2& h) : norm_(nullptr), x_(h), h_(h), have_(true) {}     // normalised already
     const Tensor2& tensor(Arena& arena, hipStream_t s);
     void linear(const Linear& lin, const Tensor2& out, int epilogue, const KvScatter* kv, Arena& arena, hipStream_t s);
     int64_t rows() const { return x_.rows; }
 
 private:
-    const Norm& norm_;
+    const Norm* norm_;
     Tensor2 x_, h_;
     bool have_ = false;
 };
@@ -162,6 +220,11 @@ public:
     virtual void forward(NormedInput& h, const StepView& step, const CacheView& cache, const Tensor2& x, bool write,
                          Arena& arena, hipStream_t s) const = 0;
     virtual size_t workspace_bytes(int tokens) const = 0;
+    virtual CacheNeed cache_need() const = 0;
+    // Scratch that the mixer's kernels need on stream `s` for steps of up to max_seqs sequences: taken
+    // now, so that no step allocates.
+    virtual void reserve(int max_seqs, hipStream_t s) const { (void)max_seqs; (void)s; }
+    virtual void add_cost(StepCost&) const {}
 };
 
 class FeedForward {
@@ -169,6 +232,8 @@ public:
     virtual ~FeedForward() = default;
     virtual void forward(NormedInput& h, const StepView& step, const Tensor2& x, Arena& arena, hipStream_t s) const = 0;
     virtual size_t workspace_bytes(int tokens) const = 0;
+    virtual void reserve(int max_seqs, hipStream_t s) const { (void)max_seqs; (void)s; }
+    virtual void add_cost(StepCost&) const {}
 };
 
 class Block {
@@ -177,22 +242,48 @@ public:
     virtual void forward(const Tensor2& x, const StepView& step, const CacheView& cache, bool write, Arena& arena,
                          hipStream_t s) const = 0;
     virtual size_t workspace_bytes(int tokens) const = 0;
+    virtual CacheNeed cache_need() const = 0;             // its mixer's
+    virtual void reserve(int max_seqs, hipStream_t s) const = 0;
+    virtual void add_cost(StepCost&) const = 0;
+};
+
+// The stream's wanted rows to fp32 logits.
+class Head {
+public:
+    virtual ~Head() = default;
+    virtual int vocab_size() const = 0;
+    // logits[i,:] = head(final_norm(x[rows[i],:]))
+    virtual void forward(const Tensor2& x, const Norm& final_norm, const int* rows, const Tensor2& logits, Arena& arena,
+                         hipStream_t s) const = 0;
+    virtual size_t workspace_bytes(int rows) const = 0;
+    virtual void add_cost(StepCost&) const {}
 };
 
 // -- registries: kind name -> factory ---------------------------------------------------------------
+using PositionFactory = std::function<std::shared_ptr<const PositionEncoding>(const Params&)>;
+using EmbeddingFactory = std::function<std::unique_ptr<Embedding>(const Params&)>;
+using HeadFactory = std::function<std::unique_ptr<Head>(const Params&)>;
 using NormFactory = std::function<std::unique_ptr<Norm>(const Params&)>;
 using MixerFactory = std::function<std::unique_ptr<Mixer>(const Params&)>;
 using FeedForwardFactory = std::function<std::unique_ptr<FeedForward>(const Params&)>;
 using BlockFactory = std::function<std::unique_ptr<Block>(std::unique_ptr<Mixer>, std::unique_ptr<FeedForward>,
                                                          std::vector<std::unique_ptr<Norm>>)>;
+void register_position(const std::string& kind, PositionFactory f);
+void register_embedding(const std::string& kind, EmbeddingFactory f);
+void register_head(const std::string& kind, HeadFactory f);
 void register_norm(const std::string& kind, NormFactory f);
 void register_mixer(const std::string& kind, MixerFactory f);
 void register_feed_forward(const std::string& kind, FeedForwardFactory f);
 void register_block(const std::string& kind, BlockFactory f);
-bool has_part(const std::string& category, const std::string& kind);     // category: norm | mixer | feed_forward | block
+// category: position | embedding | head | norm | mixer | feed_forward | block
+bool has_part(const std::string& category, const std::string& kind);
+std::shared_ptr<const PositionEncoding> build_position(const std::string& kind, const Params& p);
+std::unique_ptr<Embedding> build_embedding(const std::string& kind, const Params& p);
+std::unique_ptr<Head> build_head(const std::string& kind, const Params& p);
 std::unique_ptr<Norm> build_norm(const std::string& kind, const Params& p);
 std::unique_ptr<Mixer> build_mixer(const std::string& kind, const Params& p);
 std::unique_ptr<FeedForward> build_feed_forward(const std::string& kind, const Params& p);
+// (the feed-forward may be null: a layer without one; the norms are those of the sub-layers that exist)
 std::unique_ptr<Block> build_block(const std::string& kind, std::unique_ptr<Mixer> m, std::unique_ptr<FeedForward> f,
                                    std::vector<std::unique_ptr<Norm>> norms);
 
@@ -202,19 +293,25 @@ struct LayerCall {
     bool write = true;
 };
 
-// A decoder-only model: embedding (+ learned position table), the calls of the execution order, the
-// final norm and the head (tied to the embedding) on the wanted rows only.
+// A decoder-only model: the embedding (with the position encoding's table, if it has one), the calls
+// of the execution order, and the final norm and the head on the wanted rows only.
 class DecoderModel {
 public:
-    Tensor2 wte;                   // [V, D]
-    Tensor2 wpe;                   // [P, D] or empty
+    std::unique_ptr<Embedding> embedding;
+    std::shared_ptr<const PositionEncoding> position;     // may be null: no position encoding
     std::vector<std::unique_ptr<Block>> layers;
     std::vector<LayerCall> order;
     std::unique_ptr<Norm> final_norm;
+    std::unique_ptr<Head> head;
     int dtype = BF16;
 
-    int vocab_size() const { return static_cast<int>(wte.rows); }
-    int hidden_size() const { return static_cast<int>(wte.cols); }
+    int vocab_size() const { return head->vocab_size(); }
+    int hidden_size() const { return embedding->hidden_size(); }
+    // What each cache index of the execution order asks for: the need of the layer that writes it.
+    std::vector<CacheNeed> cache_needs() const;
+    // Every part takes the scratch its kernels need on `s` for steps of up to max_seqs sequences.
+    void reserve(int max_seqs, hipStream_t s) const;
+    StepCost cost() const;
     // Bytes of arena that a step of `tokens` tokens and `n_logits` wanted rows needs at most.
     size_t workspace_bytes(int tokens, int n_logits) const;
     // Runs the step; fp32 logits [n_logits, V] into `logits` (untouched if no logits are wanted).

@@ -41,8 +41,11 @@ SafetensorsFile::SafetensorsFile(const std::string& path) : path_(path) {
     const unsigned char* base = static_cast<const unsigned char*>(map_);
     uint64_t hlen = 0;
     for (int i = 7; i >= 0; --i) hlen = (hlen << 8) | base[i];
-    if (hlen == 0 || 8 + hlen > size_)
+    // (compared without adding to hlen, which may be anything up to 2^64 - 1; headers beyond 100 MB are refused
+    // as the format's own library does)
+    if (hlen == 0 || hlen > size_ - 8)
         throw WeightsError(path + ": header length " + std::to_string(hlen) + " exceeds the file size " + std::to_string(size_));
+    if (hlen > 100u * 1000u * 1000u) throw WeightsError(path + ": header of " + std::to_string(hlen) + " bytes is larger than 100 MB");
     Json header;
     try {
         header = Json::parse(std::string(reinterpret_cast<const char*>(base + 8), hlen));
@@ -60,7 +63,11 @@ SafetensorsFile::SafetensorsFile(const std::string& path) : path_(path) {
             const auto& off = kv.second.at("data_offsets").array();
             if (off.size() != 2) throw JsonError("data_offsets must have two entries");
             const int64_t b = off[0].integer(), e = off[1].integer();
-            const size_t want = static_cast<size_t>(t.numel()) * dtype_bytes(t.dtype, path, kv.first);
+            const int64_t numel = t.numel();
+            const size_t esz = dtype_bytes(t.dtype, path, kv.first);
+            if (numel < 0 || static_cast<uint64_t>(numel) > UINT64_MAX / 8)
+                throw WeightsError(path + ": tensor '" + kv.first + "' has a negative dimension or more elements than can be counted");
+            const size_t want = static_cast<size_t>(numel) * esz;
             if (b < 0 || e < b || static_cast<size_t>(e) > data_len)
                 throw WeightsError(path + ": tensor '" + kv.first + "' has offsets [" + std::to_string(b) + ", " + std::to_string(e) +
                                    ") outside the file's " + std::to_string(data_len) + " data bytes");

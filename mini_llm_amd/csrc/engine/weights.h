@@ -29,7 +29,15 @@ struct StoredTensor {
     std::vector<int64_t> shape;
     const unsigned char* data = nullptr;
     size_t bytes = 0;
-    int64_t numel() const { int64_t n = 1; for (int64_t s : shape) n *= s; return n; }
+    // the product of the dimensions; -1 if one is negative or the product does not fit 63 bits
+    int64_t numel() const {
+        int64_t n = 1;
+        for (int64_t s : shape) {
+            if (s < 0 || (s != 0 && n > INT64_MAX / s)) return -1;
+            n *= s;
+        }
+        return n;
+    }
 };
 
 // 8-byte little-endian header length, a JSON header {name: {dtype, shape, data_offsets}}

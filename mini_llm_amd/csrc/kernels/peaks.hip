@@ -106,26 +106,7 @@ fma_f32_loop_kernel(int iters, float* __restrict__ sink) {
     if (t == 12345.678f) sink[0] = t;
 }
 
-// out[lane] = maximum, out[64 + lane] = sum over lanes l, l ^ 16, l ^ 32, l ^ 48 of in[lane] (one wavefront),
-// then in[lane ^ 8], in[lane ^ 16], in[lane ^ 32], in[lane ^ 4]: what rows_max, rows_sum and lane_xor of
-// common.h give, for a test of the lane exchanges they are built on. out: 384 floats.
-__global__ void rows_check_kernel(const float* __restrict__ in, float* __restrict__ out) {
-    const float v = in[threadIdx.x];
-    out[threadIdx.x] = rows_max(v);
-    out[64 + threadIdx.x] = rows_sum(v);
-    out[128 + threadIdx.x] = lane_xor(v, 8);
-    out[192 + threadIdx.x] = lane_xor(v, 16);
-    out[256 + threadIdx.x] = lane_xor(v, 32);
-    out[320 + threadIdx.x] = lane_xor(v, 4);
-}
-
 extern "C" {
-
-int mllm_rows_check(const float* in, float* out, hipStream_t stream) {
-    rows_check_kernel<<<1, 64, 0, stream>>>(in, out);
-    MLLM_LAUNCH_CHECK();
-    return 0;
-}
 
 // Each launcher queues `reps` launches on the stream; the caller times them with events.
 // Bytes moved per launch: n_bytes (read) or 2 * n_bytes (copy). n_bytes must be a multiple of 16.

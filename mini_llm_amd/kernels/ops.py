@@ -1,21 +1,19 @@
 """The engine's device operations, seen from Python: a thin face over the native ops
 (csrc/engine/ops.cc), which check shapes, strides and dtypes, choose among the kernels of an
-operation by size and launch on the current HIP stream (so the calls can be captured in a HIP
-graph). The native parts call the same functions directly; this face serves the tests and parts
-written in Python.
+operation by size and launch on torch's current HIP stream. The engine's parts call the same
+functions natively; this face serves the tests of a kernel alone and tuning scripts.
 
 There is no CPU path: a tensor that is not on the GPU, or a library that cannot be built and
-loaded, raises. Parts look ops up as ``ops.<name>`` at call time.
+loaded, raises.
 """
 from __future__ import annotations
 
 import ctypes
-import weakref
 from typing import Optional
 
 import torch
 
-from ..build import load_library
+from .. import native
 
 EPILOGUES = {"store": 0, "gelu_tanh": 1, "gelu_erf": 2, "add_residual": 3, "store_f32": 4}
 _DT = {torch.float32: 0, torch.bfloat16: 1}
@@ -59,14 +57,9 @@ def engine_library():
     global _lib
     if _lib is not None:
         return _lib
-    lib = load_library("engine")
+    lib = native.lib()
     T2p, sz = ctypes.POINTER(Tensor2), ctypes.c_size_t
     sigs = {
-        "mllm_last_error": (ctypes.c_char_p, []),
-        "mllm_reserve_scratch": (_i, [_i, _i, _i, _i]),
-        "mllm_scratch_generation": (ctypes.c_ulonglong, []),
-        "mllm_scratch_address": (_vp, [ctypes.c_char_p]),
-        "mllm_set_tuning": (_i, [ctypes.c_char_p, _i, _i]),
         "mllm_op_embed": (_i, [_vp, _vp, T2p, T2p, T2p, _vp]),
         "mllm_op_select_tokens": (_i, [_vp, _vp, _vp, _i, _i, _vp]),
         "mllm_op_reset_state": (_i, [_vp, sz, _i, _vp, _vp, _i, _vp]),
@@ -148,54 +141,31 @@ def _f32vec(t: Optional[torch.Tensor], name: str, n: int) -> None:
 
 
 # -- scratch and tuning -----------------------------------------------------------------------------
-# Scratch buffers: device memory that a kernel needs beyond its inputs and outputs (argmax partial
-# results, the states of split decode attention, shared-tile sums). One set per device, owned by the
-# native side. A captured HIP graph keeps the raw address of the buffer it was captured with, so a
-# buffer is never replaced behind a graph's back: callers that capture graphs reserve room for their
-# largest launch first (``reserve_scratch``), and if a buffer must grow after all, everyone registered
-# with ``on_scratch_growth`` is told at the next ``notify_scratch_growth()``, and drops its graphs.
-_GROWTH_LISTENERS: list = []
-_seen_generation = 0
+# Scratch buffers (device memory that a kernel needs beyond its inputs and outputs: argmax partial
+# results, the states of split decode attention, shared-tile sums) are kept per stream by the native
+# side; ops called from here use the set of torch's current stream.
+
+def scratch_address(name: str) -> int:
+    """Address of a scratch buffer of the current stream (0 if it does not exist yet)."""
+    return engine_library().mllm_scratch_address(name.encode(), _stream()) or 0
 
 
-def on_scratch_growth(method) -> None:
-    """Registers a bound method that is called (with no arguments) when a scratch buffer has been
-    replaced by a larger one (noticed by ``notify_scratch_growth``). Held weakly."""
-    _GROWTH_LISTENERS.append(weakref.WeakMethod(method))
+def scratch_bytes() -> int:
+    """Bytes of scratch that all streams of the current device hold."""
+    return int(engine_library().mllm_scratch_bytes())
 
 
-def notify_scratch_growth() -> bool:
-    """Tells the listeners if a scratch buffer has been replaced since the last call. Whoever replays
-    graphs calls this first."""
-    global _seen_generation
-    gen = engine_library().mllm_scratch_generation()
-    if gen == _seen_generation:
-        return False
-    _seen_generation = gen
-    alive = []
-    for ref in _GROWTH_LISTENERS:
-        fn = ref()
-        if fn is not None:
-            fn()
-            alive.append(ref)
-    _GROWTH_LISTENERS[:] = alive
-    return True
+def seen(name: str) -> int:
+    """What the ops chose since ``reset_seen()``: "max_decode_splits", "merge_kernel_launches",
+    "prefill_tile_launches", "generic_attention_launches"."""
+    v = engine_library().mllm_get_seen(name.encode())
+    if v < 0:
+        raise KernelError(f"unknown counter '{name}'")
+    return int(v)
 
 
-def scratch_address(device, name: str) -> int:
-    """Address of a scratch buffer (0 if it does not exist yet): tests check that it stays put."""
-    with torch.cuda.device(torch.device(device)):
-        return engine_library().mllm_scratch_address(name.encode()) or 0
-
-
-def reserve_scratch(device, rows: int, vocab: int, n_heads: int = 0, head_dim: int = 0) -> None:
-    """Makes the scratch buffers large enough for ``rows`` sampled rows of ``vocab`` logits and for
-    decode attention over ``rows`` tokens of ``n_heads`` heads, so that no later launch up to these
-    sizes replaces them."""
-    if torch.device(device).type != "cuda":
-        return
-    with torch.cuda.device(torch.device(device)):
-        _ok(engine_library().mllm_reserve_scratch(int(rows), int(vocab), int(n_heads), int(head_dim)))
+def reset_seen() -> None:
+    _ok(engine_library().mllm_set_tuning(b"reset_seen", 0, 0))
 
 
 # Tuning hooks: tests and tuning scripts set these module attributes; they reach the native side at the

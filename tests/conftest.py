@@ -37,8 +37,7 @@ CONFIGS = {**TINY, **REAL}
 @pytest.fixture(scope="session")
 def real_model_dirs(tmp_path_factory):
     """Model folders at GPT-2 small and XL layer sizes (two layers each), random weights."""
-    from mini_llm_amd.weights.random_init import write_random_model
-    import mini_llm_amd.models  # noqa: F401
+    from mini_llm_amd import write_random_model
     out = {}
     for name, (cfg, seed, _) in REAL.items():
         d = tmp_path_factory.mktemp(f"real_{name}")
@@ -50,8 +49,7 @@ def real_model_dirs(tmp_path_factory):
 @pytest.fixture(scope="session")
 def tiny_model_dirs(tmp_path_factory):
     """Model folders of the two tiny configurations, random weights, made once per session."""
-    from mini_llm_amd.weights.random_init import write_random_model
-    import mini_llm_amd.models  # noqa: F401
+    from mini_llm_amd import write_random_model
     out = {}
     for name, (cfg, seed, _) in TINY.items():
         d = tmp_path_factory.mktemp(f"tiny_{name}")

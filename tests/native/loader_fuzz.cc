@@ -3,6 +3,7 @@
 // field changed, the file cut) and opened again; every outcome has to be either a file that still reads
 // or a WeightsError, never a crash, an overflow or a read outside the mapping. Also random texts through
 // the JSON parser. Usage: loader_fuzz FILE.safetensors SCRATCH_FILE [rounds]
+#include <cstdint>
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
@@ -59,6 +60,37 @@ int main(int argc, char** argv) {
         } catch (const WeightsError&) {
             ++refused;
         }
+    }
+    // Fixed inputs that random damage does not reach: a header nested millions deep (the parser recurses
+    // per level), header lengths at the top of the 64-bit range (a sum with them wraps), and shapes whose
+    // product overflows or is negative. Each has to be refused with a WeightsError.
+    {
+        auto refused_file = [&](const std::vector<char>& bytes) {
+            { std::ofstream out(argv[2], std::ios::binary | std::ios::trunc); out.write(bytes.data(), static_cast<std::streamsize>(bytes.size())); }
+            try { SafetensorsFile f(argv[2]); return false; } catch (const WeightsError&) { return true; }
+        };
+        auto with_header = [&](const std::string& header) {
+            std::vector<char> b(8);
+            const uint64_t n = header.size();
+            std::memcpy(b.data(), &n, 8);
+            b.insert(b.end(), header.begin(), header.end());
+            b.insert(b.end(), good.begin() + 8 + static_cast<std::ptrdiff_t>(hlen), good.end());
+            return b;
+        };
+        int fixed_refused = 0, fixed = 0;
+        for (const std::string& open : {std::string(3000000, '['), std::string(3000000, '{')}) { ++fixed; fixed_refused += refused_file(with_header(open)); }
+        for (uint64_t v : {UINT64_MAX, UINT64_MAX - 7, UINT64_MAX - 8, uint64_t(1) << 63}) {
+            std::vector<char> b = good;
+            std::memcpy(b.data(), &v, 8);
+            ++fixed; fixed_refused += refused_file(b);
+        }
+        for (const char* shape : {"[3000000000,3000000000,4]", "[-4]", "[9000000000000000,9000000000000000]", "[-1,-1]"}) {
+            ++fixed;
+            fixed_refused += refused_file(with_header(std::string("{\"t\":{\"dtype\":\"F32\",\"shape\":") + shape + ",\"data_offsets\":[0,16]}}"));
+        }
+        if (fixed_refused != fixed) { std::printf("failed: %d of %d fixed damaged files were refused\n", fixed_refused, fixed); return 1; }
+        try { (void)Json::parse(std::string(100000, '[')); std::puts("failed: deep nesting parsed"); return 1; } catch (const JsonError&) {}
+        refused += fixed_refused;
     }
     int parsed = 0, rejected = 0;
     const std::string alphabet = "{}[]\",:0123456789.-+eE tfnulsra\\\n\"x";

@@ -1,5 +1,5 @@
 """Builds replay traces (the four schedule families) and runs them, in-process through the
-engine's ModelRunner or through bin/trace_run, collecting logits per request position."""
+engine's runner or through bin/trace_run, collecting logits per request position."""
 from __future__ import annotations
 
 import json
@@ -122,7 +122,7 @@ def collect(steps, outputs: Dict[int, np.ndarray], vocab: int) -> Dict[str, Dict
 
 
 def run_in_process(runner, steps) -> Dict[int, np.ndarray]:
-    from mini_llm_amd.engine.step import StepEntry
+    from mini_llm_amd import StepEntry
     ids: Dict[str, int] = {}
     out = {}
     nxt = 0
@@ -135,7 +135,7 @@ def run_in_process(runner, steps) -> Dict[int, np.ndarray]:
             entries.append(StepEntry(ids[e["id"]], e["tokens"], e["want"]))
         logits = runner.step(entries)
         if logits is not None:
-            out[s["step"]] = logits.float().cpu().numpy()
+            out[s["step"]] = logits.copy()
         for rid in s["end"]:
             runner.end_request(ids.pop(rid))
     return out

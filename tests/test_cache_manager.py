@@ -5,8 +5,7 @@ import random
 import numpy as np
 import pytest
 
-from mini_llm_amd.cache.manager import (CacheManager, CacheStorage, GroupSpec, KVCacheSpec, OutOfPages,
-                                        StateCacheSpec)
+from mini_llm_amd.cache.manager import CacheManager, GroupSpec, OutOfPages
 
 
 def test_pages_are_taken_per_block_and_reused_lifo():
@@ -128,17 +127,3 @@ def test_random_orders_keep_every_page_accounted_for(seed):
     for rid in list(live):
         cm.free_request(rid)
     assert all(cm.free_pages(g) == groups[g].n_pages for g in range(3)) and cm.free_state_slots() == 6
-
-
-def test_storage_groups_layers_by_need():
-    import torch
-    specs = [KVCacheSpec(4, 16), KVCacheSpec(4, 16), StateCacheSpec((5,)), KVCacheSpec(2, 16, window=8),
-             KVCacheSpec(4, 16)]
-    st = CacheStorage(specs, page_size=4, n_pages=10, n_state_slots=3, dtype=torch.float32, device="cpu")
-    assert st.n_groups == 2 and st.cache_group == [0, 0, -1, 1, 0]
-    assert [g.window for g in st.group_specs] == [0, 8]
-    v0, v4, v3 = st.view(0), st.view(4), st.view(3)
-    assert v0.k_pages.shape == (40, 64) and v3.k_pages.shape == (40, 32) and v3.window == 8 and v3.group == 1
-    assert v0.k_pages.data_ptr() != v4.k_pages.data_ptr() and v0.group == v4.group == 0
-    assert st.view(2).slots.shape == (3, 5)
-    assert st.bytes_per_token() == (3 * 2 * 64 + 2 * 32) * 4

@@ -42,14 +42,16 @@ def test_loaded_libraries_are_in_tree(ops):
     names = {os.path.basename(m) for m in mapped}
     for lib in ("engine", "elementwise", "gemm_bf16", "gemm_f32", "attention_decode", "attention_prefill", "sampling"):
         assert os.path.basename(build.lib_path(lib)) in names, (lib, names)
-    assert all(os.path.dirname(os.path.realpath(m)) == os.path.realpath(build.LIB_DIR) for m in mapped), mapped
+    here = os.path.realpath(os.path.join(os.path.dirname(os.path.abspath(__file__)), "native", "_lib"))     # the tests' own
+    assert all(os.path.dirname(os.path.realpath(m)) in (os.path.realpath(build.LIB_DIR), here) for m in mapped), mapped
 
 
 def test_lane_exchange_between_rows(ops):
     """The reductions over one lane of each 16-lane row (built on gfx950's row swaps) against their meaning."""
     import ctypes
+    import toy  # noqa: F401  (registers the test-only library)
     from mini_llm_amd import build
-    lib = build.load_library("peaks")
+    lib = build.load_library("lane_check")
     g = torch.Generator().manual_seed(3)
     v = torch.randn(64, generator=g)
     out = torch.zeros(384, device=DEV)
@@ -290,7 +292,7 @@ def test_linear_bf16_up_to_256_rows(ops, M, N, K):
 def test_linear_bf16_few_rows_long_k_shares_tiles(ops, M, N, K):
     """Narrow products with a long K: several workgroups share a tile and the last to arrive adds their
     parts. Every call gives the same bits (the parts are added in a fixed order, the counters are
-    left at zero), eagerly and in replays of a HIP graph."""
+    left at zero), on any stream."""
     g = torch.Generator().manual_seed(M + N + K)
     a = _rand((M, K), torch.bfloat16, g).to(DEV)
     w = _rand((N, K), torch.bfloat16, g, std=1.0 / math.sqrt(K)).to(DEV)
@@ -304,21 +306,17 @@ def test_linear_bf16_few_rows_long_k_shares_tiles(ops, M, N, K):
         outs.append(x.cpu())
     assert (outs[0].double() - ref).abs().max().item() <= 2e-5 + 2e-5 * math.sqrt(K)
     assert torch.equal(outs[0], outs[1]) and torch.equal(outs[0], outs[2])
-    x = x0.clone().to(DEV)
+    # another epilogue between two runs, and a second stream with scratch of its own: the same bits again
     y = torch.empty(M, N, dtype=torch.bfloat16, device=DEV)
     ops.linear(a, w, bias, y, "gelu_tanh")
-    torch.cuda.synchronize()
-    graph = torch.cuda.CUDAGraph()
-    with torch.cuda.graph(graph):
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        x = x0.clone().to(DEV)
         ops.linear(a, w, bias, x, "add_residual")
-        ops.linear(a, w, bias, y, "gelu_tanh")
-    y_eager = y.cpu()
-    for _ in range(3):
-        x.copy_(x0)
-        y.zero_()
-        graph.replay()
-        torch.cuda.synchronize()
-        assert torch.equal(x.cpu(), outs[0]) and torch.equal(y.cpu(), y_eager)
+        assert ops.scratch_address("gemm_workspace") != 0
+    side.synchronize()
+    assert torch.equal(x.cpu(), outs[0])
 
 
 @pytest.mark.parametrize("dtype", DTYPES)

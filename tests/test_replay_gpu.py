@@ -1,34 +1,38 @@
 """The engine on the GPU against the plain implementation, in 32-bit and in bfloat16:
 each request alone and whole; most of it in one step and the last 32 tokens one by one;
 portions of changing size down to two tokens; and mixed batches of up to four live requests
-with so few pages that they are used again. In-process through ModelRunner, and through
-bin/trace_run as a user drives it."""
-import os
-
+with so few pages that they are used again. Through the engine's runner in this process, and
+through bin/trace_run (the engine's `mini-llm replay`) as a user drives it: one runner either way."""
 import numpy as np
 import pytest
-import torch
 
+import plain_gpt2
 import replay_cases as rc
 import replay_util as ru
 from conftest import CONFIGS, TINY
 
 pytestmark = pytest.mark.gpu
 DTYPES = ["float32", "bfloat16"]
+FAMILIES = ["whole", "decode_tail", "chunks", "mixed"]
 
 
-def _runner(model_dir, name, dtype, n_pages, page=None):
-    from mini_llm_amd.engine.step import ModelRunner
-    from mini_llm_amd.models import load_model
-    model = load_model(model_dir, dtype, "cuda:0")
-    runner = ModelRunner(model, page or CONFIGS[name][2], n_pages, 8)
-    runner.cache.poison()          # an unwritten or stale page that is read shows up as NaN
+def _runner(model_dir, name, dtype, n_pages, page=None, max_num_seqs=8):
+    from mini_llm_amd import Runner
+    runner = Runner(model_dir=model_dir, dtype=dtype, page_size=page or CONFIGS[name][2], n_pages=n_pages,
+                    max_num_seqs=max_num_seqs)
+    runner.poison_cache()          # an unwritten or stale page that is read shows up as NaN
     return runner
+
+
+def _all_pages_back(runner, n_pages):
+    assert runner.check() == ""
+    info = runner.info()
+    assert info["free_pages"] == n_pages and info["n_requests"] == 0
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("name", ["a", "b"])
-@pytest.mark.parametrize("family", ["whole", "decode_tail", "chunks", "mixed"])
+@pytest.mark.parametrize("family", FAMILIES)
 def test_schedule_families_match_plain(tiny_model_dirs, name, family, dtype):
     reqs = rc.requests_for(name)
     steps = rc.families(reqs)[family]
@@ -37,13 +41,12 @@ def test_schedule_families_match_plain(tiny_model_dirs, name, family, dtype):
     runner = _runner(tiny_model_dirs[name], name, dtype, n_pages)
     out = ru.run_in_process(runner, steps)
     rc.check_against_plain(tiny_model_dirs[name], name, reqs, steps, out, dtype, label=family)
-    assert runner.manager.check() == ""
-    assert runner.manager.free_pages(0) == n_pages and runner.manager.n_requests() == 0
+    _all_pages_back(runner, n_pages)
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("name", ["small2", "xl2"])
-@pytest.mark.parametrize("family", ["whole", "decode_tail", "chunks", "mixed"])
+@pytest.mark.parametrize("family", FAMILIES)
 def test_schedule_families_match_plain_at_real_layer_sizes(real_model_dirs, name, family, dtype):
     """The same four families at the layer sizes of GPT-2 small and XL (two layers, the real vocabulary):
     the sizes at which the engine picks the matrix-core attention, the 64-wide decode attention, the
@@ -56,27 +59,37 @@ def test_schedule_families_match_plain_at_real_layer_sizes(real_model_dirs, name
     runner = _runner(real_model_dirs[name], name, dtype, n_pages)
     out = ru.run_in_process(runner, steps)
     rc.check_against_plain(real_model_dirs[name], name, reqs, steps, out, dtype, skip=skip, label=family)
-    assert runner.manager.check() == ""
-    assert runner.manager.free_pages(0) == n_pages and runner.manager.n_requests() == 0
+    _all_pages_back(runner, n_pages)
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-def test_native_step_equals_the_parts_python_forward(tiny_model_dirs, dtype):
-    """A model whose parts are all native runs its step in one native call; with `use_native` off the
-    parts' Python forward methods run instead. Same kernels, same arguments: the logits are equal
-    bit for bit, and both match the plain implementation."""
-    reqs = rc.requests_for("b", seed=3, lengths=[40, 9, 100, 70])
-    steps, _ = ru.trace_mixed(reqs, seed=3)
-    outs = []
-    for native in (True, False):
-        runner = _runner(tiny_model_dirs["b"], "b", dtype, ru.peak_tokens(steps) // 8)
-        runner.model.use_native = native
-        assert (runner.model.native() is not None)
-        outs.append(ru.run_in_process(runner, steps))
-    assert outs[0].keys() == outs[1].keys()
-    for k in outs[0]:
-        assert np.array_equal(outs[0][k], outs[1][k]), k
-    rc.check_against_plain(tiny_model_dirs["b"], "b", reqs, steps, outs[0], dtype, label="native")
+@pytest.mark.parametrize("name", ["a", "b"])
+@pytest.mark.parametrize("family", FAMILIES)
+def test_trace_run_program_families(tiny_model_dirs, tmp_path, name, family, dtype):
+    """Every family through bin/trace_run with its default page size, the pool made for exactly --max-tokens."""
+    reqs = rc.requests_for(name, seed=2, lengths=rc.LENGTHS[name][:4] + [2, 64])
+    steps = rc.families(reqs, seed=2)[family]
+    skip = set()
+    if family == "mixed":
+        # a step in which nothing is wanted writes no file
+        for e in steps[0]["entries"]:
+            e["want"] = []
+            skip |= {(e["id"], p) for p in range(len(e["tokens"]))}
+    out = ru.run_trace_run(tiny_model_dirs[name], dtype, steps, str(tmp_path / "out"), ru.peak_tokens(steps))
+    if family == "mixed":
+        assert 0 not in out
+    rc.check_against_plain(tiny_model_dirs[name], name, reqs, steps, out, dtype, skip=skip, label="program " + family)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", ["small2", "xl2"])
+@pytest.mark.parametrize("family", ["decode_tail", "mixed"])
+def test_trace_run_program_at_real_layer_sizes(real_model_dirs, tmp_path, name, family, dtype):
+    reqs = rc.requests_for(name, seed=4, lengths=[15, 17, 130, 300])
+    steps = rc.families(reqs, seed=4, large=True)[family]
+    skip = rc.thin(steps)
+    out = ru.run_trace_run(real_model_dirs[name], dtype, steps, str(tmp_path / "out"), ru.peak_tokens(steps))
+    rc.check_against_plain(real_model_dirs[name], name, reqs, steps, out, dtype, skip=skip, label="program " + family)
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
@@ -113,17 +126,50 @@ def test_first_tokens_and_long_decoding(tiny_model_dirs, dtype):
     rc.check_against_plain(tiny_model_dirs[name], name, reqs, steps, out, dtype)
 
 
+# A context far beyond GPT-2's own: n_positions is a free key of config.json. Narrow (two heads of 64), so
+# that the plain implementation's 4,700 x 4,700 scores stay cheap.
+LONG = dict(architectures=["GPT2LMHeadModel"], model_type="gpt2", n_layer=2, n_embd=128, n_head=2, n_inner=256,
+            vocab_size=300, n_positions=8192, layer_norm_epsilon=1e-5, activation_function="gelu_new",
+            eos_token_id=299, bos_token_id=299)
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("name", ["a", "b"])
-def test_trace_run_program(tiny_model_dirs, tmp_path, name, dtype):
-    """bin/trace_run with its default page size, pool made for exactly --max-tokens."""
-    reqs = rc.requests_for(name, seed=2, lengths=rc.LENGTHS[name][:4] + [2, 64])
-    steps, _ = ru.trace_mixed(reqs, seed=2)
-    # a step in which nothing is wanted writes no file
-    skip = set()
-    for e in steps[0]["entries"]:
-        e["want"] = []
-        skip |= {(e["id"], p) for p in range(len(e["tokens"]))}
-    out = ru.run_trace_run(tiny_model_dirs[name], dtype, steps, str(tmp_path / "out"), ru.peak_tokens(steps))
-    assert 0 not in out
-    rc.check_against_plain(tiny_model_dirs[name], name, reqs, steps, out, dtype, skip=skip)
+def test_long_context_decode_splits_keys_over_the_chip(tmp_path, dtype):
+    """One request of 4,732 tokens: 4,700 in one step, the last 32 one by one, beside a short request that
+    decodes with it; before it a request that ends, so that the long one writes pages that were used. With
+    so few (token, head) pairs and so many keys the decode kernel splits every pair's keys over at least
+    eight workgroups and a second kernel merges their states: read back from the ops, not taken on faith.
+    Block tables have 296 entries."""
+    from mini_llm_amd import write_random_model
+    from mini_llm_amd.kernels import ops
+    d = write_random_model(LONG, str(tmp_path / "long"), seed=11)
+    cfg, w = plain_gpt2.read_model(d)
+    reqs = ru.random_requests(LONG["vocab_size"], [4732, 40, 70], seed=21)
+    long_, short, first = reqs["r0"], reqs["r1"], reqs["r2"]
+    steps = [{"step": 0, "entries": [{"id": "first", "tokens": first, "want": [len(first) - 1]}], "end": ["first"]},
+             {"step": 1, "entries": [{"id": "long", "tokens": long_[:4700], "want": [0, 1, 2047, 4095, 4096, 4699]},
+                                     {"id": "short", "tokens": short[:8], "want": [7]}], "end": []}]
+    for i in range(32):
+        steps.append({"step": 2 + i, "entries": [{"id": "short", "tokens": [short[8 + i]], "want": [0]},
+                                                  {"id": "long", "tokens": [long_[4700 + i]], "want": [0]}],
+                      "end": ["long", "short"] if i == 31 else []})
+    n_pages = ru.peak_tokens(steps) // 16
+    from mini_llm_amd import Runner
+    runner = Runner(model_dir=d, dtype=dtype, page_size=16, n_pages=n_pages, max_num_seqs=4)
+    runner.poison_cache()
+    ops.reset_seen()
+    out = ru.run_in_process(runner, steps)
+    assert ops.seen("max_decode_splits") >= 8 and ops.seen("merge_kernel_launches") >= 32 * LONG["n_layer"]
+    got = ru.collect(steps, out, LONG["vocab_size"])
+    tol = dict(max_abs=1e-5, mean_abs=2e-6) if dtype == "float32" else dict(max_abs=2e-2, mean_abs=4e-3)
+    worst = 0.0
+    for rid, toks in (("long", long_), ("short", short), ("first", first)):
+        ref = plain_gpt2.forward_logits(cfg, w, list(toks)).numpy()
+        assert got[rid], rid
+        for pos, row in got[rid].items():
+            assert np.isfinite(row).all(), (rid, pos)
+            diff = np.abs(row.astype(np.float64) - ref[pos])
+            worst = max(worst, diff.max())
+            assert diff.max() <= tol["max_abs"] and diff.mean() <= tol["mean_abs"], (rid, pos, diff.max(), diff.mean())
+    print(f"worst difference from plain at 4,732 tokens [{dtype}]: {worst:.3e} (allowed {tol['max_abs']:.1e})")
+    _all_pages_back(runner, n_pages)

@@ -196,126 +196,3 @@ def test_eos_and_abort_free_everything():
     assert s.state(3) == "failed"
     produced, _ = drive(s, eos_after={2: 3})
     assert s.generated(2) == 4 and cm.free_pages() == 64 and cm.n_requests() == 0 and not s.has_work()
-
-
-# ---- the engine above it, on the CPU reference ops -------------------------------------------
-
-@pytest.fixture()
-def cpu_ops(monkeypatch):
-    plain_ops.install(monkeypatch)
-
-
-def _engine(model_dir, **opt):
-    from mini_llm_amd import Engine, EngineOptions, load_model
-    return Engine(load_model(model_dir, "float32", "cpu"), EngineOptions(**opt))
-
-
-def test_generation_is_the_same_alone_and_under_page_pressure(cpu_ops, tiny_model_dirs):
-    from mini_llm_amd import SamplingParams
-    g = torch.Generator().manual_seed(4)
-    prompts = [torch.randint(0, 1000, (n,), generator=g).tolist() for n in (1, 9, 40, 100)]
-    params = [SamplingParams(temperature=0.8, seed=i, max_new_tokens=24, ignore_eos=True) for i in range(4)]
-    alone = []
-    for p, sp in zip(prompts, params):
-        e = _engine(tiny_model_dirs["b"], kv_block_size=8, total_kv_blocks=64, max_batch_num=4)
-        alone.append(e.generate([p], sp)[0])
-    assert all(len(o) == 24 for o in alone) and len({tuple(o) for o in alone}) == 4
-    roomy = _engine(tiny_model_dirs["b"], kv_block_size=8, total_kv_blocks=64, max_batch_num=4,
-                    max_tokens_per_step=32, prefill_chunk=16)
-    assert roomy.generate(prompts, params) == alone
-    # 26 pages: the four requests need 4+5+8+16 = 33 at the end, so some are deferred or recomputed
-    tight = _engine(tiny_model_dirs["b"], kv_block_size=8, total_kv_blocks=26, max_batch_num=4,
-                    max_tokens_per_step=32, prefill_chunk=16)
-    assert tight.generate(prompts, params) == alone
-    st = tight.stats()
-    assert st["deferred_prefills"] + st["deferred_decodes"] + st["preemptions"] > 0
-    assert st["free_pages"] == 26 and tight.runner.manager.check() == ""
-
-
-def test_greedy_generation_matches_plain_and_stops_at_eos(cpu_ops, tiny_model_dirs):
-    import plain_gpt2
-    from mini_llm_amd import SamplingParams
-    cfg, w = plain_gpt2.read_model(tiny_model_dirs["a"])
-    g = torch.Generator().manual_seed(1)
-    prompts = [torch.randint(0, 511, (n,), generator=g).tolist() for n in (5, 17, 33)]
-    e = _engine(tiny_model_dirs["a"], kv_block_size=4, total_kv_blocks=40, max_batch_num=4)
-    outs = e.generate(prompts, SamplingParams(max_new_tokens=16, ignore_eos=True))
-    for p, o in zip(prompts, outs):
-        assert o == plain_gpt2.greedy_generate(cfg, w, p, 16)
-    # declare the first generated token to be EOS: generation ends there
-    e2 = _engine(tiny_model_dirs["a"], kv_block_size=4, total_kv_blocks=40, max_batch_num=4)
-    e2.eos_token_id = outs[0][0]
-    assert e2.generate([prompts[0]], SamplingParams(max_new_tokens=16)) == [[outs[0][0]]]
-    assert e2.generate([prompts[0]], SamplingParams(max_new_tokens=3, ignore_eos=True)) == [outs[0][:3]]
-
-
-def test_overlapped_decode_gives_the_same_tokens(cpu_ops, tiny_model_dirs):
-    """Decode steps launched before the previous step's tokens are read (tokens fed on the
-    device) produce what step-by-step decoding produces, also when pages run out on the way."""
-    from mini_llm_amd import SamplingParams
-    g = torch.Generator().manual_seed(11)
-    prompts = [torch.randint(0, 1000, (n,), generator=g).tolist() for n in (3, 20, 41, 64)]
-    params = [SamplingParams(temperature=0.7 if i % 2 else 0.0, seed=10 + i, max_new_tokens=12 + 5 * i,
-                             ignore_eos=True) for i in range(4)]
-    for pages in (64, 24):
-        outs = []
-        for overlap in (False, True):
-            e = _engine(tiny_model_dirs["b"], kv_block_size=8, total_kv_blocks=pages, max_batch_num=4,
-                        max_tokens_per_step=32, prefill_chunk=16, overlap_decode=overlap)
-            outs.append(e.generate(prompts, params))
-            assert e.stats()["free_pages"] == pages and e.runner.manager.check() == ""
-        assert outs[0] == outs[1]
-        assert [len(o) for o in outs[0]] == [12, 17, 22, 27]
-
-
-def test_end_of_sequence_seen_one_step_late(cpu_ops, tiny_model_dirs):
-    """A decoded token that is the end of sequence is read only after the next step has been
-    launched: the request still ends with that token, the extra step's token is dropped and every
-    page comes back, while the other requests go on undisturbed."""
-    from mini_llm_amd import SamplingParams
-    g = torch.Generator().manual_seed(5)
-    prompts = [torch.randint(0, 511, (n,), generator=g).tolist() for n in (7, 19, 30)]
-    free = _engine(tiny_model_dirs["a"], kv_block_size=4, total_kv_blocks=60, max_batch_num=4)
-    sp = [SamplingParams(temperature=1.5, seed=3 + i, max_new_tokens=14, ignore_eos=True) for i in range(3)]
-    full = free.generate(prompts, sp)
-    # a token that request 0 decodes (not its first, which the prompt step samples), where it first occurs
-    j = next(j for j in range(2, 14) if full[0][j] not in full[0][:j])
-    eos = full[0][j]
-    expect = [o[:o.index(eos) + 1] if eos in o else o for o in full]
-    assert len(expect[0]) == j + 1
-    for overlap in (True, False):
-        e = _engine(tiny_model_dirs["a"], kv_block_size=4, total_kv_blocks=60, max_batch_num=4,
-                    overlap_decode=overlap)
-        e.eos_token_id = eos
-        stop = [SamplingParams(temperature=1.5, seed=3 + i, max_new_tokens=14) for i in range(3)]
-        assert e.generate(prompts, stop) == expect
-        assert e.stats()["free_pages"] == 60 and e.runner.manager.check() == ""
-        assert not e.has_unfinished()
-
-
-def test_outputs_of_steps_arrive_in_order_and_abort_in_flight(cpu_ops, tiny_model_dirs):
-    from mini_llm_amd import SamplingParams
-    e = _engine(tiny_model_dirs["a"], kv_block_size=4, total_kv_blocks=60, max_batch_num=4)
-    a = e.add_request([5, 6, 7, 8], SamplingParams(max_new_tokens=6, ignore_eos=True))
-    b = e.add_request([9, 10, 11], SamplingParams(max_new_tokens=9, ignore_eos=True))
-    seen = {a: [], b: []}
-    steps = 0
-    while e.has_unfinished():
-        for out in e.step():
-            seen[out.request_id].append((out.token, out.finished))
-        steps += 1
-        if steps == 4:
-            b_out = e.abort(b)       # b has a token in flight; it is dropped
-    assert len(seen[a]) == 6 and [f for _, f in seen[a]] == [False] * 5 + [True]
-    ref = _engine(tiny_model_dirs["a"], kv_block_size=4, total_kv_blocks=60, max_batch_num=4)
-    whole = ref.generate([[5, 6, 7, 8], [9, 10, 11]], SamplingParams(max_new_tokens=9, ignore_eos=True))
-    assert [t for t, _ in seen[a]] == whole[0][:6]
-    assert 0 < len(seen[b]) < 9 and [t for t, _ in seen[b]] == b_out == whole[1][:len(b_out)]
-    assert e.stats()["free_pages"] == 60 and e.runner.manager.check() == ""
-    # nothing of a finished or aborted request stays behind, and its id can be used again
-    assert e.requests == {} and e.scheduler.n_known() == 0
-    again = e.add_request([5, 6, 7, 8], SamplingParams(max_new_tokens=6, ignore_eos=True), request_id=a)
-    toks = []
-    while e.has_unfinished():
-        toks += [o.token for o in e.step() if o.request_id == again]
-    assert toks == whole[0][:6]
