@@ -90,7 +90,7 @@ def prefill_run(model_dir, dtype, cfg, n_req=2, n_tok=1024, reps=5):
     from mini_llm_amd import Runner, StepEntry
     runner = Runner(model_dir=model_dir, dtype=dtype, page_size=16, n_pages=n_req * n_tok // 16 + 8, max_num_seqs=n_req)
     g = torch.Generator().manual_seed(3)
-    toks = [torch.randint(0, cfg["vocab_size"], (n_tok,), generator=g).tolist() for _ in range(n_req)]
+    toks = [torch.randint(0, cfg["vocab_size"], (n_tok,), generator=g).to(torch.int32).numpy() for _ in range(n_req)]
     times = []
     for rep in range(reps + 2):
         entries = [StepEntry(i, toks[i], [n_tok - 1]) for i in range(n_req)]

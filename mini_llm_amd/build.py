@@ -255,6 +255,32 @@ def build_all(verbose: bool = True, jobs: int = 4) -> None:
         _loaded.clear()
 
 
+_runtime_shared = False
+
+
+def _share_hip_runtime_with_torch() -> None:
+    """One HIP runtime per process. PyTorch-ROCm bundles a copy of the HIP runtime and loads it by another
+    file name than the system's, so a process that loads the system's copy first (through these libraries)
+    and imports torch afterwards ends up with two runtimes, and the second finds no GPU. If torch is
+    installed and not imported yet, its copy is therefore loaded first, by path, without importing torch:
+    these libraries then bind to it (it carries the system copy's name), as they do when torch came first."""
+    global _runtime_shared
+    if _runtime_shared or "torch" in sys.modules:
+        _runtime_shared = True
+        return
+    _runtime_shared = True
+    try:
+        import importlib.util
+        spec = importlib.util.find_spec("torch")
+        if spec is None or not spec.submodule_search_locations:
+            return
+        path = os.path.join(list(spec.submodule_search_locations)[0], "lib", "libamdhip64.so")
+        if os.path.isfile(path):
+            ctypes.CDLL(path, mode=ctypes.RTLD_GLOBAL)
+    except (OSError, ImportError, ValueError):
+        pass          # no torch, or a torch without a bundled runtime: the system's copy is the only one
+
+
 def load_library(name: str) -> ctypes.CDLL:
     """Loads a library, building it first if it is missing or out of date."""
     with _lock:
@@ -263,6 +289,8 @@ def load_library(name: str) -> ctypes.CDLL:
             return lib
         if not is_current(name):
             build_library(name)
+        if LIBRARIES[name]["kind"] != "cxx":
+            _share_hip_runtime_with_torch()
         lib = ctypes.CDLL(lib_path(name))
         _loaded[name] = lib
         return lib

@@ -22,7 +22,7 @@ from ..config import as_config
 @dataclass
 class StepEntry:
     request_id: int
-    tokens: Sequence[int]               # the request's next tokens
+    tokens: Sequence[int]               # the request's next tokens (a list, or an int32 array: no conversion then)
     want: Sequence[int] = field(default_factory=list)     # indices into ``tokens`` whose logits are wanted
 
 
@@ -61,7 +61,8 @@ class Runner:
         entry's ``want``, or None if nothing is wanted."""
         ids = np.asarray([e.request_id for e in entries], dtype=np.int64)
         n_tok = np.asarray([len(e.tokens) for e in entries], dtype=np.int32)
-        toks = np.asarray([t for e in entries for t in e.tokens], dtype=np.int32)
+        toks = np.concatenate([np.asarray(e.tokens, dtype=np.int32).reshape(-1) for e in entries]) if entries \
+            else np.empty(0, dtype=np.int32)
         n_want = np.asarray([len(e.want) for e in entries], dtype=np.int32)
         want = np.asarray([w for e in entries for w in e.want], dtype=np.int32)
         rows = int(n_want.sum())
