@@ -74,13 +74,15 @@ int mllm_set_tuning(const char* name, int a, int b) {
     });
 }
 // What the ops chose since the last "reset_seen": "max_decode_splits" (most workgroups a (token, head) pair's keys
-// were split over), "merge_kernel_launches", "prefill_tile_launches", "generic_attention_launches". -1: unknown name.
+// were split over), "merge_kernel_launches", "prefill_tile_launches" (the bfloat16 matrix-core kernel), "tiled_f32_launches" (the 32-bit one),
+// "generic_attention_launches". -1: unknown name.
 long long mllm_get_seen(const char* name) {
     const Tuning::Seen& s = tuning().seen;
     const std::string n(name);
     if (n == "max_decode_splits") return s.max_decode_splits;
     if (n == "merge_kernel_launches") return s.merge_kernel_launches;
     if (n == "prefill_tile_launches") return s.prefill_tile_launches;
+    if (n == "tiled_f32_launches") return s.tiled_f32_launches;
     if (n == "generic_attention_launches") return s.generic_attention_launches;
     return -1;
 }

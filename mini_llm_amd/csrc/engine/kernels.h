@@ -40,6 +40,10 @@ int mllm_paged_attention_generic(const void* q, int q_stride, int q_col, const v
                                  const int* token_seq, const int* positions, int n_tokens, int n_heads,
                                  int n_kv_heads, int head_dim, int page_size, float scale, int window,
                                  void* out, int out_stride, int dtype, hipStream_t stream);
+int mllm_paged_attention_tiled(const void* q, int q_stride, int q_col, const void* k_pages, const void* v_pages,
+                               int kv_dim, const int* block_tables, int max_blocks, const int* cu_q, const int* ctx_len,
+                               int n_seqs, int n_tiles_upper, int n_heads, int n_kv_heads, int head_dim, int page_size,
+                               float scale, int window, void* out, int out_stride, int dtype, hipStream_t stream);
 int mllm_decode_attention(const void* q, int q_stride, int q_col, const void* k_pages, const void* v_pages,
                           int kv_dim, const int* block_tables, int max_blocks, const int* token_seq,
                           const int* positions, int n_q, int n_heads, int n_kv_heads, int head_dim,

@@ -395,28 +395,55 @@ bool paged_attention(const AttentionArgs& a, AttentionSplits* splits, hipStream_
             slots = a.slots;
         }
     }
-    const bool tiles_ok = a.q.dtype == BF16 && (a.head_dim == 32 || a.head_dim == 64 || a.head_dim == 128) && a.max_q_len > 1 &&
-                          a.cu_q != nullptr && a.ctx_len != nullptr && pow2(a.page_size) && a.page_size >= a.head_dim / 16 &&
-                          a.max_blocks <= 2048;
+    // Prompt portions go to a kernel that shares key tiles among 64 queries: the bfloat16 matrix-core kernel at
+    // its head and page sizes, otherwise the kernel that works in true 32-bit at any head size (multiples of 16)
+    // and page size. What neither takes, and single tokens at sizes the decode kernel refuses, go to the
+    // one-wavefront-per-query kernel.
+    const bool have_tiles = a.max_q_len > 1 && a.cu_q != nullptr && a.ctx_len != nullptr;
+    const bool tiles_ok = have_tiles && a.q.dtype == BF16 && (a.head_dim == 32 || a.head_dim == 64 || a.head_dim == 128) &&
+                          pow2(a.page_size) && a.page_size >= a.head_dim / 16 && a.max_blocks <= 2048;
+    const bool tiled_ok = have_tiles && !tiles_ok && a.head_dim % 16 == 0 && (kv_dim * esz) % 16 == 0 && (a.out.stride * esz) % 8 == 0 &&
+                          aligned(a.out.data, 16) && aligned(a.k_pages.data, 16) && aligned(a.v_pages.data, 16);
     if (tiles_ok && (!aligned(a.out.data, 16) || (a.out.stride * esz) % 8)) fail("paged_attention: output rows must be 8-byte aligned");
-    if (tiles_ok && a.n_single > 0 && a.n_single < a.n_seqs && single_ok) {
+    auto portions = [&](int first_seq) {
+        const int B = a.n_seqs - first_seq, tiles = (T - first_seq) / 64 + B;      // (the leading sequences bring one row each)
+        if (tiles_ok) {
+            tuning().seen.prefill_tile_launches += 1;
+            check(mllm_prefill_attention_bf16(a.q.data, static_cast<int>(a.q.stride), a.q_col, a.k_pages.data, a.v_pages.data, kv_dim,
+                                              a.block_tables + static_cast<size_t>(first_seq) * a.max_blocks, a.max_blocks,
+                                              a.cu_q + first_seq, a.ctx_len + first_seq, B, tiles, a.n_heads, a.n_kv_heads,
+                                              a.head_dim, a.page_size, a.scale, a.window, a.out.data,
+                                              static_cast<int>(a.out.stride), stream), "prefill_attention");
+        } else {
+            tuning().seen.tiled_f32_launches += 1;
+            check(mllm_paged_attention_tiled(a.q.data, static_cast<int>(a.q.stride), a.q_col, a.k_pages.data, a.v_pages.data, kv_dim,
+                                             a.block_tables + static_cast<size_t>(first_seq) * a.max_blocks, a.max_blocks,
+                                             a.cu_q + first_seq, a.ctx_len + first_seq, B, tiles, a.n_heads, a.n_kv_heads,
+                                             a.head_dim, a.page_size, a.scale, a.window, a.out.data,
+                                             static_cast<int>(a.out.stride), a.q.dtype, stream), "paged_attention (tiles)");
+        }
+    };
+    if ((tiles_ok || tiled_ok) && a.n_single > 0 && a.n_single < a.n_seqs) {
         // A mixed step: the leading single tokens, then the portions, two launches over disjoint rows
         // (every row's keys and values are in the pages by now). Row numbers in cu_q are absolute, so q
         // and out are passed whole and the per-sequence arrays from the first portion on.
-        AttentionArgs d = a;
-        d.q = a.q.row_range(0, a.n_single);
-        d.out = a.out.row_range(0, a.n_single);
-        d.n_seqs = a.n_single;
-        d.max_q_len = 1;
-        d.append = 0;
-        d.may_split = 0;
-        paged_attention(d, nullptr, stream);
-        const int B = a.n_seqs - a.n_single;
-        check(mllm_prefill_attention_bf16(a.q.data, static_cast<int>(a.q.stride), a.q_col, a.k_pages.data, a.v_pages.data, kv_dim,
-                                          a.block_tables + static_cast<size_t>(a.n_single) * a.max_blocks, a.max_blocks,
-                                          a.cu_q + a.n_single, a.ctx_len + a.n_single, B, (T - a.n_single) / 64 + B, a.n_heads,
-                                          a.n_kv_heads, a.head_dim, a.page_size, a.scale, a.window, a.out.data,
-                                          static_cast<int>(a.out.stride), stream), "prefill_attention");
+        if (single_ok) {
+            AttentionArgs d = a;
+            d.q = a.q.row_range(0, a.n_single);
+            d.out = a.out.row_range(0, a.n_single);
+            d.n_seqs = a.n_single;
+            d.max_q_len = 1;
+            d.append = 0;
+            d.may_split = 0;
+            paged_attention(d, nullptr, stream);
+        } else {
+            tuning().seen.generic_attention_launches += 1;
+            check(mllm_paged_attention_generic(a.q.data, static_cast<int>(a.q.stride), a.q_col, a.k_pages.data, a.v_pages.data, kv_dim,
+                                               a.block_tables, a.max_blocks, a.token_seq, a.positions, a.n_single, a.n_heads,
+                                               a.n_kv_heads, a.head_dim, a.page_size, a.scale, a.window, a.out.data,
+                                               static_cast<int>(a.out.stride), a.q.dtype, stream), "paged_attention");
+        }
+        portions(a.n_single);
         return false;
     }
     if (decode) {
@@ -452,13 +479,8 @@ bool paged_attention(const AttentionArgs& a, AttentionSplits* splits, hipStream_
         }
         return false;
     }
-    if (tiles_ok) {
-        // prompt portions: tiles of 64 queries on the matrix cores
-        tuning().seen.prefill_tile_launches += 1;
-        check(mllm_prefill_attention_bf16(a.q.data, static_cast<int>(a.q.stride), a.q_col, a.k_pages.data, a.v_pages.data, kv_dim,
-                                          a.block_tables, a.max_blocks, a.cu_q, a.ctx_len, a.n_seqs, T / 64 + a.n_seqs, a.n_heads,
-                                          a.n_kv_heads, a.head_dim, a.page_size, a.scale, a.window, a.out.data,
-                                          static_cast<int>(a.out.stride), stream), "prefill_attention");
+    if (tiles_ok || tiled_ok) {
+        portions(0);
         return false;
     }
     tuning().seen.generic_attention_launches += 1;

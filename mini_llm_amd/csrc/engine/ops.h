@@ -109,7 +109,7 @@ struct Tuning {
     // what the ops chose since the last reset (tests read it back instead of trusting the thresholds)
     struct Seen {
         int max_decode_splits = 0;                    // most workgroups a (token, head) pair's keys were split over
-        long long merge_kernel_launches = 0, prefill_tile_launches = 0, generic_attention_launches = 0;
+        long long merge_kernel_launches = 0, prefill_tile_launches = 0, tiled_f32_launches = 0, generic_attention_launches = 0;
     } seen;
 };
 Tuning& tuning();

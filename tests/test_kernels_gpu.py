@@ -560,6 +560,33 @@ def test_paged_attention_prefill_tiles(ops, H, Hkv, dh, page, window):
     assert (out - ref).abs().max() <= _tol(torch.bfloat16, 2)
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("H,Hkv,dh,page", [(12, 12, 64, 16), (4, 4, 16, 4), (6, 2, 48, 12), (5, 1, 80, 8), (3, 3, 128, 20),
+                                           (2, 1, 256, 64), (7, 7, 32, 1)])
+@pytest.mark.parametrize("window", [0, 1, 50, 64, 200])
+def test_paged_attention_tiles_in_true_32_bit(ops, dtype, H, Hkv, dh, page, window):
+    """The prompt-portion kernel that shares key tiles among 64 queries at any head size (steps of 16 up to 256),
+    any page size (12 and 20 are no powers of two; 1), grouped heads, float32 and bfloat16 storage: query tiles that
+    are full, partial and a single row; portions that start mid-sequence and mid-page; windows that cut inside a key
+    tile. Read back from the ops: this kernel ran wherever the bfloat16 matrix-core kernel does not take the sizes."""
+    g = torch.Generator().manual_seed(H + dh + window + page)
+    seqs = [(0, 64), (0, 150), (37, 2), (100, 129), (511, 1), (64, 64), (5, 63)]
+    ops.reset_seen()
+    out, ref = _attention_case(ops, dtype, H, Hkv, dh, page, seqs, window, g)
+    mfma_bf16 = dtype == torch.bfloat16 and dh in (32, 64, 128) and page & (page - 1) == 0 and page >= dh // 16
+    assert ops.seen("tiled_f32_launches") == (0 if mfma_bf16 else 1) and ops.seen("generic_attention_launches") == 0
+    assert torch.isfinite(out).all()
+    assert (out - ref).abs().max() <= _tol(dtype, 2)
+    # single tokens in front of the portions (a mixed step): at page sizes the decode kernel refuses they go to the
+    # one-wavefront-per-query kernel, the portions to the tiles
+    seqs = [(300, 1), (0, 1), (77, 1), (0, 70), (130, 3), (64, 129)]
+    ops.reset_seen()
+    out, ref = _attention_case(ops, dtype, H, Hkv, dh, page, seqs, window, g, n_single=3)
+    assert ops.seen("tiled_f32_launches") == (0 if mfma_bf16 else 1)
+    assert torch.isfinite(out).all()
+    assert (out - ref).abs().max() <= _tol(dtype, 2)
+
+
 @pytest.mark.parametrize("T", [1, 8, 16])
 @pytest.mark.parametrize("H,Hkv,dh,page,N", [(12, 12, 64, 16, 768), (25, 25, 64, 16, 1600), (3, 3, 32, 8, 96),
                                              (4, 2, 128, 16, 200), (16, 16, 64, 16, 1024)])
