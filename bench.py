@@ -109,7 +109,8 @@ def prefill_run(model_dir, dtype, cfg, n_req=2, n_tok=1024, reps=5):
     return T / dt, dt, flops
 
 
-def serving_run(model_dir, dtype, cfg, n_req, prompt_lo, prompt_hi, new_tokens, max_batch, chunk, pages, seed):
+def serving_run(model_dir, dtype, cfg, n_req, prompt_lo, prompt_hi, new_tokens, max_batch, chunk, pages, seed,
+                preempt_for_decode=True):
     """Continuous batching from a full queue: n_req requests with prompt lengths uniform in
     [prompt_lo, prompt_hi] and new_tokens generated each, prompts fed in portions of `chunk`, at most
     max_batch requests a step, `pages` pages of 16 tokens in the pool. Returns a dictionary of
@@ -117,7 +118,8 @@ def serving_run(model_dir, dtype, cfg, n_req, prompt_lo, prompt_hi, new_tokens, 
     import torch
     from mini_llm_amd import Engine, EngineOptions, SamplingParams
     options = EngineOptions(kv_block_size=16, total_kv_blocks=pages, max_batch_num=max_batch,
-                            max_tokens_per_step=max(2048, max_batch + chunk), prefill_chunk=chunk)
+                            max_tokens_per_step=max(2048, max_batch + chunk), prefill_chunk=chunk,
+                            preempt_for_decode=preempt_for_decode)
     engine = Engine.from_pretrained(model_dir, dtype=dtype, options=options)
     engine.generate([[0]] * min(max_batch, 8), SamplingParams(max_new_tokens=2, ignore_eos=True))     # loads the kernels
     base = engine.stats()
@@ -176,7 +178,8 @@ def serving_main(args, cfg, model_dir):
     else:
         n_req, lo, hi, new, max_batch, chunk = 256, 512, 512, 512, 64, 512
         pages = int(0.6 * max_batch * ((hi + new + 15) // 16))
-    r = serving_run(model_dir, args.dtype, cfg, n_req, lo, hi, new, max_batch, chunk, pages, seed=7)
+    r = serving_run(model_dir, args.dtype, cfg, n_req, lo, hi, new, max_batch, chunk, pages, seed=7,
+                    preempt_for_decode=not args.defer_decodes)
     c = r["counters"]
     rec = {"metric": f"generated tok/s, {args.workload} workload ({args.size} sizes)",
            "value": round(r["generated"] / r["seconds"], 1), "unit": "tok/s", "n_gpus": 1,
@@ -187,7 +190,8 @@ def serving_main(args, cfg, model_dir):
                    "; a few two-token requests before the clock starts",
            "config": {"model": args.size + "-sizes", "n_layer": cfg["n_layer"], "n_layer_full": SIZES[args.size][0],
                       "requests": n_req, "prompt_min": lo, "prompt_max": hi, "new_tokens": new,
-                      "max_batch_num": max_batch, "prefill_chunk": chunk, "kv_blocks": pages, "kv_block_size": 16},
+                      "max_batch_num": max_batch, "prefill_chunk": chunk, "kv_blocks": pages, "kv_block_size": 16,
+                      "preempt_for_decode": not args.defer_decodes},
            # what the run did (the configuration above holds sizes only)
            "serving": {"prompt_tokens": r["prompt_tokens"], "generated_tokens": r["generated"],
                        "total_tok_per_s": round((r["generated"] + r["prompt_tokens"]) / r["seconds"], 1),
@@ -217,6 +221,9 @@ def main():
     ap.add_argument("--prefill-only", action="store_true", help="measure only the prefill step (profiling)")
     ap.add_argument("--prefill-requests", type=int, default=2, help="with --prefill-only: prompts in the step")
     ap.add_argument("--prefill-tokens", type=int, default=1024, help="with --prefill-only: tokens of each prompt")
+    ap.add_argument("--defer-decodes", action="store_true",
+                    help="serving workloads: a decode that gets no page waits on its pages (the reference's manner) "
+                         "instead of preempting a younger request at once")
     ap.add_argument("--plugin", action="append", default=[],
                     help="a shared library that registers further architectures (with --config)")
     ap.add_argument("--config", help="a config.json to measure in place of the GPT-2 sizes (any registered architecture; "

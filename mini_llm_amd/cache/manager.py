@@ -48,7 +48,7 @@ def _rt():
         "mllm_cache_free_state_slots": (i, [vp]),
         "mllm_cache_n_requests": (i, [vp]),
         "mllm_cache_check": (i, [vp, ctypes.c_char_p, i]),
-        "mllm_sched_create": (vp, [vp, i, i, i, i]),
+        "mllm_sched_create": (vp, [vp, i, i, i, i, i]),
         "mllm_sched_destroy": (None, [vp]),
         "mllm_sched_add": (i, [vp, i64, i, i]),
         "mllm_sched_schedule": (i, [vp, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, i]),

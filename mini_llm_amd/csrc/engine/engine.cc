@@ -425,6 +425,7 @@ Engine::Engine(std::unique_ptr<LoadedModel> model, const EngineOptions& o) : mod
     so.max_tokens_per_step = o.max_tokens_per_step;
     so.prefill_chunk = o.prefill_chunk;
     so.max_positions = model_->max_positions;
+    so.preempt_for_decode = o.preempt_for_decode;
     scheduler_.reset(new Scheduler(&runner_->manager(), so));
 }
 

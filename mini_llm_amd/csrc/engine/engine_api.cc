@@ -349,23 +349,23 @@ void mllm_runner_synchronize(void* runner) { guarded([&] { static_cast<ModelRunn
 
 // -- the engine (engine.h) ---------------------------------------------------------------------------
 // options: kv_block_size, total_kv_blocks, max_batch_num, max_tokens_per_step, prefill_chunk, overlap (0/1),
-// kv_memory_fraction in millionths (0: total_kv_blocks counts)
+// kv_memory_fraction in millionths (0: total_kv_blocks counts), preempt_for_decode (0/1)
 static EngineOptions options_of(const int* o) {
     EngineOptions e;
     e.kv_block_size = o[0]; e.total_kv_blocks = o[1]; e.max_batch_num = o[2]; e.max_tokens_per_step = o[3];
-    e.prefill_chunk = o[4]; e.overlap = o[5] != 0; e.kv_memory_fraction = o[6] * 1e-6;
+    e.prefill_chunk = o[4]; e.overlap = o[5] != 0; e.kv_memory_fraction = o[6] * 1e-6; e.preempt_for_decode = o[7] != 0;
     return e;
 }
-void* mllm_engine_from_pretrained(const char* model_dir, int dtype, const int* options7) {
+void* mllm_engine_from_pretrained(const char* model_dir, int dtype, const int* options8) {
     Engine* e = nullptr;
-    guarded([&] { e = Engine::from_pretrained(model_dir, dtype, options_of(options7)).release(); });
+    guarded([&] { e = Engine::from_pretrained(model_dir, dtype, options_of(options8)).release(); });
     return e;
 }
 // config_json: the text of a config.json. The weights are the values a written folder holds (matrices rounded
 // to bfloat16 whatever `dtype` computes in), so this and make-model + from_pretrained give the same model.
-void* mllm_engine_from_random(const char* config_json, unsigned long long seed, int dtype, const int* options7) {
+void* mllm_engine_from_random(const char* config_json, unsigned long long seed, int dtype, const int* options8) {
     Engine* e = nullptr;
-    guarded([&] { e = Engine::from_random(Json::parse(config_json), seed, dtype, options_of(options7)).release(); });
+    guarded([&] { e = Engine::from_random(Json::parse(config_json), seed, dtype, options_of(options8)).release(); });
     return e;
 }
 void mllm_engine_destroy(void* e) { delete static_cast<Engine*>(e); }

@@ -125,7 +125,7 @@ int cmd_generate(int argc, char** argv) {
                               {"model", "preset", "weights-seed", "dtype", "device", "prompt-ids", "prompts-file", "max-new-tokens",
                                "temperature", "seed", "kv-block-size", "total-kv-blocks", "kv-memory-fraction", "max-batch-num",
                                "max-tokens-per-step", "prefill-chunk", "plugin"},
-                              {"ignore-eos", "stream", "stats", "no-overlap"});
+                              {"ignore-eos", "stream", "stats", "no-overlap", "defer-decodes"});
     load_plugins(a);
     if (a.has("model") == a.has("preset")) { std::fprintf(stderr, "give either --model DIR or --preset NAME\n"); return 1; }
     const std::string device = a.get("device", "cuda:0");
@@ -153,6 +153,7 @@ int cmd_generate(int argc, char** argv) {
     o.max_tokens_per_step = static_cast<int>(a.integer("max-tokens-per-step", 2048));
     o.prefill_chunk = static_cast<int>(a.integer("prefill-chunk", 512));
     o.overlap = !a.has("no-overlap");
+    o.preempt_for_decode = !a.has("defer-decodes");
     const int dtype = dtype_of(a.get("dtype", "bfloat16"));
     std::unique_ptr<Engine> engine;
     if (a.has("preset"))
@@ -312,7 +313,7 @@ int main(int argc, char** argv) {
                  "  generate   --model DIR | --preset NAME [--weights-seed S]  [--dtype bfloat16|float32] [--prompt-ids \"1 2 3\"]...\n"
                  "             [--prompts-file F] [--max-new-tokens 8] [--temperature 0] [--seed 0] [--ignore-eos] [--stream] [--stats]\n"
                  "             [--kv-block-size 16] [--total-kv-blocks 4096 | --kv-memory-fraction F] [--max-batch-num 16] [--max-tokens-per-step 2048]\n"
-                 "             [--prefill-chunk 512]\n"
+                 "             [--prefill-chunk 512] [--defer-decodes] [--no-overlap]\n"
                  "  every command: [--plugin LIB.so]...  shared libraries that register further parts and architectures\n"
                  "             (also: the paths in the environment variable MINI_LLM_PLUGINS, separated by colons)\n"
                  "  make-model (--preset NAME | --config FILE) --seed S --out DIR [--weights-dtype bfloat16|float32]\n"

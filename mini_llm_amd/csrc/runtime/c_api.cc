@@ -64,12 +64,13 @@ int mllm_cache_check(void* c, char* out, int cap) {
 }
 
 void* mllm_sched_create(void* cache, int max_num_seqs, int max_tokens_per_step, int prefill_chunk,
-                        int max_positions) {
+                        int max_positions, int preempt_for_decode) {
     SchedulerOptions o;
     o.max_num_seqs = max_num_seqs;
     o.max_tokens_per_step = max_tokens_per_step;
     o.prefill_chunk = prefill_chunk;
     o.max_positions = max_positions;
+    o.preempt_for_decode = preempt_for_decode != 0;
     return new Scheduler(static_cast<CacheManager*>(cache), o);
 }
 void mllm_sched_destroy(void* s) { delete static_cast<Scheduler*>(s); }

@@ -68,13 +68,17 @@ const std::vector<PlanEntry>& Scheduler::schedule() {
 
         // 1. One token for every request that is decoding.
         std::deque<int64_t> ready;
-        for (int64_t id : decode_) {
+        const std::vector<int64_t> decoding(decode_.begin(), decode_.end());      // (a preemption below edits decode_)
+        for (int64_t id : decoding) {
             Req& r = reqs_.at(id);
+            if (r.state != RequestState::DecodeReady) continue;      // preempted a moment ago for an older one
             if (n_seqs >= opt_.max_num_seqs || budget < 1) {
                 ready.push_back(id);          // waits for the next step, loses nothing
                 continue;
             }
-            if (try_plan_tokens(r, 1, &budget, &n_seqs)) {
+            bool planned = try_plan_tokens(r, 1, &budget, &n_seqs);
+            while (!planned && opt_.preempt_for_decode && preempt_younger_than(r)) planned = try_plan_tokens(r, 1, &budget, &n_seqs);
+            if (planned) {
                 ready.push_back(id);
             } else {
                 r.state = RequestState::DeferredDecode;
@@ -83,7 +87,9 @@ const std::vector<PlanEntry>& Scheduler::schedule() {
                 events_.push_back({id, EventKind::Deferred});
             }
         }
-        decode_.swap(ready);
+        decode_.clear();
+        for (int64_t id : ready)
+            if (reqs_.at(id).state == RequestState::DecodeReady) decode_.push_back(id);      // (not those preempted meanwhile)
 
         // 2. The next portion of every prompt that is under way, first come first served.
         bool blocked = false;
@@ -152,15 +158,38 @@ bool Scheduler::resolve_stall() {
         Req& r = reqs_.at(id);
         if (!victim || r.admit_seq > victim->admit_seq) victim = &r;
     }
-    remove_from(prefill_, victim->id);
-    remove_from(decode_, victim->id);
-    remove_from(deferred_decode_, victim->id);
-    cache_->free_request(victim->id);
-    victim->computed = 0;
-    victim->state = RequestState::DeferredPrefill;
-    deferred_prefill_.push_front(victim->id);
+    preempt(*victim);
+    return true;
+}
+
+void Scheduler::preempt(Req& victim) {
+    remove_from(prefill_, victim.id);
+    remove_from(decode_, victim.id);
+    remove_from(deferred_decode_, victim.id);
+    cache_->free_request(victim.id);
+    victim.computed = 0;
+    victim.state = RequestState::DeferredPrefill;
+    deferred_prefill_.push_front(victim.id);
     ++counters_.preemptions;
-    events_.push_back({victim->id, EventKind::Preempted});
+    events_.push_back({victim.id, EventKind::Preempted});
+}
+
+// Frees the pages of the most recently admitted running request that was admitted after `r` and has no
+// tokens in the plan under way. False if there is none.
+bool Scheduler::preempt_younger_than(const Req& r) {
+    Req* victim = nullptr;
+    auto consider = [&](int64_t id) {
+        Req& c = reqs_.at(id);
+        if (c.id == r.id || c.admit_seq <= r.admit_seq) return;
+        for (const PlanEntry& e : plan_)
+            if (e.id == id) return;
+        if (!victim || c.admit_seq > victim->admit_seq) victim = &c;
+    };
+    for (int64_t id : prefill_) consider(id);
+    for (int64_t id : decode_) consider(id);
+    for (int64_t id : deferred_decode_) consider(id);
+    if (victim == nullptr) return false;
+    preempt(*victim);
     return true;
 }
 

@@ -39,6 +39,12 @@ struct SchedulerOptions {
     int max_tokens_per_step = 2048; // token budget of one step
     int prefill_chunk = 512;        // longest prompt portion
     int max_positions = 0;          // 0: unbounded; else no token at a position >= this
+    // What happens to a decode that gets no page. false (the reference's manner): it is deferred and keeps its
+    // pages until somebody finishes; only when nobody can step is a request preempted. true: the most recently
+    // admitted running request that is younger than it and not in this step's plan is preempted at once (its
+    // pages freed, recomputed later), so that pages do not idle under requests that wait; if there is none
+    // (it is the youngest itself), it is deferred.
+    bool preempt_for_decode = false;
 };
 
 struct PlanEntry {
@@ -105,6 +111,8 @@ private:
     bool try_plan_tokens(Req& r, int n, int* budget, int* n_seqs);
     bool admit(Req& r);
     bool resolve_stall();
+    void preempt(Req& victim);
+    bool preempt_younger_than(const Req& r);
     void finish(Req& r, RequestState final_state);
     void remove_from(std::deque<int64_t>& q, int64_t id);
 

@@ -35,6 +35,8 @@ class EngineOptions:
     max_tokens_per_step: int = 2048     # token budget of one step
     prefill_chunk: int = 512            # longest prompt portion
     overlap_decode: bool = True         # launch a step before the previous one's tokens are read
+    preempt_for_decode: bool = True     # a decode that gets no page preempts a younger request at once; False: it
+                                        # waits on its pages until somebody finishes (the reference's manner)
 
 
 @dataclass
@@ -88,8 +90,9 @@ class Engine:
 
     @staticmethod
     def _pack(o: EngineOptions):
-        return (ctypes.c_int * 7)(o.kv_block_size, o.total_kv_blocks, o.max_batch_num, o.max_tokens_per_step,
-                                  o.prefill_chunk, 1 if o.overlap_decode else 0, int(round(o.kv_memory_fraction * 1e6)))
+        return (ctypes.c_int * 8)(o.kv_block_size, o.total_kv_blocks, o.max_batch_num, o.max_tokens_per_step,
+                                  o.prefill_chunk, 1 if o.overlap_decode else 0, int(round(o.kv_memory_fraction * 1e6)),
+                                  1 if o.preempt_for_decode else 0)
 
     @classmethod
     def from_pretrained(cls, model_dir: str, dtype: str = "bfloat16", options: Optional[EngineOptions] = None, **kw):

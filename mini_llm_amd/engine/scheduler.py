@@ -29,12 +29,13 @@ class PlanEntry:
 
 class Scheduler:
     def __init__(self, cache: CacheManager, max_num_seqs: int, max_tokens_per_step: int,
-                 prefill_chunk: int, max_positions: Optional[int]):
+                 prefill_chunk: int, max_positions: Optional[int], preempt_for_decode: bool = False):
         self._lib = _rt()
         self._cache = cache       # keeps the native cache manager alive
         self.max_num_seqs = int(max_num_seqs)
         self._h = self._lib.mllm_sched_create(cache.handle, int(max_num_seqs), int(max_tokens_per_step),
-                                              int(prefill_chunk), int(max_positions or 0))
+                                              int(prefill_chunk), int(max_positions or 0),
+                                              1 if preempt_for_decode else 0)
         cap = self.max_num_seqs
         self._ids = np.empty(cap, dtype=np.int64)
         self._start = np.empty(cap, dtype=np.int32)

@@ -42,6 +42,7 @@ static void one_run(unsigned seed) {
     opt.prefill_chunk = pick(2, 24);
     opt.max_tokens_per_step = opt.prefill_chunk + opt.max_num_seqs + pick(0, 16);
     opt.max_positions = max_pos;
+    opt.preempt_for_decode = pick(0, 1) == 1;      // both policies for a decode that gets no page
     Scheduler sched(&cache, opt);
     int64_t next_id = 1;
     std::map<int64_t, int> want_new;            // live requests -> tokens still to come

@@ -28,9 +28,9 @@ def drive(s, eos_after=None, max_iters=10000):
     return produced, plans
 
 
-def make(n_pages=64, page=4, seqs=4, budget=32, chunk=16, max_pos=128, slots=None):
+def make(n_pages=64, page=4, seqs=4, budget=32, chunk=16, max_pos=128, slots=None, preempt_for_decode=False):
     cm = CacheManager([GroupSpec(page, n_pages)], slots or seqs)
-    return cm, Scheduler(cm, seqs, budget, chunk, max_pos)
+    return cm, Scheduler(cm, seqs, budget, chunk, max_pos, preempt_for_decode)
 
 
 def test_single_request_lifecycle():
@@ -167,6 +167,44 @@ def test_out_of_pages_defers_decodes_then_preempts_the_latest():
     c = s.counters()
     assert c["preemptions"] >= 1 and c["deferred_decodes"] >= 1 and c["failures"] == 0
     assert cm.free_pages() == 4 and cm.n_requests() == 0
+
+
+def test_a_decode_without_a_page_preempts_a_younger_request_at_once():
+    """The engine's default policy: an older request never waits on its pages for a younger one. Three requests
+    of 7 + 8 tokens through 7 pages of 4: all are admitted (2 pages each); both request 1 and request 2 need a third
+    page at position 8 and one is free: request 1 takes it, and for request 2 the youngest, request 3, is preempted
+    in that same iteration (no deferral). Later request 2 is the youngest that runs: it then waits (there is nobody
+    younger to take pages from). Request 3 is recomputed once pages are free again, and everybody finishes."""
+    cm, s = make(n_pages=7, page=4, budget=32, chunk=16, preempt_for_decode=True)
+    for rid in (1, 2, 3):
+        s.add_request(rid, 7, 8)
+    events, produced, order = [], {}, []
+    for it in range(200):
+        plan = s.schedule()
+        for ev in s.pop_events():
+            events.append((it,) + ev)
+        if not plan:
+            break
+        s.commit()
+        for e in plan:
+            if e.want_last:
+                produced[e.request_id] = produced.get(e.request_id, 0) + 1
+                if s.on_token(e.request_id, False):
+                    order.append(e.request_id)
+        assert cm.check() == ""
+    kinds = [(rid, kind) for _, rid, kind in events]
+    assert events[0] == (2, 3, "preempted")            # in the iteration in which request 2 found no page
+    assert not any(rid == 1 for rid, _ in kinds)       # the oldest neither waits nor is preempted
+    assert (2, "preempted") not in kinds and all(it > 2 for it, rid, kind in events if (rid, kind) == (2, "deferred"))
+    assert produced == {1: 8, 2: 8, 3: 8} and order[:2] == [1, 2]
+    c = s.counters()
+    assert c["preemptions"] >= 1 and c["failures"] == 0 and cm.free_pages() == 7 and cm.n_requests() == 0
+    # the reference's manner on the same workload: the decode waits (is deferred) instead
+    cm2, s2 = make(n_pages=7, page=4, budget=32, chunk=16, preempt_for_decode=False)
+    for rid in (1, 2, 3):
+        s2.add_request(rid, 7, 8)
+    produced2, _ = drive(s2)
+    assert produced2 == {1: 8, 2: 8, 3: 8} and s2.counters()["deferred_decodes"] >= 1
 
 
 def test_a_request_larger_than_the_pool_fails_alone():
