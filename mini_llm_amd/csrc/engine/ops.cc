@@ -74,8 +74,11 @@ void* scratch(const char* name, size_t bytes, bool zero, hipStream_t stream) {
     hipError_t e = hipMalloc(&fresh, bytes);
     if (e != hipSuccess) fail("scratch '%s': hipMalloc of %zu bytes failed: %s", name, bytes, hipGetErrorString(e));
     if (zero) {
+        // (the fill runs on the null stream, which a non-blocking stream does not wait for: the device is
+        // synchronised so that no kernel on `stream` meets counters that are still being cleared)
         e = hipMemset(fresh, 0, bytes);
-        if (e != hipSuccess) fail("scratch '%s': hipMemset failed: %s", name, hipGetErrorString(e));
+        if (e == hipSuccess) e = hipDeviceSynchronize();
+        if (e != hipSuccess) fail("scratch '%s': clearing it failed: %s", name, hipGetErrorString(e));
     }
     if (b.ptr != nullptr) {
         // work queued with the old buffer may still run: wait for it, then free
