@@ -247,9 +247,14 @@ def main():
         # another architecture, served by the same engine: sizes from its own config.json
         with open(args.config) as f:
             cfg = json.load(f)
+        # (what the measurement itself needs to know: where token ids and positions end; keys the architecture does
+        # not read are ignored by it)
         cfg.setdefault("vocab_size", args.vocab or cfg.get("vocab", 0))
         cfg.setdefault("n_positions", args.positions)
-        cfg.setdefault("n_layer", args.layers)
+        if cfg["vocab_size"] < 1:
+            print("bench.py: --config names no vocab_size; give --vocab")
+            return 2
+        cfg.setdefault("n_layer", None)
         args.size = cfg.get("architectures", ["?"])[0]
         SIZES[args.size] = (cfg["n_layer"], 0, 0, 0)
     if "n_embd" not in cfg:

@@ -141,6 +141,7 @@ public:
         return h;
     }
     size_t workspace_bytes(int rows) const override { return static_cast<size_t>(rows) * size_ * dtype_size(dtype) + 256; }
+    void add_cost(StepCost& c) const override { if (mode_ == 1) c.weight_bytes += 4.0 * size_; }
 
 private:
     int size_ = 0, mode_ = 0;

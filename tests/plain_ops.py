@@ -1,8 +1,7 @@
 """Plain torch references of the engine's device ops, one per kernel, same signatures.
 
-Two uses: GPU tests compare each kernel with its reference here; CPU tests put these
-in place of ``mini_llm_amd.kernels.ops`` to exercise the step function, the cache and
-the scheduler without a GPU (``install()``). They are not part of the product path.
+GPU tests compare each kernel with its reference here, and CPU tests compare these with the
+plain C++ twins (csrc/ref/ref_ops.cc). They are not part of the product path.
 Accumulation is done in float64 (``PRECISE``) so that the reference is the more
 accurate side of every comparison.
 """
@@ -56,17 +55,8 @@ def reset_state(state, slots, starts):
             state[int(slots[b])] = 0
 
 
-ROW_BY_ROW = False     # True (set by install()): every output row is a matrix-vector product of its own, so that a
-                       # row's result cannot depend on how many rows share the call (the library may block a
-                       # product differently for different row counts)
-
-
 def linear(a, w, bias, out, epilogue="store", kv_scatter=None):
-    if ROW_BY_ROW:
-        w64 = w.to(PRECISE)
-        y = torch.stack([w64 @ a[i].to(PRECISE) for i in range(a.shape[0])])
-    else:
-        y = a.to(PRECISE) @ w.to(PRECISE).T
+    y = a.to(PRECISE) @ w.to(PRECISE).T
     if bias is not None:
         y = y + bias.to(PRECISE)
     if epilogue == "gelu_tanh":
@@ -142,16 +132,3 @@ def sample(logits, temperature, u, out):
         idx = int(torch.searchsorted(c, torch.tensor(target, dtype=PRECISE), right=True))
         out[i] = min(idx, row.numel() - 1)
     return out
-
-
-_NAMES = ("embed", "select_tokens", "reset_state", "layernorm", "linear", "ln_linear", "kv_append", "paged_attention", "argmax", "sample")
-
-
-def install(monkeypatch):
-    """Replaces the engine's device ops with the references above (CPU tests only)."""
-    from mini_llm_amd.kernels import ops
-    g = globals()
-    for name in _NAMES:
-        monkeypatch.setattr(ops, name, g[name])
-    import sys
-    monkeypatch.setattr(sys.modules[__name__], "ROW_BY_ROW", True)

@@ -1,5 +1,5 @@
-"""The replay comparisons shared by the CPU tests (engine over plain ops) and the GPU tests
-(engine over the HIP kernels): every schedule family against the plain implementation."""
+"""The replay comparisons of the GPU tests: request sets, the four schedule families, tolerances, and the
+check of an engine's logits against the plain implementation's, position by position."""
 from __future__ import annotations
 
 from typing import Dict
@@ -11,7 +11,7 @@ import plain_gpt2
 import replay_util as ru
 from conftest import CONFIGS
 
-# request lengths: BASELINE's prompt lengths plus generated tokens, and page-edge cases
+# request lengths: the tiny workloads' prompt lengths (5, 17, 33 and 1, 9, 40, 100) plus their generated tokens, and page-edge cases
 LENGTHS = {"a": [5 + 16, 17 + 16, 33 + 16, 1, 3, 4, 5, 64, 128], "b": [1 + 24, 9 + 24, 40 + 24, 100 + 24, 7, 8, 9, 256]}
 
 # at GPT-2 small / XL layer sizes: the reference's own page-edge lengths (5, 15, 16, 17 around its 16-token

@@ -283,6 +283,26 @@ def test_toy_architecture_is_served_by_the_engine_and_the_command_line(tmp_path)
     assert r.returncode == 0, r.stderr
 
 
+def test_toy_architecture_through_the_benchmark(tmp_path):
+    """bench.py measures the plugin's architecture through the same engine and the same accounting (bytes and flops
+    from the model's parts, whatever they are)."""
+    path = toy.load()
+    (tmp_path / "toy.json").write_text(json.dumps(TOY_CFG))
+    r = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--plugin", path, "--config", str(tmp_path / "toy.json"),
+                        "--positions", "256", "--prompt-len", "64", "--batch", "4", "--steps", "16", "--warmup", "4"],
+                       capture_output=True, text=True, timeout=600)
+    assert r.returncode == 0, r.stderr
+    rec = json.loads(r.stdout.strip().splitlines()[-1])
+    assert rec["config"]["model"] == "ToyLM-sizes" and rec["config"]["vocab_size"] == 203 and rec["value"] > 0
+    # weights a step reads: the attention layer's, the stateful layer's, the final norm's and the tied head's (bf16
+    # matrices, fp32 vectors); the cache: one layer of one key/value head of 16
+    D, dh = 48, 16
+    matrices = (D + 2 * dh) * D + D * D + 2 * D * D * 2 + 203 * D
+    vectors = 2 * D + D + 2 * D + D + 2 * D
+    live = 4 * rec["config"]["mean_context"] * 2 * dh * 2
+    assert rec["roofline"]["bytes_per_step"] == int(2 * matrices + 4 * vectors + live)
+
+
 def test_toy_architecture_through_trace_replay(tmp_path):
     """bin/trace_run replays a trace on the plugin's architecture (the plugin named by the environment)."""
     import replay_util as ru

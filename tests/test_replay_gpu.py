@@ -161,15 +161,18 @@ def test_long_context_decode_splits_keys_over_the_chip(tmp_path, dtype):
     out = ru.run_in_process(runner, steps)
     assert ops.seen("max_decode_splits") >= 8 and ops.seen("merge_kernel_launches") >= 32 * LONG["n_layer"]
     got = ru.collect(steps, out, LONG["vocab_size"])
-    tol = dict(max_abs=1e-5, mean_abs=2e-6) if dtype == "float32" else dict(max_abs=2e-2, mean_abs=4e-3)
-    worst = 0.0
+    # about three times the worst seen (float32: max 2.6e-7 of a row, mean 4e-8; bfloat16: 2.2e-3 and 4e-4; the
+    # logits' own standard deviation is about 0.2)
+    tol = dict(max_abs=1e-6, mean_abs=1.5e-7) if dtype == "float32" else dict(max_abs=7e-3, mean_abs=1.5e-3)
+    worst = worst_mean = 0.0
     for rid, toks in (("long", long_), ("short", short), ("first", first)):
         ref = plain_gpt2.forward_logits(cfg, w, list(toks)).numpy()
         assert got[rid], rid
         for pos, row in got[rid].items():
             assert np.isfinite(row).all(), (rid, pos)
             diff = np.abs(row.astype(np.float64) - ref[pos])
-            worst = max(worst, diff.max())
+            worst, worst_mean = max(worst, diff.max()), max(worst_mean, diff.mean())
             assert diff.max() <= tol["max_abs"] and diff.mean() <= tol["mean_abs"], (rid, pos, diff.max(), diff.mean())
-    print(f"worst difference from plain at 4,732 tokens [{dtype}]: {worst:.3e} (allowed {tol['max_abs']:.1e})")
+    print(f"worst difference from plain at 4,732 tokens [{dtype}]: max {worst:.3e}, mean {worst_mean:.3e} "
+          f"(allowed {tol['max_abs']:.1e}, {tol['mean_abs']:.1e})")
     _all_pages_back(runner, n_pages)
