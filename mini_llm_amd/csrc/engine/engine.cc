@@ -300,7 +300,13 @@ StepView ModelRunner::build(const std::vector<StepEntry>& entries, const std::ve
     if (d_uniforms) *d_uniforms = reinterpret_cast<const float*>(d + o_u);
     if (any_feed) {
         if (tok_out_ == nullptr) throw EngineError("no earlier launch has sampled a token");
-        select_tokens(dev_ints_ + offs[0], d + o_src, tok_out_, T, tok_out_cap_, stream_);
+        if (model_.model.embedding->resolves_fed_tokens()) {
+            sv.fed.src = d + o_src;
+            sv.fed.prev = tok_out_;
+            sv.fed.n_prev = tok_out_cap_;
+        } else {
+            select_tokens(dev_ints_ + offs[0], d + o_src, tok_out_, T, tok_out_cap_, stream_);
+        }
     }
     return sv;
 }

@@ -89,8 +89,12 @@ long long mllm_get_seen(const char* name) {
 
 // -- the ops (see ops.h) -----------------------------------------------------------------------------
 int mllm_op_embed(const int* ids, const int* positions, const Tensor2* wte, const Tensor2* wpe, const Tensor2* out,
-                  hipStream_t s) {
-    return guarded([&] { embed(ids, positions, *wte, wpe, *out, s); });
+                  const int* src, const int* prev, int n_prev, hipStream_t s) {
+    return guarded([&] {
+        FedTokens fed;
+        fed.src = src; fed.prev = prev; fed.n_prev = n_prev;
+        embed(ids, positions, *wte, wpe, *out, s, src ? &fed : nullptr);
+    });
 }
 int mllm_op_select_tokens(int* ids, const int* src, const int* prev, int n, int n_prev, hipStream_t s) {
     return guarded([&] { select_tokens(ids, src, prev, n, n_prev, s); });

@@ -10,7 +10,7 @@ extern "C" {
 
 // elementwise.hip
 int mllm_embed(const int* ids, const int* pos, const void* wte, const void* wpe, float* x, int T, int D,
-               int dtype, hipStream_t stream);
+               int dtype, const int* src, const int* prev, int n_prev, hipStream_t stream);
 int mllm_select_tokens(int* ids, const int* src, const int* prev, int n, int n_prev, hipStream_t stream);
 int mllm_reset_state(void* state, size_t slot_bytes, int n_slots, const int* slots, const int* starts, int B,
                      hipStream_t stream);

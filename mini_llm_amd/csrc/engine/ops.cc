@@ -151,7 +151,7 @@ Tuning& tuning() {
 // elementwise
 // ---------------------------------------------------------------------------------------------
 void embed(const int* ids, const int* positions, const Tensor2& wte, const Tensor2* wpe, const Tensor2& out,
-           hipStream_t stream) {
+           hipStream_t stream, const FedTokens* fed) {
     need_dtype(wte, "wte");
     const int T = static_cast<int>(out.rows), D = static_cast<int>(wte.cols);
     if (!wte.contiguous()) fail("embed: wte must be contiguous");
@@ -163,8 +163,10 @@ void embed(const int* ids, const int* positions, const Tensor2& wte, const Tenso
             fail("embed: wpe must be contiguous [P, %d] in wte's dtype", D);
         table = wpe->data;
     }
+    const bool feeds = fed != nullptr && fed->src != nullptr;
+    if (feeds && (fed->prev == nullptr || fed->n_prev < 1)) fail("embed: fed tokens need the earlier step's sampled tokens");
     check(mllm_embed(ids, table ? positions : nullptr, wte.data, table, static_cast<float*>(out.data), T, D, wte.dtype,
-                     stream), "embed");
+                     feeds ? fed->src : nullptr, feeds ? fed->prev : nullptr, feeds ? fed->n_prev : 0, stream), "embed");
 }
 
 void select_tokens(int* ids, const int* src, const int* prev, int n, int n_prev, hipStream_t stream) {

@@ -114,9 +114,17 @@ struct Tuning {
 };
 Tuning& tuning();
 
+// Token ids that an earlier step sampled on the device and the host has not read yet: where src[t] >= 0,
+// token t's id is prev[src[t]] (n_prev entries) and not ids[t].
+struct FedTokens {
+    const int* src = nullptr;
+    const int* prev = nullptr;
+    int n_prev = 0;
+};
+
 // -- the ops -----------------------------------------------------------------------------------------
 void embed(const int* ids, const int* positions, const Tensor2& wte, const Tensor2* wpe, const Tensor2& out,
-           hipStream_t stream);
+           hipStream_t stream, const FedTokens* fed = nullptr);
 void select_tokens(int* ids, const int* src, const int* prev, int n, int n_prev, hipStream_t stream);
 void reset_state(void* state, size_t slot_bytes, int n_slots, const int* slots, const int* starts, int n_seqs,
                  hipStream_t stream);

@@ -366,8 +366,9 @@ public:
     int vocab_size() const override { return static_cast<int>(table_.rows); }
     int hidden_size() const override { return static_cast<int>(table_.cols); }
     void forward(const StepView& step, const PositionEncoding* position, const Tensor2& x, hipStream_t s) const override {
-        embed(step.token_ids, step.positions, table_, position ? position->table() : nullptr, x, s);
+        embed(step.token_ids, step.positions, table_, position ? position->table() : nullptr, x, s, &step.fed);
     }
+    bool resolves_fed_tokens() const override { return true; }
 
 private:
     Tensor2 table_;         // [V, D]

@@ -84,6 +84,8 @@ private:
 struct StepView {
     int n_tokens = 0, n_seqs = 0, n_logits = 0, max_q_len = 0, max_ctx_len = 0, n_single = 0;
     const int* token_ids = nullptr;    // [T]
+    FedTokens fed;                     // tokens to take on the device from the step before (only if the model's embedding
+                                       // says that it resolves them; otherwise token_ids holds every id already)
     const int* positions = nullptr;    // [T]
     const int* token_seq = nullptr;    // [T]
     const int* cu_q = nullptr;         // [B+1]
@@ -181,6 +183,9 @@ public:
     virtual int vocab_size() const = 0;
     virtual int hidden_size() const = 0;
     virtual void forward(const StepView& step, const PositionEncoding* position, const Tensor2& x, hipStream_t s) const = 0;
+    // true: forward() takes `step.fed` into account itself (one kernel fewer in a decode step); false: the runner
+    // writes the fed ids into token_ids with a kernel of its own before the step
+    virtual bool resolves_fed_tokens() const { return false; }
     virtual void add_cost(StepCost&) const {}
 };
 

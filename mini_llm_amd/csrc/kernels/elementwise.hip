@@ -6,13 +6,21 @@
 // ---------------------------------------------------------------------------
 // Token + position embedding: x[t,:] = wte[ids[t],:] + wpe[pos[t],:]   (fp32 out)
 // /root/reference/src/kernels/embedding.cu:23-43. wpe may be null (no learned positions).
+// With `src` (optional): where src[t] >= 0, token t's id is prev[src[t]], a token that an earlier step
+// sampled on the device and the host has not read yet; ids[t] is not read then.
 // ---------------------------------------------------------------------------
 template <typename T>
 __global__ void embed_kernel(const int* __restrict__ ids, const int* __restrict__ pos,
                              const T* __restrict__ wte, const T* __restrict__ wpe,
-                             float* __restrict__ x, int D) {
+                             float* __restrict__ x, int D, const int* __restrict__ src,
+                             const int* __restrict__ prev, int n_prev) {
     const int t = blockIdx.x;
-    const T* te = wte + static_cast<size_t>(ids[t]) * D;
+    int id = ids[t];
+    if (src != nullptr) {
+        const int s = src[t];
+        if (s >= 0 && s < n_prev) id = prev[s];
+    }
+    const T* te = wte + static_cast<size_t>(id) * D;
     float* xr = x + static_cast<size_t>(t) * D;
     if (wpe != nullptr) {
         const T* pe = wpe + static_cast<size_t>(pos[t]) * D;
@@ -208,12 +216,12 @@ int mllm_reset_state(void* state, size_t slot_bytes, int n_slots, const int* slo
 }
 
 int mllm_embed(const int* ids, const int* pos, const void* wte, const void* wpe, float* x, int T, int D,
-               int dtype, hipStream_t stream) {
+               int dtype, const int* src, const int* prev, int n_prev, hipStream_t stream) {
     if (T <= 0) return 0;
     if (dtype == MLLM_F32)
-        embed_kernel<float><<<T, 256, 0, stream>>>(ids, pos, (const float*)wte, (const float*)wpe, x, D);
+        embed_kernel<float><<<T, 256, 0, stream>>>(ids, pos, (const float*)wte, (const float*)wpe, x, D, src, prev, n_prev);
     else
-        embed_kernel<bf16_t><<<T, 256, 0, stream>>>(ids, pos, (const bf16_t*)wte, (const bf16_t*)wpe, x, D);
+        embed_kernel<bf16_t><<<T, 256, 0, stream>>>(ids, pos, (const bf16_t*)wte, (const bf16_t*)wpe, x, D, src, prev, n_prev);
     MLLM_LAUNCH_CHECK();
     return 0;
 }

@@ -60,7 +60,7 @@ def engine_library():
     lib = native.lib()
     T2p, sz = ctypes.POINTER(Tensor2), ctypes.c_size_t
     sigs = {
-        "mllm_op_embed": (_i, [_vp, _vp, T2p, T2p, T2p, _vp]),
+        "mllm_op_embed": (_i, [_vp, _vp, T2p, T2p, T2p, _vp, _vp, _i, _vp]),
         "mllm_op_select_tokens": (_i, [_vp, _vp, _vp, _i, _i, _vp]),
         "mllm_op_reset_state": (_i, [_vp, sz, _i, _vp, _vp, _i, _vp]),
         "mllm_op_layernorm": (_i, [T2p, _vp, _vp, _f, T2p, _vp, _vp]),
@@ -199,10 +199,15 @@ def push_tuning() -> None:
 # -- the ops -----------------------------------------------------------------------------------------
 
 def embed(ids: torch.Tensor, positions: Optional[torch.Tensor], wte: torch.Tensor,
-          wpe: Optional[torch.Tensor], out: torch.Tensor) -> torch.Tensor:
+          wpe: Optional[torch.Tensor], out: torch.Tensor, src: Optional[torch.Tensor] = None,
+          prev: Optional[torch.Tensor] = None) -> torch.Tensor:
     """out[t,:] = wte[ids[t],:] + wpe[positions[t],:] in fp32. ids/positions must be in range
-    (the caller checks them on the host)."""
-    _gpu(ids, positions, wte, wpe, out)
+    (the caller checks them on the host). With ``src`` and ``prev``: where src[t] >= 0, token t's id is
+    prev[src[t]] (a token that an earlier step sampled on the device) instead of ids[t]."""
+    _gpu(ids, positions, wte, wpe, out, src, prev)
+    if src is not None:
+        _i32(src, "src", ids.numel())
+        _i32(prev, "prev")
     T = ids.numel()
     _i32(ids, "ids")
     if wpe is not None:
@@ -213,7 +218,8 @@ def embed(ids: torch.Tensor, positions: Optional[torch.Tensor], wte: torch.Tenso
         raise KernelError(f"out must be contiguous fp32 [{T}, {wte.shape[1]}]")
     _ok(engine_library().mllm_op_embed(_p(ids), _p(positions), ctypes.byref(t2(wte, "wte")),
                                        ctypes.byref(t2(wpe, "wpe")) if wpe is not None else None,
-                                       ctypes.byref(t2(out, "out")), _stream()))
+                                       ctypes.byref(t2(out, "out")), _p(src), _p(prev),
+                                       0 if prev is None else prev.numel(), _stream()))
     return out
 
 

@@ -14,7 +14,9 @@ import torch
 PRECISE = torch.float64
 
 
-def embed(ids, positions, wte, wpe, out):
+def embed(ids, positions, wte, wpe, out, src=None, prev=None):
+    if src is not None:
+        ids = torch.where((src >= 0) & (src < prev.numel()), prev[src.clamp(0, prev.numel() - 1).long()], ids)
     x = wte[ids.long()].to(PRECISE)
     if wpe is not None:
         x = x + wpe[positions.long()[: ids.numel()]].to(PRECISE)

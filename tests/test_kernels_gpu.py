@@ -88,6 +88,15 @@ def test_embed_reference_vector(ops, dtype):
     # without a position table
     ops.embed(ids.to(DEV), None, wte.to(DEV), None, out)
     assert torch.equal(out.cpu(), wte[ids.long()].float())
+    # tokens taken on the device from what an earlier step sampled: rows 1, 4 and 6 (a source beyond the
+    # sampled tokens is ignored, as by select_tokens)
+    src = torch.tensor([-1, 2, -1, -1, 0, 9, 1], dtype=torch.int32)
+    prev = torch.tensor([60, 61, 62], dtype=torch.int32)
+    ops.embed(ids.to(DEV), pos.to(DEV), wte.to(DEV), wpe.to(DEV), out, src=src.to(DEV), prev=prev.to(DEV))
+    fed = torch.tensor([3, 62, 7, 5, 60, 13, 61])
+    assert (out.cpu() - (wte[fed].float() + wpe[pos.long()].float())).abs().max() <= 1e-6
+    want = plain_ops.embed(ids, pos, wte, wpe, torch.empty(7, D, dtype=torch.float64), src=src, prev=prev)
+    assert (out.cpu().double() - want).abs().max() <= 1e-6
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
