@@ -165,6 +165,7 @@ ModelRunner::~ModelRunner() {
         if (host_tok_[i]) (void)hipHostFree(host_tok_[i]);
         if (host_tok_event_[i]) (void)hipEventDestroy(host_tok_event_[i]);
     }
+    if (host_logits_) (void)hipHostFree(host_logits_);
     for (void* p : {static_cast<void*>(dev_ints_), arena_, static_cast<void*>(logits_), static_cast<void*>(tok_out_)})
         if (p) (void)hipFree(p);
     if (stream_) {
@@ -326,7 +327,7 @@ float* ModelRunner::run(const StepView& step) {
     return logits;
 }
 
-std::vector<float> ModelRunner::step(const std::vector<StepEntry>& entries, bool manage_cache, int* n_rows) {
+const float* ModelRunner::step(const std::vector<StepEntry>& entries, bool manage_cache, int* n_rows) {
     CacheManager& mgr = manager();
     if (manage_cache) {
         std::vector<int64_t> fresh;
@@ -349,14 +350,19 @@ std::vector<float> ModelRunner::step(const std::vector<StepEntry>& entries, bool
     float* logits = run(sv);
     if (manage_cache)
         for (const StepEntry& e : entries) mgr.commit(e.request_id, mgr.length(e.request_id) + static_cast<int>(e.tokens.size()));
-    std::vector<float> host;
-    if (n_rows) *n_rows = sv.n_logits;
+    if (n_rows) *n_rows = logits != nullptr ? sv.n_logits : 0;
     if (logits != nullptr) {
-        host.resize(static_cast<size_t>(sv.n_logits) * model_.model.vocab_size());
-        HIP_OK(hipMemcpyAsync(host.data(), logits, host.size() * sizeof(float), hipMemcpyDeviceToHost, stream_));
+        const size_t bytes = static_cast<size_t>(sv.n_logits) * model_.model.vocab_size() * sizeof(float);
+        if (host_logits_bytes_ < bytes) {
+            if (host_logits_) HIP_OK(hipHostFree(host_logits_));
+            host_logits_ = nullptr;
+            host_logits_bytes_ = bytes + bytes / 4;
+            HIP_OK(hipHostMalloc(reinterpret_cast<void**>(&host_logits_), host_logits_bytes_, hipHostMallocDefault));
+        }
+        HIP_OK(hipMemcpyAsync(host_logits_, logits, bytes, hipMemcpyDeviceToHost, stream_));
     }
     HIP_OK(hipStreamSynchronize(stream_));
-    return host;
+    return logits != nullptr ? host_logits_ : nullptr;
 }
 
 int ModelRunner::launch(const std::vector<StepEntry>& entries, const std::vector<float>& temperatures,

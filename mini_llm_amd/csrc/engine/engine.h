@@ -118,9 +118,10 @@ public:
     const LoadedModel& model() const { return model_; }
 
     // Runs one batch and returns the fp32 logits [wanted, vocab] on the host, in the order of the entries
-    // and of each entry's `want` (empty if nothing is wanted). With manage_cache the runner registers new
-    // requests, takes their pages and commits the new lengths itself (replay, tests).
-    std::vector<float> step(const std::vector<StepEntry>& entries, bool manage_cache, int* n_rows);
+    // and of each entry's `want` (nullptr and 0 rows if nothing is wanted). The rows lie in a pinned buffer of
+    // the runner and stay valid until its next step. With manage_cache the runner registers new requests,
+    // takes their pages and commits the new lengths itself (replay, tests).
+    const float* step(const std::vector<StepEntry>& entries, bool manage_cache, int* n_rows);
     void end_request(int64_t id) { manager().free_request(id); }
 
     // Starts one step (pages reserved, lengths committed by the caller) and returns at once. One token is
@@ -166,6 +167,8 @@ private:
     size_t arena_bytes_ = 0;
     float* logits_ = nullptr;
     size_t logits_bytes_ = 0;
+    float* host_logits_ = nullptr;     // pinned: what step() returns
+    size_t host_logits_bytes_ = 0;
     int* tok_out_ = nullptr;           // sampled tokens of the last launched step
     int tok_out_cap_ = 0;
     int* host_tok_[2] = {nullptr, nullptr};

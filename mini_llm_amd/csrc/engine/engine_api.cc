@@ -296,8 +296,9 @@ int mllm_runner_step(void* runner, const long long* ids, const int* n_tokens, co
         }
         if (total > cap_rows) fail("%lld rows of logits are wanted, the buffer holds %lld", total, cap_rows);
         int n = 0;
-        const std::vector<float> host = static_cast<ModelRunner*>(runner)->step(entries, true, &n);
-        if (!host.empty()) std::memcpy(logits, host.data(), host.size() * sizeof(float));
+        ModelRunner* r = static_cast<ModelRunner*>(runner);
+        const float* host = r->step(entries, true, &n);
+        if (host != nullptr) std::memcpy(logits, host, static_cast<size_t>(n) * r->model().model.vocab_size() * sizeof(float));
         rows = n;
     });
     return rows;

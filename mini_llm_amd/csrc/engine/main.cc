@@ -273,10 +273,11 @@ int cmd_replay(int argc, char** argv) {
         }
         if (!entries.empty()) {
             int rows = 0;
-            const std::vector<float> logits = runner.step(entries, true, &rows);
+            const float* logits = runner.step(entries, true, &rows);
             if (rows > 0) {
                 std::ofstream f(out_dir + "/" + step + ".f32", std::ios::binary);
-                f.write(reinterpret_cast<const char*>(logits.data()), static_cast<std::streamsize>(logits.size() * sizeof(float)));
+                f.write(reinterpret_cast<const char*>(logits),
+                        static_cast<std::streamsize>(static_cast<size_t>(rows) * model->model.vocab_size() * sizeof(float)));
                 if (!f) throw EngineError("cannot write " + out_dir + "/" + step + ".f32");
             }
         }
