@@ -489,6 +489,34 @@ def test_two_engines_stepped_in_turn_do_not_share_scratch(dtype):
     assert alone[0] != alone[1]
 
 
+def test_engines_give_their_memory_back(tiny_model_dirs):
+    """An engine owns a stream, and the kernels' scratch memory belongs to that stream: closing the engine frees
+    both, so that engines made and dropped one after the other do not pile up device memory."""
+    from mini_llm_amd import Engine, EngineOptions, SamplingParams
+    from mini_llm_amd.kernels import ops
+    o = EngineOptions(kv_block_size=8, total_kv_blocks=64, max_batch_num=4)
+    sp = SamplingParams(max_new_tokens=4, ignore_eos=True)
+
+    def once():
+        e = Engine.from_pretrained(tiny_model_dirs["b"], dtype="bfloat16", options=o)
+        out = e.generate([[1, 2, 3, 4, 5]], sp)
+        held = ops.scratch_bytes()
+        e.close()
+        return out, held
+
+    first, held = once()
+    torch.cuda.synchronize()
+    base_scratch, (base_free, _) = ops.scratch_bytes(), torch.cuda.mem_get_info()
+    assert held > base_scratch                  # (the engine's stream held scratch of its own while it lived)
+    for _ in range(12):
+        out, _ = once()
+        assert out == first
+    torch.cuda.synchronize()
+    assert ops.scratch_bytes() == base_scratch
+    free, _ = torch.cuda.mem_get_info()
+    assert base_free - free < 8 << 20, (base_free, free)
+
+
 def test_stage_times_of_the_forward_pass(tiny_model_dirs):
     """MINI_LLM_STAGE_TIMES: one line per stage and step on standard error, in the reference's format
     (kind,batch_size,total_tokens,layer,stage,ms); the tokens on standard output are unchanged."""
