@@ -83,59 +83,74 @@ gemm_f32_kernel(const float* __restrict__ A, int lda, const float* __restrict__ 
 }
 
 // Few rows (decode): the product is bound by reading W once, and the tiled kernel above would
-// start N/64 workgroups for it. Here a wavefront owns one output column: its lanes walk the
-// column's weights in 16-byte steps (a wavefront's load is 1 KB of one row), the activations of
-// up to ROWS rows wait in LDS in chunks of F32R_KC floats, and a lane's partial sums (k ascending)
-// are added over the wavefront in a fixed order. More rows than ROWS take further passes over W.
+// start N/64 workgroups for it. Here a wavefront owns one output column (WAVES columns a workgroup):
+// its lanes walk the column's weights in 16-byte steps (a wavefront's load is 1 KB of one row), the
+// activations of up to ROWS rows wait in LDS in chunks of F32R_KC floats, and a lane's partial sums
+// (k ascending) are added over the wavefront in a fixed order. More rows than ROWS take further passes over W.
 // Needs K and the row strides in multiples of 4 floats and 16-byte aligned operands.
 #define F32R_KC 512      // 128 16-byte steps: two per lane
 
-template <int ROWS>
-__global__ void __launch_bounds__(256)
+template <int ROWS, int WAVES>
+__global__ void __launch_bounds__(64 * WAVES)
 gemm_f32_rows_kernel(const float* __restrict__ A, int lda, const float* __restrict__ W, int ldw,
                      const float* __restrict__ bias, void* __restrict__ C, int ldc, int M, int N, int K, int mode) {
     __shared__ __attribute__((aligned(16))) float a_s[ROWS][F32R_KC];
     const int tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid / 64), lane = tid % 64;
-    const int n = blockIdx.x * 4 + wave;
+    const int n = blockIdx.x * WAVES + wave;
     const float* wrow = W + static_cast<size_t>(min(n, N - 1)) * ldw;       // a surplus wavefront repeats the last column
+    constexpr int STAGED = (ROWS * (F32R_KC / 4) + 64 * WAVES - 1) / (64 * WAVES);   // 16-byte steps of a chunk a thread stages
     for (int m0 = 0; m0 < M; m0 += ROWS) {
         float acc[ROWS];
 #pragma unroll
         for (int r = 0; r < ROWS; ++r) acc[r] = 0.f;
+        // With a handful of wavefronts on a compute unit nothing hides a load's latency but the kernel itself:
+        // the weights and the activations of the next chunk are asked for before the chunk in LDS is used.
+        // A chunk is at most two 16-byte steps per lane (the second from a clamped address; its product is
+        // left out where it is past the chunk).
+        const int q0 = lane, q1 = lane + 64;
+        float4 w0, w1, v[STAGED];
+        auto fetch = [&](int kc0) {
+            const int quads = min(F32R_KC, K - kc0) / 4;
+            w0 = *reinterpret_cast<const float4*>(wrow + kc0 + 4 * min(q0, quads - 1));
+            w1 = *reinterpret_cast<const float4*>(wrow + kc0 + 4 * min(q1, quads - 1));
+#pragma unroll
+            for (int u = 0; u < STAGED; ++u) {
+                const int idx = tid + 64 * WAVES * u, r = idx / quads, q = idx % quads;
+                v[u] = make_float4(0.f, 0.f, 0.f, 0.f);
+                if (idx < ROWS * quads && m0 + r < M)
+                    v[u] = *reinterpret_cast<const float4*>(A + static_cast<size_t>(m0 + r) * lda + kc0 + 4 * q);
+            }
+        };
+        fetch(0);
         for (int kc0 = 0; kc0 < K; kc0 += F32R_KC) {
             const int quads = min(F32R_KC, K - kc0) / 4;
-            // a chunk is at most two 16-byte steps per lane: both loads are issued here, ahead of the
-            // staging of the activations (the second from a clamped address; its product is left out
-            // where it is past the chunk)
-            const int q0 = lane, q1 = lane + 64;
-            const float4 w0 = *reinterpret_cast<const float4*>(wrow + kc0 + 4 * min(q0, quads - 1));
-            const float4 w1 = *reinterpret_cast<const float4*>(wrow + kc0 + 4 * min(q1, quads - 1));
+            const float4 c0 = w0, c1 = w1;
             __syncthreads();          // the chunk before has been read
-            for (int idx = tid; idx < ROWS * quads; idx += 256) {
-                const int r = idx / quads, q = idx % quads;
-                float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
-                if (m0 + r < M) v = *reinterpret_cast<const float4*>(A + static_cast<size_t>(m0 + r) * lda + kc0 + 4 * q);
-                *reinterpret_cast<float4*>(&a_s[r][4 * q]) = v;
+#pragma unroll
+            for (int u = 0; u < STAGED; ++u) {
+                const int idx = tid + 64 * WAVES * u, r = idx / quads, q = idx % quads;
+                if (idx < ROWS * quads) *reinterpret_cast<float4*>(&a_s[r][4 * q]) = v[u];
             }
+            if (kc0 + F32R_KC < K) fetch(kc0 + F32R_KC);
             __syncthreads();
             if (q0 < quads) {
 #pragma unroll
                 for (int r = 0; r < ROWS; ++r) {
                     const float4 a4 = *reinterpret_cast<const float4*>(&a_s[r][4 * q0]);
-                    acc[r] = fmaf(a4.x, w0.x, acc[r]);
-                    acc[r] = fmaf(a4.y, w0.y, acc[r]);
-                    acc[r] = fmaf(a4.z, w0.z, acc[r]);
-                    acc[r] = fmaf(a4.w, w0.w, acc[r]);
+                    acc[r] = fmaf(a4.x, c0.x, acc[r]);
+                    acc[r] = fmaf(a4.y, c0.y, acc[r]);
+                    acc[r] = fmaf(a4.z, c0.z, acc[r]);
+                    acc[r] = fmaf(a4.w, c0.w, acc[r]);
                 }
             }
             if (q1 < quads) {
 #pragma unroll
                 for (int r = 0; r < ROWS; ++r) {
                     const float4 a4 = *reinterpret_cast<const float4*>(&a_s[r][4 * q1]);
-                    acc[r] = fmaf(a4.x, w1.x, acc[r]);
-                    acc[r] = fmaf(a4.y, w1.y, acc[r]);
-                    acc[r] = fmaf(a4.z, w1.z, acc[r]);
-                    acc[r] = fmaf(a4.w, w1.w, acc[r]);
+                    acc[r] = fmaf(a4.x, c1.x, acc[r]);
+                    acc[r] = fmaf(a4.y, c1.y, acc[r]);
+                    acc[r] = fmaf(a4.z, c1.z, acc[r]);
+                    acc[r] = fmaf(a4.w, c1.w, acc[r]);
                 }
             }
         }
@@ -158,9 +173,18 @@ int mllm_gemm_f32(const float* A, int lda, const float* W, int ldw, const float*
     const bool quads = K % 4 == 0 && lda % 4 == 0 && ldw % 4 == 0 &&
                        ((reinterpret_cast<uintptr_t>(A) | reinterpret_cast<uintptr_t>(W)) & 15) == 0;
     if (M <= 64 && quads && K > 0) {
-        const dim3 rows_grid((N + 3) / 4);
-        if (M <= 8) gemm_f32_rows_kernel<8><<<rows_grid, 256, 0, stream>>>(A, lda, W, ldw, bias, C, ldc, M, N, K, mode);
-        else gemm_f32_rows_kernel<16><<<rows_grid, 256, 0, stream>>>(A, lda, W, ldw, bias, C, ldc, M, N, K, mode);
+        // Workgroups start at a limited rate (a few hundred a microsecond over the chip): from 2,048 columns on
+        // a workgroup takes eight instead of four, which also halves what is staged (sixteen lose again: at
+        // 50,257 columns 54 us against 45).
+        if (N >= 2048) {
+            const dim3 rows_grid((N + 7) / 8);
+            if (M <= 8) gemm_f32_rows_kernel<8, 8><<<rows_grid, 512, 0, stream>>>(A, lda, W, ldw, bias, C, ldc, M, N, K, mode);
+            else gemm_f32_rows_kernel<16, 8><<<rows_grid, 512, 0, stream>>>(A, lda, W, ldw, bias, C, ldc, M, N, K, mode);
+        } else {
+            const dim3 rows_grid((N + 3) / 4);
+            if (M <= 8) gemm_f32_rows_kernel<8, 4><<<rows_grid, 256, 0, stream>>>(A, lda, W, ldw, bias, C, ldc, M, N, K, mode);
+            else gemm_f32_rows_kernel<16, 4><<<rows_grid, 256, 0, stream>>>(A, lda, W, ldw, bias, C, ldc, M, N, K, mode);
+        }
         MLLM_LAUNCH_CHECK();
         return 0;
     }
