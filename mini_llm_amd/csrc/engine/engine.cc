@@ -24,6 +24,16 @@ float uniform01(uint64_t seed, uint64_t index) {
 CacheStorage::CacheStorage(const std::vector<CacheNeed>& needs, int page_size, int n_pages, int n_state_slots, int dtype)
     : page_size_(page_size), dtype_(dtype) {
     if (page_size < 1 || n_pages < 0 || n_state_slots < 1) throw EngineError("cache: bad page size, page count or slot count");
+    try {
+        allocate(needs, n_pages, n_state_slots);
+    } catch (...) {
+        for (void* p : allocations_) (void)hipFree(p);    // (no destructor runs for a constructor that throws)
+        throw;
+    }
+}
+
+void CacheStorage::allocate(const std::vector<CacheNeed>& needs, int n_pages, int n_state_slots) {
+    const int page_size = page_size_, dtype = dtype_;
     struct Key { int hkv, hd, window; bool operator==(const Key& o) const { return hkv == o.hkv && hd == o.hd && window == o.window; } };
     std::vector<Key> keys;
     std::vector<std::vector<int>> members;
@@ -50,9 +60,9 @@ CacheStorage::CacheStorage(const std::vector<CacheNeed>& needs, int page_size, i
         const size_t bytes = one * 2 * members[g].size();
         void* pool = nullptr;
         HIP_OK(hipMalloc(&pool, std::max<size_t>(bytes, 16)));
-        HIP_OK(hipMemset(pool, 0, std::max<size_t>(bytes, 16)));
         allocations_.push_back(pool);
         allocation_bytes_.push_back(bytes);
+        HIP_OK(hipMemset(pool, 0, std::max<size_t>(bytes, 16)));
         for (size_t j = 0; j < members[g].size(); ++j) {
             CacheView& v = views_[members[g][j]];
             v.kind = 1;
@@ -69,9 +79,9 @@ CacheStorage::CacheStorage(const std::vector<CacheNeed>& needs, int page_size, i
         void* state = nullptr;
         const size_t bytes = needs[c].state_bytes * n_state_slots;
         HIP_OK(hipMalloc(&state, std::max<size_t>(bytes, 16)));
-        HIP_OK(hipMemset(state, 0, std::max<size_t>(bytes, 16)));
         allocations_.push_back(state);
         allocation_bytes_.push_back(bytes);
+        HIP_OK(hipMemset(state, 0, std::max<size_t>(bytes, 16)));
         views_[c].kind = 2;
         views_[c].state = state;
         views_[c].slot_bytes = needs[c].state_bytes;
@@ -115,14 +125,24 @@ static int pages_for_memory_fraction(const std::vector<CacheNeed>& needs, int dt
 
 ModelRunner::ModelRunner(LoadedModel& model, const RunnerOptions& o)
     : model_(model), page_size_(o.page_size), n_pages_(o.n_pages), max_num_seqs_(std::max(o.max_num_seqs, 1)) {
-    init(o);
+    try {
+        init(o);
+    } catch (...) {
+        destroy();                   // (no destructor runs for a constructor that throws)
+        throw;
+    }
 }
 
 ModelRunner::ModelRunner(LoadedModel& model, int page_size, int n_pages, int max_num_seqs)
     : model_(model), page_size_(page_size), n_pages_(n_pages), max_num_seqs_(std::max(max_num_seqs, 1)) {
     RunnerOptions o;
     o.page_size = page_size; o.n_pages = n_pages; o.max_num_seqs = max_num_seqs;
-    init(o);
+    try {
+        init(o);
+    } catch (...) {
+        destroy();
+        throw;
+    }
 }
 
 void ModelRunner::init(const RunnerOptions& o) {
@@ -155,8 +175,11 @@ void ModelRunner::init(const RunnerOptions& o) {
     cache_.reset(new CacheStorage(model_.caches, page_size_, n_pages_, max_num_seqs_, model_.dtype));
 }
 
-ModelRunner::~ModelRunner() {
-    (void)hipStreamSynchronize(stream_);
+ModelRunner::~ModelRunner() { destroy(); }
+
+void ModelRunner::destroy() noexcept {
+    if (stream_) (void)hipStreamSynchronize(stream_);
+    cache_.reset();
     for (auto& st : staging_) {
         if (st.host) (void)hipHostFree(st.host);
         if (st.copied) (void)hipEventDestroy(st.copied);
@@ -169,8 +192,9 @@ ModelRunner::~ModelRunner() {
     for (void* p : {static_cast<void*>(dev_ints_), arena_, static_cast<void*>(logits_), static_cast<void*>(tok_out_)})
         if (p) (void)hipFree(p);
     if (stream_) {
-        release_scratch(stream_);
+        try { release_scratch(stream_); } catch (...) {}
         (void)hipStreamDestroy(stream_);
+        stream_ = nullptr;
     }
 }
 
@@ -329,8 +353,8 @@ float* ModelRunner::run(const StepView& step) {
 
 const float* ModelRunner::step(const std::vector<StepEntry>& entries, bool manage_cache, int* n_rows) {
     CacheManager& mgr = manager();
+    std::vector<int64_t> fresh;
     if (manage_cache) {
-        std::vector<int64_t> fresh;
         try {
             for (const StepEntry& e : entries) {
                 if (!mgr.has_request(e.request_id)) {
@@ -346,8 +370,15 @@ const float* ModelRunner::step(const std::vector<StepEntry>& entries, bool manag
             throw;
         }
     }
-    const StepView sv = build(entries, nullptr, nullptr, nullptr, nullptr);
-    float* logits = run(sv);
+    StepView sv;
+    float* logits = nullptr;
+    try {
+        sv = build(entries, nullptr, nullptr, nullptr, nullptr);
+        logits = run(sv);
+    } catch (...) {
+        for (int64_t id : fresh) mgr.free_request(id);       // a step that fails registers nothing
+        throw;
+    }
     if (manage_cache)
         for (const StepEntry& e : entries) mgr.commit(e.request_id, mgr.length(e.request_id) + static_cast<int>(e.tokens.size()));
     if (n_rows) *n_rows = logits != nullptr ? sv.n_logits : 0;
@@ -367,6 +398,7 @@ const float* ModelRunner::step(const std::vector<StepEntry>& entries, bool manag
 
 int ModelRunner::launch(const std::vector<StepEntry>& entries, const std::vector<float>& temperatures,
                         const std::vector<float>& uniforms) {
+    if (pending_.size() >= 2) throw EngineError("two launches have tokens unread: collect() before a third");
     const float *d_temps = nullptr, *d_u = nullptr;
     const StepView sv = build(entries, &temperatures, &uniforms, &d_temps, &d_u);
     float* logits = run(sv);

@@ -72,6 +72,8 @@ class CacheStorage {
 public:
     CacheStorage(const std::vector<CacheNeed>& needs, int page_size, int n_pages, int n_state_slots, int dtype);
     ~CacheStorage();
+    CacheStorage(const CacheStorage&) = delete;
+    CacheStorage& operator=(const CacheStorage&) = delete;
     CacheManager& manager() { return *manager_; }
     const std::vector<CacheView>& views() const { return views_; }
     int n_groups() const { return static_cast<int>(group_specs_.size()); }
@@ -81,6 +83,7 @@ public:
     void poison();                     // fills every page with NaN (tests)
 
 private:
+    void allocate(const std::vector<CacheNeed>& needs, int n_pages, int n_state_slots);
     int page_size_, dtype_;
     std::vector<GroupSpec> group_specs_;
     std::vector<CacheView> views_;
@@ -138,6 +141,7 @@ public:
 
 private:
     void init(const RunnerOptions& o);
+    void destroy() noexcept;
     struct Staging {
         int* host = nullptr;
         size_t capacity = 0;

@@ -283,10 +283,12 @@ int mllm_runner_step(void* runner, const long long* ids, const int* n_tokens, co
                      const int* want, int B, float* logits, long long cap_rows) {
     int rows = -1;
     guarded([&] {
+        if (B < 0) fail("a step of %d entries", B);
         std::vector<StepEntry> entries(B);
         size_t t = 0, w = 0;
         long long total = 0;
         for (int i = 0; i < B; ++i) {
+            if (n_tokens[i] < 0 || n_want[i] < 0) fail("entry %d brings %d tokens and wants %d places", i, n_tokens[i], n_want[i]);
             entries[i].request_id = ids[i];
             entries[i].tokens.assign(tokens + t, tokens + t + n_tokens[i]);
             entries[i].want.assign(want + w, want + w + n_want[i]);
@@ -382,16 +384,22 @@ long long mllm_engine_add_request(void* e, const int* tokens, int n, float tempe
                                   int max_new_tokens, int ignore_eos, long long request_id) {
     long long id = -1;
     guarded([&] {
+        if (n < 0 || (n > 0 && tokens == nullptr)) fail("a prompt of %d tokens", n);
         SamplingParams sp;
         sp.temperature = temperature; sp.seed = seed; sp.max_new_tokens = max_new_tokens; sp.ignore_eos = ignore_eos != 0;
         id = static_cast<Engine*>(e)->add_request(std::vector<int>(tokens, tokens + n), sp, request_id);
     });
     return id;
 }
-int mllm_engine_has_unfinished(void* e) { return static_cast<Engine*>(e)->has_unfinished() ? 1 : 0; }
+int mllm_engine_has_unfinished(void* e) {
+    int r = 0;
+    guarded([&] { r = static_cast<Engine*>(e)->has_unfinished() ? 1 : 0; });
+    return r;
+}
 // One iteration. Up to `cap` outputs are written (ids, tokens, finished flags; a token of -1 is a failed request);
 // outputs beyond `cap` wait for the next call, and mllm_engine_has_unfinished stays 1 meanwhile. Returns their
-// number, or -1 on an error. The reason of the i-th output's failure: mllm_engine_output_error(e, i).
+// number, or -1 on an error. The reason of the i-th output's failure: mllm_engine_output_error(i), on the thread
+// that made the call.
 namespace { thread_local std::vector<std::string> g_output_errors; }
 int mllm_engine_step(void* e, long long* ids, int* tokens, int* finished, int cap) {
     int n = -1;
@@ -413,11 +421,13 @@ const char* mllm_engine_output_error(int i) {
 int mllm_engine_abort(void* e, long long id) { return guarded([&] { static_cast<Engine*>(e)->abort(id); }); }
 // names: steps, scheduled_tokens, prefill_tokens, decode_tokens, deferred_decodes, deferred_prefills, preemptions,
 // failures, finished, peak_pages_used, free_pages, total_pages (in this order)
-void mllm_engine_stats(void* e, long long* out12) {
-    const auto st = static_cast<Engine*>(e)->stats();
-    const char* names[12] = {"steps", "scheduled_tokens", "prefill_tokens", "decode_tokens", "deferred_decodes", "deferred_prefills",
-                             "preemptions", "failures", "finished", "peak_pages_used", "free_pages", "total_pages"};
-    for (int i = 0; i < 12; ++i) out12[i] = st.at(names[i]);
+int mllm_engine_stats(void* e, long long* out12) {
+    return guarded([&] {
+        const auto st = static_cast<Engine*>(e)->stats();
+        const char* names[12] = {"steps", "scheduled_tokens", "prefill_tokens", "decode_tokens", "deferred_decodes", "deferred_prefills",
+                                 "preemptions", "failures", "finished", "peak_pages_used", "free_pages", "total_pages"};
+        for (int i = 0; i < 12; ++i) out12[i] = st.at(names[i]);
+    });
 }
 void mllm_engine_synchronize(void* e) { guarded([&] { static_cast<Engine*>(e)->runner().synchronize(); }); }
 

@@ -97,10 +97,10 @@ __global__ void layernorm_kernel(const float* __restrict__ x, const int* __restr
     }
 }
 
-// Same norm, one wavefront per row (four rows per workgroup), the row in registers as float4:
+// Same norm, one wavefront per row (WAVES rows per workgroup), the row in registers as float4:
 // for D % 4 == 0 and D <= 2048. Fewer, fatter workgroups and 16-byte accesses.
-template <typename OutT>
-__global__ void __launch_bounds__(256)
+template <typename OutT, int WAVES>
+__global__ void __launch_bounds__(64 * WAVES)
 layernorm_wave_kernel(const float* __restrict__ x, const int* __restrict__ rows,
                       const float* __restrict__ gamma, const float* __restrict__ beta,
                       OutT* __restrict__ y, int n, int D, float eps) {
@@ -109,7 +109,7 @@ layernorm_wave_kernel(const float* __restrict__ x, const int* __restrict__ rows,
     // load under a condition, or one left inside the last loop, starts only when the statistics
     // are done and adds its whole latency)
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / MLLM_WAVE), lane = threadIdx.x % MLLM_WAVE;
-    const int r = blockIdx.x * 4 + wave;
+    const int r = blockIdx.x * WAVES + wave;
     if (r >= n) return;
     const int src = rows ? rows[r] : r;
     const float4* xr = reinterpret_cast<const float4*>(x + static_cast<size_t>(src) * D);
@@ -239,11 +239,21 @@ int mllm_layernorm(const float* x, const int* rows, const float* gamma, const fl
     const bool aligned = ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(gamma) |
                            reinterpret_cast<uintptr_t>(beta) | reinterpret_cast<uintptr_t>(y)) & 15) == 0;
     if (D % 4 == 0 && D <= 2048 && aligned) {
-        const int blocks = (n + 3) / 4;
-        if (out_dtype == MLLM_F32)
-            layernorm_wave_kernel<float><<<blocks, 256, 0, stream>>>(x, rows, gamma, beta, (float*)y, n, D, eps);
-        else
-            layernorm_wave_kernel<bf16_t><<<blocks, 256, 0, stream>>>(x, rows, gamma, beta, (bf16_t*)y, n, D, eps);
+        // Workgroups start at a limited rate (about 200 a microsecond over the chip): many rows go eight to a
+        // workgroup instead of four (2,048 rows of 768: 6.9 us with 512 workgroups of four)
+        if (n >= 512) {
+            const int blocks = (n + 7) / 8;
+            if (out_dtype == MLLM_F32)
+                layernorm_wave_kernel<float, 8><<<blocks, 512, 0, stream>>>(x, rows, gamma, beta, (float*)y, n, D, eps);
+            else
+                layernorm_wave_kernel<bf16_t, 8><<<blocks, 512, 0, stream>>>(x, rows, gamma, beta, (bf16_t*)y, n, D, eps);
+        } else {
+            const int blocks = (n + 3) / 4;
+            if (out_dtype == MLLM_F32)
+                layernorm_wave_kernel<float, 4><<<blocks, 256, 0, stream>>>(x, rows, gamma, beta, (float*)y, n, D, eps);
+            else
+                layernorm_wave_kernel<bf16_t, 4><<<blocks, 256, 0, stream>>>(x, rows, gamma, beta, (bf16_t*)y, n, D, eps);
+        }
         MLLM_LAUNCH_CHECK();
         return 0;
     }

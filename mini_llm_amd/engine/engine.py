@@ -169,7 +169,7 @@ class Engine:
 
     def stats(self) -> Dict[str, int]:
         buf = np.zeros(12, dtype=np.int64)
-        self._lib.mllm_engine_stats(self._h, buf.ctypes.data)
+        native.check(self._lib.mllm_engine_stats(self._h, buf.ctypes.data))
         return dict(zip(_STATS, (int(v) for v in buf)))
 
     def synchronize(self) -> None:

@@ -77,7 +77,7 @@ def lib():
         "mllm_engine_step": (_i, [_vp, _vp, _vp, _vp, _i]),
         "mllm_engine_output_error": (_cp, [_i]),
         "mllm_engine_abort": (_i, [_vp, _ll]),
-        "mllm_engine_stats": (None, [_vp, _vp]),
+        "mllm_engine_stats": (_i, [_vp, _vp]),
         "mllm_engine_synchronize": (None, [_vp]),
         # tuning and scratch (tests)
         "mllm_set_tuning": (_i, [_cp, _i, _i]),
