@@ -419,12 +419,7 @@ int ModelRunner::launch(const std::vector<StepEntry>& entries, const std::vector
         tok_out_ = fresh;
         tok_out_cap_ = cap;
     }
-    const Tensor2 lg(logits, F32, n, model_.model.vocab_size());
-    bool greedy = true;
-    for (float t : temperatures) greedy = greedy && t <= 0.f;
-    if (greedy) argmax(lg, tok_out_, stream_);
-    else sample(lg, d_temps, d_u, tok_out_, stream_);
-    // two host buffers in turn: one may still be unread when the next step's copy is queued
+    // two host buffers in turn: one may still be unread when the next step writes its own
     host_turn_ ^= 1;
     if (host_tok_cap_ < n) {
         HIP_OK(hipStreamSynchronize(stream_));
@@ -432,10 +427,17 @@ int ModelRunner::launch(const std::vector<StepEntry>& entries, const std::vector
         host_tok_cap_ = std::max(n, 64) * 2;
         for (int i = 0; i < 2; ++i) {
             if (host_tok_[i]) HIP_OK(hipHostFree(host_tok_[i]));
+            host_tok_[i] = nullptr;
             HIP_OK(hipHostMalloc(reinterpret_cast<void**>(&host_tok_[i]), host_tok_cap_ * sizeof(int), hipHostMallocDefault));
         }
     }
-    HIP_OK(hipMemcpyAsync(host_tok_[host_turn_], tok_out_, n * sizeof(int), hipMemcpyDeviceToHost, stream_));
+    // the sampling kernel writes the tokens to the device (for the next launch) and to the pinned host buffer
+    // itself; the event behind it tells the host when they are there
+    const Tensor2 lg(logits, F32, n, model_.model.vocab_size());
+    bool greedy = true;
+    for (float t : temperatures) greedy = greedy && t <= 0.f;
+    if (greedy) argmax(lg, tok_out_, stream_, host_tok_[host_turn_]);
+    else sample(lg, d_temps, d_u, tok_out_, stream_, host_tok_[host_turn_]);
     HIP_OK(hipEventRecord(host_tok_event_[host_turn_], stream_));
     pending_.push_back({host_tok_[host_turn_], n, host_tok_event_[host_turn_]});
     return n;

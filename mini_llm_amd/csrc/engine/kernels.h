@@ -60,9 +60,9 @@ int mllm_prefill_attention_bf16(const void* q, int q_stride, int q_col, const vo
 
 // sampling.hip
 int mllm_argmax_chunks(int V);
-int mllm_argmax(const float* logits, int ld, int n, int V, int* out, float* part_val, int* part_idx,
+int mllm_argmax_mirrored(const float* logits, int ld, int n, int V, int* out, int* mirror, float* part_val, int* part_idx,
                 hipStream_t stream);
-int mllm_sample(const float* logits, int ld, int n, int V, const float* temperature, const float* u, int* out,
+int mllm_sample_mirrored(const float* logits, int ld, int n, int V, const float* temperature, const float* u, int* out, int* mirror,
                 hipStream_t stream);
 
 }  // extern "C"

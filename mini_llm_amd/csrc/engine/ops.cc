@@ -499,20 +499,20 @@ bool paged_attention(const AttentionArgs& a, AttentionSplits* splits, hipStream_
 // ---------------------------------------------------------------------------------------------
 // sampling
 // ---------------------------------------------------------------------------------------------
-void argmax(const Tensor2& logits, int* out, hipStream_t stream) {
+void argmax(const Tensor2& logits, int* out, hipStream_t stream, int* mirror) {
     if (logits.dtype != F32) fail("argmax: logits must be float32");
     const int n = static_cast<int>(logits.rows), V = static_cast<int>(logits.cols);
     const size_t chunks = static_cast<size_t>(mllm_argmax_chunks(V));
     float* pv = argmax_values(n * chunks, stream);
     int* pi = argmax_indices(n * chunks, stream);
-    check(mllm_argmax(static_cast<const float*>(logits.data), static_cast<int>(logits.stride), n, V, out, pv, pi, stream), "argmax");
+    check(mllm_argmax_mirrored(static_cast<const float*>(logits.data), static_cast<int>(logits.stride), n, V, out, mirror, pv, pi, stream), "argmax");
 }
 
-void sample(const Tensor2& logits, const float* temperature, const float* u, int* out, hipStream_t stream) {
+void sample(const Tensor2& logits, const float* temperature, const float* u, int* out, hipStream_t stream, int* mirror) {
     if (logits.dtype != F32) fail("sample: logits must be float32");
     if (temperature == nullptr || u == nullptr) fail("sample: temperatures and uniform numbers are needed");
-    check(mllm_sample(static_cast<const float*>(logits.data), static_cast<int>(logits.stride), static_cast<int>(logits.rows),
-                      static_cast<int>(logits.cols), temperature, u, out, stream), "sample");
+    check(mllm_sample_mirrored(static_cast<const float*>(logits.data), static_cast<int>(logits.stride), static_cast<int>(logits.rows),
+                      static_cast<int>(logits.cols), temperature, u, out, mirror, stream), "sample");
 }
 
 }  // namespace minillm

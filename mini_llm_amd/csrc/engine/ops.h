@@ -149,7 +149,9 @@ void ln_linear(const Tensor2& x, const float* gamma, const float* beta, float ep
 // Causal attention of the step's queries over the pages. Returns true and fills *splits when the result is
 // left unmerged (only with may_split); otherwise `out` holds it.
 bool paged_attention(const AttentionArgs& a, AttentionSplits* splits, hipStream_t stream);
-void argmax(const Tensor2& logits, int* out, hipStream_t stream);
-void sample(const Tensor2& logits, const float* temperature, const float* u, int* out, hipStream_t stream);
+// `mirror` (optional): a second place for the chosen tokens, which may be pinned host memory (the kernel that
+// chooses writes it: no copy has to be launched for the host to read them).
+void argmax(const Tensor2& logits, int* out, hipStream_t stream, int* mirror = nullptr);
+void sample(const Tensor2& logits, const float* temperature, const float* u, int* out, hipStream_t stream, int* mirror = nullptr);
 
 }  // namespace minillm

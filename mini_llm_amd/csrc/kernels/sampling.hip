@@ -17,8 +17,11 @@ __device__ __forceinline__ bool better(float v, int i, float bv, int bi) {
 
 // Stage 1: the best (value, index) of one chunk of one row. Stage 2 (n_chunks == 1 input
 // chunks of pairs) reduces the chunks' results. Both keep the lowest index on ties.
+// `mirror` (in all kernels here; may be null): a second place for the tokens, which may be pinned host memory:
+// the kernel that chooses a token hands it to the host itself, where a copy would be one more launch.
 __global__ void argmax_stage1(const float* __restrict__ logits, int ld, int V, int n_chunks,
-                              float* __restrict__ part_val, int* __restrict__ part_idx, int* __restrict__ out) {
+                              float* __restrict__ part_val, int* __restrict__ part_idx, int* __restrict__ out,
+                              int* __restrict__ mirror) {
     __shared__ float sv[SAMPLE_THREADS / MLLM_WAVE];
     __shared__ int si[SAMPLE_THREADS / MLLM_WAVE];
     const int row_id = blockIdx.y, chunk = blockIdx.x;
@@ -50,7 +53,9 @@ __global__ void argmax_stage1(const float* __restrict__ logits, int ld, int V, i
         for (int w = 1; w < SAMPLE_THREADS / MLLM_WAVE; ++w)
             if (better(sv[w], si[w], bv, bi)) { bv = sv[w]; bi = si[w]; }
         if (n_chunks == 1) {
-            out[row_id] = (bi == 0x7fffffff) ? 0 : bi;       // a row of NaNs yields 0
+            const int tok = (bi == 0x7fffffff) ? 0 : bi;     // a row of NaNs yields 0
+            out[row_id] = tok;
+            if (mirror != nullptr) mirror[row_id] = tok;
         } else {
             part_val[static_cast<size_t>(row_id) * n_chunks + chunk] = bv;
             part_idx[static_cast<size_t>(row_id) * n_chunks + chunk] = bi;
@@ -59,7 +64,7 @@ __global__ void argmax_stage1(const float* __restrict__ logits, int ld, int V, i
 }
 
 __global__ void argmax_stage2(const float* __restrict__ part_val, const int* __restrict__ part_idx,
-                              int n_chunks, int* __restrict__ out) {
+                              int n_chunks, int* __restrict__ out, int* __restrict__ mirror) {
     const int row_id = blockIdx.x, lane = threadIdx.x;      // one wavefront per row
     float bv = -INFINITY;
     int bi = 0x7fffffff;
@@ -74,7 +79,11 @@ __global__ void argmax_stage2(const float* __restrict__ part_val, const int* __r
         int oi = __shfl_xor(bi, off, MLLM_WAVE);
         if (better(ov, oi, bv, bi)) { bv = ov; bi = oi; }
     }
-    if (lane == 0) out[row_id] = (bi == 0x7fffffff) ? 0 : bi;
+    if (lane == 0) {
+        const int tok = (bi == 0x7fffffff) ? 0 : bi;
+        out[row_id] = tok;
+        if (mirror != nullptr) mirror[row_id] = tok;
+    }
 }
 
 // ---------------------------------------------------------------------------
@@ -95,7 +104,7 @@ __global__ void argmax_stage2(const float* __restrict__ part_val, const int* __r
 
 __global__ void __launch_bounds__(SAMPLE_BLOCK)
 sample_kernel(const float* __restrict__ logits, int ld, int V, const float* __restrict__ temperature,
-              const float* __restrict__ u, int* __restrict__ out) {
+              const float* __restrict__ u, int* __restrict__ out, int* __restrict__ mirror) {
     __shared__ float sv[SAMPLE_BLOCK / MLLM_WAVE];
     __shared__ int si[SAMPLE_BLOCK / MLLM_WAVE];
     __shared__ float tile_mass[SAMPLE_MAX_TILES];
@@ -134,7 +143,11 @@ sample_kernel(const float* __restrict__ logits, int ld, int V, const float* __re
     for (int w = 1; w < SAMPLE_BLOCK / MLLM_WAVE; ++w)
         if (better(sv[w], si[w], bv, bi)) { bv = sv[w]; bi = si[w]; }
     if (temp <= 0.f) {                       // greedy row (uniform over the workgroup)
-        if (tid == 0) out[r] = (bi == 0x7fffffff) ? 0 : bi;
+        if (tid == 0) {
+            const int tok = (bi == 0x7fffffff) ? 0 : bi;
+            out[r] = tok;
+            if (mirror != nullptr) mirror[r] = tok;
+        }
         return;
     }
     // e^((x - max)/T) as 2^((x - max) * log2(e)/T)
@@ -218,7 +231,9 @@ sample_kernel(const float* __restrict__ logits, int ld, int V, const float* __re
             c += p[k];
             if (pick < 0 && rest < c && p[k] > 0.f) pick = base + k;
         }
-        out[r] = pick >= 0 ? pick : last;
+        const int tok = pick >= 0 ? pick : last;
+        out[r] = tok;
+        if (mirror != nullptr) mirror[r] = tok;
     }
 }
 
@@ -227,18 +242,24 @@ extern "C" {
 // Chunks of the first stage for a row of V values: the scratch holds n * chunks floats and ints.
 int mllm_argmax_chunks(int V) { return (V + ARGMAX_CHUNK - 1) / ARGMAX_CHUNK; }
 
-int mllm_argmax(const float* logits, int ld, int n, int V, int* out, float* part_val, int* part_idx,
-                hipStream_t stream) {
+// out[r] = index of the largest of row r (the lowest on ties); `mirror`, if given, gets the same (see above).
+int mllm_argmax_mirrored(const float* logits, int ld, int n, int V, int* out, int* mirror, float* part_val,
+                         int* part_idx, hipStream_t stream) {
     if (n <= 0) return 0;
     if (V <= 0) return -1;
     const int n_chunks = (V + ARGMAX_CHUNK - 1) / ARGMAX_CHUNK;
-    argmax_stage1<<<dim3(n_chunks, n), SAMPLE_THREADS, 0, stream>>>(logits, ld, V, n_chunks, part_val, part_idx, out);
+    argmax_stage1<<<dim3(n_chunks, n), SAMPLE_THREADS, 0, stream>>>(logits, ld, V, n_chunks, part_val, part_idx, out, mirror);
     MLLM_LAUNCH_CHECK();
     if (n_chunks > 1) {
-        argmax_stage2<<<n, MLLM_WAVE, 0, stream>>>(part_val, part_idx, n_chunks, out);
+        argmax_stage2<<<n, MLLM_WAVE, 0, stream>>>(part_val, part_idx, n_chunks, out, mirror);
         MLLM_LAUNCH_CHECK();
     }
     return 0;
+}
+
+int mllm_argmax(const float* logits, int ld, int n, int V, int* out, float* part_val, int* part_idx,
+                hipStream_t stream) {
+    return mllm_argmax_mirrored(logits, ld, n, V, out, nullptr, part_val, part_idx, stream);
 }
 
 }  // extern "C"
@@ -288,13 +309,18 @@ int mllm_argmax_noalloc(const float* logits, int ld, int n, int V, int* out, hip
     return mllm_argmax(logits, ld, n, V, out, part_val, part_idx, stream);
 }
 
-int mllm_sample(const float* logits, int ld, int n, int V, const float* temperature, const float* u, int* out,
-                hipStream_t stream) {
+int mllm_sample_mirrored(const float* logits, int ld, int n, int V, const float* temperature, const float* u,
+                         int* out, int* mirror, hipStream_t stream) {
     if (n <= 0) return 0;
     if (V <= 0 || V > SAMPLE_TILE * SAMPLE_MAX_TILES) return -1;
-    sample_kernel<<<n, SAMPLE_BLOCK, 0, stream>>>(logits, ld, V, temperature, u, out);
+    sample_kernel<<<n, SAMPLE_BLOCK, 0, stream>>>(logits, ld, V, temperature, u, out, mirror);
     MLLM_LAUNCH_CHECK();
     return 0;
+}
+
+int mllm_sample(const float* logits, int ld, int n, int V, const float* temperature, const float* u, int* out,
+                hipStream_t stream) {
+    return mllm_sample_mirrored(logits, ld, n, V, temperature, u, out, nullptr, stream);
 }
 
 }  // extern "C"

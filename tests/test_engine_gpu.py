@@ -454,6 +454,37 @@ def test_more_failed_requests_than_a_step_call_has_room_for(tiny_model_dirs):
     assert e.stats()["failures"] == 60 and e.stats()["free_pages"] == 8
 
 
+def test_a_step_that_fails_leaves_the_runner_as_it_was(tiny_model_dirs):
+    """A step with a token outside the vocabulary, with a wanted place outside its tokens, or with counts that make
+    no sense is refused with a message; the requests it would have registered hold nothing afterwards, and the
+    same ids step normally after it."""
+    import ctypes
+    import numpy as np
+    from mini_llm_amd import EngineError, Runner, StepEntry, native
+    cfg = TINY["a"][0]
+    runner = Runner(model_dir=tiny_model_dirs["a"], dtype="float32", page_size=4, n_pages=16, max_num_seqs=4)
+    with pytest.raises(EngineError, match="token ids must lie in"):
+        runner.step([StepEntry(1, [3, 4, 5], want=[2]), StepEntry(2, [7, cfg["vocab_size"]], want=[])])
+    with pytest.raises(EngineError, match="wanted index 3 is outside its 3 tokens"):
+        runner.step([StepEntry(1, [3, 4, 5], want=[3])])
+    info = runner.info()
+    assert info["n_requests"] == 0 and info["free_pages"] == 16 and runner.check() == ""
+    # the C function itself refuses counts below zero (the Python face cannot produce them)
+    lib = native.lib()
+    ids, n_tok, toks = np.array([1], np.int64), np.array([-1], np.int32), np.array([3], np.int32)
+    n_want, want, out = np.array([0], np.int32), np.array([0], np.int32), np.zeros(cfg["vocab_size"], np.float32)
+    rc = lib.mllm_runner_step(runner._h, ids.ctypes.data, n_tok.ctypes.data, toks.ctypes.data, n_want.ctypes.data,
+                              want.ctypes.data, 1, out.ctypes.data, 1)
+    assert rc == -1 and "brings -1 tokens" in native.last_error()
+    assert lib.mllm_runner_step(runner._h, None, None, None, None, None, -2, None, 0) == -1
+    # and the ids are free for a proper step
+    got = runner.step([StepEntry(1, [3, 4, 5], want=[2]), StepEntry(2, [7, 8], want=[1])])
+    assert got.shape == (2, cfg["vocab_size"]) and np.isfinite(got).all()
+    runner.end_request(1)
+    runner.end_request(2)
+    assert runner.info()["free_pages"] == 16
+
+
 XL_WIDTH = dict(architectures=["GPT2LMHeadModel"], model_type="gpt2", n_layer=2, n_embd=1600, n_head=25, n_inner=6400,
                 vocab_size=5003, n_positions=1024, layer_norm_epsilon=1e-5, activation_function="gelu_new",
                 eos_token_id=5002, bos_token_id=5002)
