@@ -126,6 +126,54 @@ def test_first_tokens_and_long_decoding(tiny_model_dirs, dtype):
     rc.check_against_plain(tiny_model_dirs[name], name, reqs, steps, out, dtype)
 
 
+def _other(L, H, dh, F, V, P, eps, act):
+    return dict(architectures=["GPT2LMHeadModel"], model_type="gpt2", n_layer=L, n_embd=H * dh, n_head=H, n_inner=F,
+                vocab_size=V, n_positions=P, layer_norm_epsilon=eps, activation_function=act, eos_token_id=V - 1,
+                bos_token_id=V - 1)
+
+
+# sizes that neither the tiny nor the real configurations have: seven heads of 16, three of 48, two of 80, one of 256;
+# widths, inner widths and vocabularies that are no power of two; one to five layers; four eps; the three activation names
+OTHER_SIZES = {
+    "7x16": _other(2, 7, 16, 200, 517, 192, 1e-3, "gelu"),
+    "3x48": _other(3, 3, 48, 576, 777, 200, 1e-6, "gelu_pytorch_tanh"),
+    "2x80": _other(5, 2, 80, 328, 4099, 300, 1e-5, "gelu_new"),
+    "1x256": _other(1, 1, 256, 1000, 333, 130, 1e-4, "gelu"),
+}
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", sorted(OTHER_SIZES))
+def test_other_sizes_end_to_end(tmp_path, name, dtype):
+    """Whole prompts and mixed batches at further sizes, against the plain implementation. Allowed: about three
+    times the worst seen over these four (float32 1.5e-6 of a row, mean 2.0e-7; bfloat16 4.3e-3 and 1.0e-3; the
+    logits' own standard deviation is 0.2 to 0.3)."""
+    from mini_llm_amd import Runner, write_random_model
+    cfg = OTHER_SIZES[name]
+    d = write_random_model(cfg, str(tmp_path / name), seed=50 + len(name))
+    pc, w = plain_gpt2.read_model(d)
+    P, V = cfg["n_positions"], cfg["vocab_size"]
+    reqs = ru.random_requests(V, [1, 2, 15, 16, 17, P // 3, P - 1, P], seed=300)
+    ref = {rid: plain_gpt2.forward_logits(pc, w, list(t)).numpy() for rid, t in reqs.items()}
+    tol = dict(max_abs=4.5e-6, mean_abs=6e-7) if dtype == "float32" else dict(max_abs=1.3e-2, mean_abs=3e-3)
+    worst = worst_mean = 0.0
+    for fam, steps, page in (("whole", ru.trace_whole(reqs), 16), ("mixed", ru.trace_mixed(reqs, seed=3)[0], 8)):
+        n_pages = -(-ru.peak_tokens(steps) // page)
+        runner = Runner(model_dir=d, dtype=dtype, page_size=page, n_pages=n_pages, max_num_seqs=8)
+        runner.poison_cache()
+        got = ru.collect(steps, ru.run_in_process(runner, steps), V)
+        for rid, rows in got.items():
+            assert len(rows) == len(reqs[rid])
+            for pos, row in rows.items():
+                assert np.isfinite(row).all(), (fam, rid, pos)
+                diff = np.abs(row.astype(np.float64) - ref[rid][pos])
+                worst, worst_mean = max(worst, diff.max()), max(worst_mean, diff.mean())
+                assert diff.max() <= tol["max_abs"] and diff.mean() <= tol["mean_abs"], (fam, rid, pos, diff.max(), diff.mean())
+        _all_pages_back(runner, n_pages)
+    print(f"worst difference from plain at {name} [{dtype}]: max {worst:.3e}, mean {worst_mean:.3e} "
+          f"(allowed {tol['max_abs']:.1e}, {tol['mean_abs']:.1e})")
+
+
 # A context far beyond GPT-2's own: n_positions is a free key of config.json. Narrow (two heads of 64), so
 # that the plain implementation's 4,700 x 4,700 scores stay cheap.
 LONG = dict(architectures=["GPT2LMHeadModel"], model_type="gpt2", n_layer=2, n_embd=128, n_head=2, n_inner=256,
