@@ -677,7 +677,8 @@ std::map<std::string, int64_t> Engine::stats() const {
     CacheManager& m = runner_->manager();
     return {{"steps", c.steps}, {"scheduled_tokens", c.scheduled_tokens}, {"prefill_tokens", c.prefill_tokens},
             {"decode_tokens", c.decode_tokens}, {"deferred_decodes", c.deferred_decodes}, {"deferred_prefills", c.deferred_prefills},
-            {"preemptions", c.preemptions}, {"failures", c.failures}, {"finished", c.finished}, {"peak_pages_used", c.peak_pages_used},
+            {"preemptions", c.preemptions}, {"failures", c.failures}, {"finished", c.finished}, {"aborted", c.aborted},
+            {"peak_pages_used", c.peak_pages_used},
             {"free_pages", m.n_groups() ? m.free_pages(0) : 0}, {"total_pages", m.n_groups() ? m.total_pages(0) : 0}};
 }
 

@@ -420,13 +420,13 @@ const char* mllm_engine_output_error(int i) {
 }
 int mllm_engine_abort(void* e, long long id) { return guarded([&] { static_cast<Engine*>(e)->abort(id); }); }
 // names: steps, scheduled_tokens, prefill_tokens, decode_tokens, deferred_decodes, deferred_prefills, preemptions,
-// failures, finished, peak_pages_used, free_pages, total_pages (in this order)
-int mllm_engine_stats(void* e, long long* out12) {
+// failures, finished, peak_pages_used, free_pages, total_pages, aborted (in this order)
+int mllm_engine_stats(void* e, long long* out13) {
     return guarded([&] {
         const auto st = static_cast<Engine*>(e)->stats();
-        const char* names[12] = {"steps", "scheduled_tokens", "prefill_tokens", "decode_tokens", "deferred_decodes", "deferred_prefills",
-                                 "preemptions", "failures", "finished", "peak_pages_used", "free_pages", "total_pages"};
-        for (int i = 0; i < 12; ++i) out12[i] = st.at(names[i]);
+        const char* names[13] = {"steps", "scheduled_tokens", "prefill_tokens", "decode_tokens", "deferred_decodes", "deferred_prefills",
+                                 "preemptions", "failures", "finished", "peak_pages_used", "free_pages", "total_pages", "aborted"};
+        for (int i = 0; i < 13; ++i) out13[i] = st.at(names[i]);
     });
 }
 void mllm_engine_synchronize(void* e) { guarded([&] { static_cast<Engine*>(e)->runner().synchronize(); }); }

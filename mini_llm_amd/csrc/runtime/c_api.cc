@@ -105,11 +105,11 @@ int mllm_sched_pop_event(void* s, int64_t* id, int* kind) {
     return 1;
 }
 int mllm_sched_queue_length(void* s, int which) { return static_cast<Scheduler*>(s)->queue_length(which); }
-void mllm_sched_counters(void* s, int64_t* out10) {
+void mllm_sched_counters(void* s, int64_t* out11) {
     const Counters& c = static_cast<Scheduler*>(s)->counters();
-    out10[0] = c.steps; out10[1] = c.scheduled_tokens; out10[2] = c.prefill_tokens; out10[3] = c.decode_tokens;
-    out10[4] = c.deferred_decodes; out10[5] = c.deferred_prefills; out10[6] = c.preemptions;
-    out10[7] = c.failures; out10[8] = c.finished; out10[9] = c.peak_pages_used;
+    out11[0] = c.steps; out11[1] = c.scheduled_tokens; out11[2] = c.prefill_tokens; out11[3] = c.decode_tokens;
+    out11[4] = c.deferred_decodes; out11[5] = c.deferred_prefills; out11[6] = c.preemptions;
+    out11[7] = c.failures; out11[8] = c.finished; out11[9] = c.peak_pages_used; out11[10] = c.aborted;
 }
 
 }  // extern "C"

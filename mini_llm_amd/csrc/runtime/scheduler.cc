@@ -4,6 +4,11 @@
 
 namespace minillm {
 
+static inline bool is_final(RequestState s) {
+    return s == RequestState::Finished || s == RequestState::Failed || s == RequestState::Aborted;
+}
+
+
 Scheduler::Scheduler(CacheManager* cache, const SchedulerOptions& opt) : cache_(cache), opt_(opt) {
     if (opt_.max_num_seqs < 1) opt_.max_num_seqs = 1;
     if (opt_.max_tokens_per_step < 1) opt_.max_tokens_per_step = 1;
@@ -198,7 +203,7 @@ void Scheduler::commit() {
         auto it = reqs_.find(e.id);
         if (it == reqs_.end()) continue;
         Req& r = it->second;
-        if (r.state == RequestState::Finished || r.state == RequestState::Failed) continue;
+        if (is_final(r.state)) continue;
         r.computed = e.start + e.n_tokens;
         cache_->commit(r.id, r.computed);
         counters_.scheduled_tokens += e.n_tokens;
@@ -212,7 +217,7 @@ int Scheduler::on_token(int64_t id, bool is_eos) {
     auto it = reqs_.find(id);
     if (it == reqs_.end()) return -2;
     Req& r = it->second;
-    if (r.state == RequestState::Finished || r.state == RequestState::Failed) return 1;
+    if (is_final(r.state)) return 1;
     r.total_len += 1;
     r.generated += 1;
     if (r.state == RequestState::Prefill) {
@@ -239,6 +244,8 @@ void Scheduler::finish(Req& r, RequestState final_state) {
     if (final_state == RequestState::Failed) {
         ++counters_.failures;
         events_.push_back({r.id, EventKind::Failed});
+    } else if (final_state == RequestState::Aborted) {
+        ++counters_.aborted;             // (no event: the caller who aborts knows)
     } else {
         ++counters_.finished;
     }
@@ -248,10 +255,10 @@ int Scheduler::abort(int64_t id) {
     auto it = reqs_.find(id);
     if (it == reqs_.end()) return -2;
     Req& r = it->second;
-    if (r.state == RequestState::Finished || r.state == RequestState::Failed) return 0;
+    if (is_final(r.state)) return 0;
     plan_.erase(std::remove_if(plan_.begin(), plan_.end(),
                                [id](const PlanEntry& e) { return e.id == id; }), plan_.end());
-    finish(r, RequestState::Failed);
+    finish(r, RequestState::Aborted);
     return 0;
 }
 
@@ -259,7 +266,7 @@ int Scheduler::stop(int64_t id) {
     auto it = reqs_.find(id);
     if (it == reqs_.end()) return -2;
     Req& r = it->second;
-    if (r.state == RequestState::Finished || r.state == RequestState::Failed) return 0;
+    if (is_final(r.state)) return 0;
     plan_.erase(std::remove_if(plan_.begin(), plan_.end(),
                                [id](const PlanEntry& e) { return e.id == id; }), plan_.end());
     finish(r, RequestState::Finished);
@@ -270,7 +277,7 @@ int Scheduler::forget(int64_t id) {
     auto it = reqs_.find(id);
     if (it == reqs_.end()) return -2;
     RequestState st = it->second.state;
-    if (st != RequestState::Finished && st != RequestState::Failed) return -1;
+    if (!is_final(st)) return -1;
     reqs_.erase(it);
     return 0;
 }

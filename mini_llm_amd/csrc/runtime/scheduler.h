@@ -28,7 +28,8 @@ enum class RequestState : int {
     DecodeReady = 3,
     DeferredDecode = 4,    // no page for its next token in this iteration
     Finished = 5,
-    Failed = 6,            // can never run (larger than the whole pool) or aborted
+    Failed = 6,            // can never run (larger than the whole pool)
+    Aborted = 7,           // taken out by the caller
     Unknown = -1,
 };
 
@@ -62,7 +63,7 @@ struct Event {
 struct Counters {
     int64_t steps = 0, scheduled_tokens = 0, prefill_tokens = 0, decode_tokens = 0;
     int64_t deferred_decodes = 0, deferred_prefills = 0, preemptions = 0, failures = 0, finished = 0;
-    int64_t peak_pages_used = 0;
+    int64_t peak_pages_used = 0, aborted = 0;
 };
 
 class Scheduler {

@@ -22,7 +22,7 @@ from ..config import as_config
 from .runner import Runner, StepEntry
 
 _STATS = ("steps", "scheduled_tokens", "prefill_tokens", "decode_tokens", "deferred_decodes", "deferred_prefills",
-          "preemptions", "failures", "finished", "peak_pages_used", "free_pages", "total_pages")
+          "preemptions", "failures", "finished", "peak_pages_used", "free_pages", "total_pages", "aborted")
 
 
 @dataclass
@@ -168,7 +168,7 @@ class Engine:
         return self.runner.step(entries)
 
     def stats(self) -> Dict[str, int]:
-        buf = np.zeros(12, dtype=np.int64)
+        buf = np.zeros(len(_STATS), dtype=np.int64)
         native.check(self._lib.mllm_engine_stats(self._h, buf.ctypes.data))
         return dict(zip(_STATS, (int(v) for v in buf)))
 

@@ -11,12 +11,12 @@ from ..cache.manager import CacheManager, _rt
 
 STATE_NAMES = {
     0: "waiting_prefill", 1: "deferred_prefill", 2: "prefill", 3: "decode_ready",
-    4: "deferred_decode", 5: "finished", 6: "failed", -1: "unknown",
+    4: "deferred_decode", 5: "finished", 6: "failed", 7: "aborted", -1: "unknown",
 }
 EVENT_NAMES = {1: "preempted", 2: "failed", 3: "deferred"}
 QUEUES = {"waiting_prefill": 0, "deferred_prefill": 1, "prefill": 2, "decode": 3, "deferred_decode": 4}
 COUNTER_NAMES = ("steps", "scheduled_tokens", "prefill_tokens", "decode_tokens", "deferred_decodes",
-                 "deferred_prefills", "preemptions", "failures", "finished", "peak_pages_used")
+                 "deferred_prefills", "preemptions", "failures", "finished", "peak_pages_used", "aborted")
 
 
 @dataclass(frozen=True)
@@ -108,6 +108,6 @@ class Scheduler:
         return self._lib.mllm_sched_queue_length(self._h, QUEUES[name])
 
     def counters(self) -> Dict[str, int]:
-        buf = np.zeros(10, dtype=np.int64)
+        buf = np.zeros(len(COUNTER_NAMES), dtype=np.int64)
         self._lib.mllm_sched_counters(self._h, buf.ctypes.data)
         return dict(zip(COUNTER_NAMES, (int(v) for v in buf)))

@@ -260,6 +260,7 @@ def test_outputs_arrive_in_order_and_a_request_is_aborted_in_flight(tiny_model_d
     assert [t for t, _ in seen[a]] == whole[0][:6]
     assert 0 < len(seen[b]) < 9 and [t for t, _ in seen[b]] == whole[1][:len(seen[b])] and not any(f for _, f in seen[b])
     assert e.stats()["free_pages"] == 60 and e.runner.check() == ""
+    assert e.stats()["aborted"] == 1 and e.stats()["failures"] == 0 and e.stats()["finished"] == 1
     with pytest.raises(KeyError):
         e.abort(b)
     # nothing of a finished or aborted request stays behind: its id can be used again

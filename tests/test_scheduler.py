@@ -231,6 +231,7 @@ def test_eos_and_abort_free_everything():
             s.on_token(e.request_id, e.request_id == 1)
     assert s.state(1) == "finished" and s.state(3) == "prefill"
     s.abort(3)
-    assert s.state(3) == "failed"
+    assert s.state(3) == "aborted" and s.counters()["aborted"] == 1 and s.counters()["failures"] == 0
+    assert s.pop_events() == []                   # (no event: the caller who aborts knows)
     produced, _ = drive(s, eos_after={2: 3})
     assert s.generated(2) == 4 and cm.free_pages() == 64 and cm.n_requests() == 0 and not s.has_work()
