@@ -192,6 +192,38 @@ def test_random_workloads_match_plain_and_give_every_page_back(tiny_model_dirs):
     assert preempted >= 3 and deferred >= 5
 
 
+@pytest.mark.parametrize("overlap", [True, False])
+def test_generation_stops_at_the_last_position(tiny_model_dirs, overlap):
+    """Prompts that end 0, 1, 3 and 10 tokens before the model's last position ask for 10 tokens and get what fits
+    (the token after the last position is still chosen: 1, 2, 4 and 10), the plain model's; a prompt longer than
+    the positions is refused when it is added."""
+    from mini_llm_amd import Engine, EngineOptions, SamplingParams
+    cfg, w = plain_gpt2.read_model(tiny_model_dirs["a"])
+    P = TINY_A["n_positions"]
+    e = Engine.from_pretrained(tiny_model_dirs["a"], dtype="float32",
+                               options=EngineOptions(kv_block_size=4, total_kv_blocks=200, max_batch_num=8, overlap_decode=overlap))
+    g = torch.Generator().manual_seed(1)
+    reqs = {}
+    for length in (P, P - 1, P - 3, P - 10):
+        prompt = torch.randint(0, TINY_A["vocab_size"] - 1, (length,), generator=g).tolist()
+        reqs[e.add_request(prompt, SamplingParams(max_new_tokens=10, ignore_eos=True))] = (prompt, [])
+    with pytest.raises(ValueError, match="prompt of %d tokens" % (P + 1)):
+        e.add_request([1] * (P + 1), SamplingParams(max_new_tokens=2))
+    last = {}
+    while e.has_unfinished():
+        for o in e.step():
+            assert o.token >= 0 and o.request_id not in last
+            reqs[o.request_id][1].append(o.token)
+            if o.finished:
+                last[o.request_id] = True
+    for rid, (prompt, toks) in reqs.items():
+        want = min(10, P - len(prompt) + 1)
+        assert len(toks) == want and last.get(rid), (len(prompt), toks)
+        _near_ties_only(cfg, w, prompt, toks, SLACK["float32"])
+    st = e.stats()
+    assert st["free_pages"] == st["total_pages"] and st["failures"] == 0 and st["finished"] == 4
+
+
 def test_end_of_sequence_token_ends_a_request(tiny_model_dirs, tmp_path):
     """Without --ignore-eos a request ends with the model's end-of-sequence token (read one step late while the
     next step is already in flight); --no-overlap waits for every step and must give the same lines; so must the
