@@ -251,13 +251,17 @@ int cmd_replay(int argc, char** argv) {
     const int n_pages = static_cast<int>((a.integer("max-tokens", 0) + page - 1) / page);
     ModelRunner runner(*model, page, n_pages, static_cast<int>(a.integer("max-requests", 16)));
     const std::string out_dir = a.get("out");
-    ::mkdir(out_dir.c_str(), 0755);
+    for (size_t at = 1; at <= out_dir.size(); ++at)      // the folder and the folders above it
+        if (at == out_dir.size() || out_dir[at] == '/') ::mkdir(out_dir.substr(0, at).c_str(), 0755);
     std::map<std::string, int64_t> ids;          // the trace's request ids (any JSON scalar) -> integers
     int64_t next_id = 0;
+    // a scalar as it is written in file names and messages: a string without its quotes
+    auto plain = [](const Json& v) { return v.is_string() ? v.string() : v.dump(); };
     for (std::string line; std::getline(std::cin, line);) {
         if (line.find_first_not_of(" \t\r") == std::string::npos) continue;
         const Json rec = Json::parse(line);
-        const std::string step = rec.at("step").dump();
+        const std::string step = plain(rec.at("step"));
+        if (step.empty() || step.find('/') != std::string::npos) throw EngineError("a step's name must be a number or a plain word");
         std::vector<StepEntry> entries;
         if (const Json* es = rec.find("entries")) {
             for (const Json& e : es->array()) {
@@ -273,7 +277,17 @@ int cmd_replay(int argc, char** argv) {
         }
         if (!entries.empty()) {
             int rows = 0;
-            const float* logits = runner.step(entries, true, &rows);
+            const float* logits = nullptr;
+            try {
+                logits = runner.step(entries, true, &rows);
+            } catch (const std::exception& e) {
+                // the runner numbers requests; say which of the trace's ids those numbers are
+                std::string msg = std::string("step ") + step + ": " + e.what() + " (";
+                for (const auto& kv : ids)
+                    for (const StepEntry& se : entries)
+                        if (se.request_id == kv.second) msg += "request " + std::to_string(kv.second) + " is " + kv.first + "; ";
+                throw EngineError(msg + "requests are numbered as they first appear)");
+            }
             if (rows > 0) {
                 std::ofstream f(out_dir + "/" + step + ".f32", std::ios::binary);
                 f.write(reinterpret_cast<const char*>(logits),

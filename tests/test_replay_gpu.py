@@ -92,6 +92,34 @@ def test_trace_run_program_at_real_layer_sizes(real_model_dirs, tmp_path, name, 
     rc.check_against_plain(real_model_dirs[name], name, reqs, steps, out, dtype, skip=skip, label="program " + family)
 
 
+def test_trace_run_program_names_and_refusals(tiny_model_dirs, tmp_path):
+    """Steps may be named by words, request ids may be numbers or strings, the output folder is made with the
+    folders above it; a step that cannot run ends the program with a message that names the step and says which
+    of the trace's ids the request is, and with a status other than 0."""
+    import json
+    import os
+    import subprocess
+    import sys
+    name, dtype = "a", "float32"
+    reqs = rc.requests_for(name, seed=6, lengths=[9, 5])
+    a, b = reqs["r0"], reqs["r1"]
+    steps = [{"step": "first", "entries": [{"id": "a", "tokens": a[:7], "want": [6]}, {"id": 7, "tokens": b, "want": [0, 4]}], "end": [7]},
+             {"step": 1, "entries": [{"id": "a", "tokens": a[7:], "want": [0, 1]}], "end": ["a"]}]
+    out_dir = str(tmp_path / "deep" / "er" / "out")
+    out = ru.run_trace_run(tiny_model_dirs[name], dtype, steps, out_dir, 128)
+    assert sorted(os.listdir(out_dir)) == ["1.f32", "first.f32"]
+    cfg, w = plain_gpt2.read_model(tiny_model_dirs[name])
+    ref_a, ref_b = plain_gpt2.forward_logits(cfg, w, a).numpy(), plain_gpt2.forward_logits(cfg, w, b).numpy()
+    tol = rc.TOL[(name, dtype)]["max_abs"]
+    assert np.abs(out["first"] - np.stack([ref_a[6], ref_b[0], ref_b[4]])).max() <= tol
+    assert np.abs(out[1] - np.stack([ref_a[7], ref_a[8]])).max() <= tol
+    bad = {"step": 3, "entries": [{"id": "x", "tokens": [1, 2], "want": [5]}], "end": []}
+    r = subprocess.run([sys.executable, os.path.join(ru.ROOT, "bin", "trace_run"), "--model", tiny_model_dirs[name], "--dtype", dtype,
+                        "--out", out_dir, "--max-tokens", "64"], input=json.dumps(bad) + "\n", capture_output=True, text=True, timeout=300)
+    assert r.returncode != 0 and "done" not in r.stdout
+    assert "step 3" in r.stderr and "wanted index 5 is outside its 2 tokens" in r.stderr and 'is "x"' in r.stderr
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_schedules_agree_with_each_other(tiny_model_dirs, dtype):
     """Cutting, batching and page placement change the logits by rounding only."""
